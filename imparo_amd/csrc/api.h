@@ -1,0 +1,87 @@
+// C entry points of the gfx950 kernel library. Every pointer is device memory
+// unless named host_*. Every entry validates its sizes, launches on `stream`
+// and returns IMPARO_OK, IMPARO_BAD_ARGUMENT (nothing launched) or
+// IMPARO_LAUNCH_FAILED. dtype codes: 0 = float32, 1 = bfloat16.
+#pragma once
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* imparo_stream;
+
+// x[t, :] = table[ids[t], :] as float32.
+int imparo_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* x,
+                        int n_tokens, int width, int vocab, imparo_stream stream);
+
+// Row-wise RMS norm. For output row i the source row is rows ? rows[i] : i.
+// If delta is given the row is x + delta first; with write_back (rows must be
+// null) the sum is stored to x. out[i, :] = v * rsqrt(mean(v^2) + eps) * weight.
+int imparo_rms_norm(float* x, const float* delta, const int32_t* rows, const float* weight,
+                    void* out, int out_dtype, int n_rows, int width, float eps, int write_back,
+                    imparo_stream stream);
+
+// out[t, j] = silu(gu[t, j]) * gu[t, hidden + j]; gu is [n, 2*hidden].
+int imparo_silu_mul(const void* gu, int in_dtype, void* out, int out_dtype, int n_tokens, int hidden,
+                    imparo_stream stream);
+
+// y = x (+ bias): adds a float32 bias [n] to every row of a float32 [m, n] in place.
+int imparo_add_bias(float* y, const float* bias, int m, int n, imparo_stream stream);
+
+// Y[m, n] = X[m, k] . W[n, k]^T, float32 accumulate. X and W share `dtype`.
+int imparo_gemm(const void* x, const void* w, void* y, int dtype, int out_dtype,
+                int m, int n, int k, imparo_stream stream);
+
+// Per (token, head): RMS norm over the head (weight null: none), NeoX rotation
+// with angles pos * inv_freq[i] over the first 2*n_freq dims (n_freq 0: none).
+// qkv is float32 [n_tokens, (heads + 2*kv_heads) * head_dim]; q goes to q_out
+// [n_tokens, heads, head_dim], k and v into the paged cache at each token's
+// position: page = table[row_of_token[t] * table_stride + pos / page_size].
+// Cache layout [n_pages, kv_heads, page_size, head_dim]. write_kv 0 skips the cache.
+int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight, const float* k_weight, float eps,
+                              const float* inv_freq, int n_freq,
+                              const int32_t* positions, const int32_t* row_of_token,
+                              const int32_t* block_table, int table_stride, int page_size,
+                              void* q_out, void* k_cache, void* v_cache, int dtype, int write_kv,
+                              int n_tokens, int heads, int kv_heads, int head_dim, int n_pages,
+                              imparo_stream stream);
+
+// Causal grouped-query attention over the paged cache; one query per (token,
+// head); keys lo..pos with lo = max(0, pos + 1 - window) (window 0: all keys).
+int imparo_attention(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
+                     const int32_t* positions, const int32_t* row_of_token,
+                     const int32_t* block_table, int table_stride, int page_size,
+                     int n_tokens, int heads, int kv_heads, int head_dim, int n_pages,
+                     float scale, int window, imparo_stream stream);
+
+// Gated short convolution over each request's segment, continuing from its
+// state slot. bcx float32 [n_tokens, 3*width] = [B | C | x]. state float32
+// [n_slots, taps-1, width], oldest first. seg_start[r], seg_len[r], slot[r]
+// describe request r's tokens in the batch. out[t] = C_t * (sum_k w[ch,k] *
+// seq[t+k] + bias[ch]).
+int imparo_short_conv(const float* bcx, const float* weight, const float* bias, const float* state,
+                      const int32_t* row_of_token, const int32_t* seg_start, const int32_t* slot,
+                      void* out, int out_dtype, int n_tokens, int width, int taps, int n_slots, int n_rows,
+                      imparo_stream stream);
+
+// state' = the last taps-1 rows of (state ++ B*x) for every request; runs after
+// imparo_short_conv on the same stream.
+int imparo_short_conv_state(const float* bcx, float* state, const int32_t* seg_start, const int32_t* seg_len,
+                            const int32_t* slot, int n_rows, int n_tokens, int width, int taps, int n_slots,
+                            imparo_stream stream);
+
+// out[r] = smallest index of the maximum of logits[r, :]; NaN never wins.
+int imparo_argmax_rows(const float* logits, int32_t* out, int n_rows, int vocab, imparo_stream stream);
+
+// out[r] = the first index whose cumulative softmax(logits[r]/temperature[r])
+// reaches uniform[r]; temperature <= 0 is argmax.
+int imparo_sample_rows(const float* logits, const float* temperature, const float* uniform, int32_t* out,
+                       int n_rows, int vocab, imparo_stream stream);
+
+// Fills n float32 values (or n int32 values of the same bits) without a memset node.
+int imparo_fill_f32(float* p, float value, int64_t n, imparo_stream stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,77 @@
+// Shared device helpers for the gfx950 kernels: storage types, bf16
+// conversion, wave64 reductions, and the error codes the C entry points return.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define IMPARO_OK 0
+#define IMPARO_BAD_ARGUMENT 1
+#define IMPARO_LAUNCH_FAILED 2
+
+// dtype codes shared with the Python side
+#define IMPARO_F32 0
+#define IMPARO_BF16 1
+
+#define WAVE 64
+
+typedef uint16_t bf16_t;   // raw bfloat16 bits
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+    return __uint_as_float(((uint32_t)v) << 16);
+}
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (bf16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ float load_f32(const T* p, size_t i);
+template <> __device__ __forceinline__ float load_f32<float>(const float* p, size_t i) { return p[i]; }
+template <> __device__ __forceinline__ float load_f32<bf16_t>(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }
+
+template <typename T> __device__ __forceinline__ void store_f32(T* p, size_t i, float v);
+template <> __device__ __forceinline__ void store_f32<float>(float* p, size_t i, float v) { p[i] = v; }
+template <> __device__ __forceinline__ void store_f32<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f32_to_bf16(v); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, WAVE));
+    return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.
+// `scratch` holds at least 16 floats of LDS. The order of the additions
+// depends only on the block size, never on the data.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x / WAVE;
+    const int n_waves = (blockDim.x + WAVE - 1) / WAVE;
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+    for (int i = 0; i < n_waves; ++i) total += scratch[i];
+    return total;
+}
+
+// Orders LDS traffic between the lanes of one wave: what any lane wrote before
+// is visible to every lane after.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+static inline int launch_status() {
+    return hipGetLastError() == hipSuccess ? IMPARO_OK : IMPARO_LAUNCH_FAILED;
+}

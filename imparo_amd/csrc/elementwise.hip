@@ -1,0 +1,247 @@
+// Row-wise and element-wise kernels: embedding gather, RMS norm (with the
+// residual add fused in), SiLU gating, bias, fill, and the gated short
+// convolution with its per-request state.
+#include "common.h"
+#include "api.h"
+
+// ---------------------------------------------------------------- embedding
+template <typename T>
+__global__ void k_embed_gather(const T* __restrict__ table, const int32_t* __restrict__ ids,
+                               float* __restrict__ x, int width) {
+    const int t = blockIdx.x;
+    const size_t src = (size_t)ids[t] * width;
+    const size_t dst = (size_t)t * width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) x[dst + i] = load_f32<T>(table, src + i);
+}
+
+extern "C" int imparo_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* x,
+                                   int n_tokens, int width, int vocab, imparo_stream stream) {
+    if (!table || !ids || !x || n_tokens < 0 || width <= 0 || vocab <= 0) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens == 0) return IMPARO_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const int threads = width >= 1024 ? 256 : 64;
+    if (table_dtype == IMPARO_F32)
+        k_embed_gather<float><<<n_tokens, threads, 0, s>>>((const float*)table, ids, x, width);
+    else if (table_dtype == IMPARO_BF16)
+        k_embed_gather<bf16_t><<<n_tokens, threads, 0, s>>>((const bf16_t*)table, ids, x, width);
+    else
+        return IMPARO_BAD_ARGUMENT;
+    return launch_status();
+}
+
+// ---------------------------------------------------------------- RMS norm
+// One block per output row. Sum of squares in float32, reduced in an order
+// fixed by the block size. Two passes over the row; the second re-reads what
+// the first left in registers when the row fits (width <= 8 * blockDim).
+template <typename TOut, int PER_THREAD>
+__global__ void k_rms_norm(float* __restrict__ x, const float* __restrict__ delta,
+                           const int32_t* __restrict__ rows, const float* __restrict__ weight,
+                           TOut* __restrict__ out, int width, float eps, int write_back) {
+    __shared__ float scratch[16];
+    const int i_out = blockIdx.x;
+    const size_t src = (size_t)(rows ? rows[i_out] : i_out) * width;
+    const size_t dst = (size_t)i_out * width;
+    float v[PER_THREAD];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        float a = 0.f;
+        if (i < width) {
+            a = x[src + i];
+            if (delta) a += delta[src + i];
+            if (write_back) x[src + i] = a;
+        }
+        v[j] = a;
+        ss += a * a;
+    }
+    // rows wider than PER_THREAD * blockDim: the tail is not kept in registers
+    for (int i = threadIdx.x + PER_THREAD * blockDim.x; i < width; i += blockDim.x) {
+        float a = x[src + i];
+        if (delta) a += delta[src + i];
+        if (write_back) x[src + i] = a;
+        ss += a * a;
+    }
+    const float total = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(total / (float)width + eps);
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        if (i < width) store_f32<TOut>(out, dst + i, v[j] * scale * weight[i]);
+    }
+    for (int i = threadIdx.x + PER_THREAD * blockDim.x; i < width; i += blockDim.x) {
+        float a = x[src + i];
+        if (delta && !write_back) a += delta[src + i];
+        store_f32<TOut>(out, dst + i, a * scale * weight[i]);
+    }
+}
+
+extern "C" int imparo_rms_norm(float* x, const float* delta, const int32_t* rows, const float* weight,
+                               void* out, int out_dtype, int n_rows, int width, float eps, int write_back,
+                               imparo_stream stream) {
+    if (!x || !weight || !out || n_rows < 0 || width <= 0) return IMPARO_BAD_ARGUMENT;
+    if (write_back && rows) return IMPARO_BAD_ARGUMENT;
+    if (n_rows == 0) return IMPARO_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const int threads = width <= 256 ? 64 : 256;
+    if (out_dtype == IMPARO_F32)
+        k_rms_norm<float, 8><<<n_rows, threads, 0, s>>>(x, delta, rows, weight, (float*)out, width, eps, write_back);
+    else if (out_dtype == IMPARO_BF16)
+        k_rms_norm<bf16_t, 8><<<n_rows, threads, 0, s>>>(x, delta, rows, weight, (bf16_t*)out, width, eps, write_back);
+    else
+        return IMPARO_BAD_ARGUMENT;
+    return launch_status();
+}
+
+// ---------------------------------------------------------------- SiLU gate
+template <typename TIn, typename TOut>
+__global__ void k_silu_mul(const TIn* __restrict__ gu, TOut* __restrict__ out, int64_t total, int hidden) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int64_t t = i / hidden;
+    const int j = (int)(i - t * hidden);
+    const float g = load_f32<TIn>(gu, (size_t)t * 2 * hidden + j);
+    const float u = load_f32<TIn>(gu, (size_t)t * 2 * hidden + hidden + j);
+    store_f32<TOut>(out, (size_t)i, g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int imparo_silu_mul(const void* gu, int in_dtype, void* out, int out_dtype, int n_tokens, int hidden,
+                               imparo_stream stream) {
+    if (!gu || !out || n_tokens < 0 || hidden <= 0) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens == 0) return IMPARO_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t total = (int64_t)n_tokens * hidden;
+    const int threads = 256;
+    const unsigned blocks = (unsigned)((total + threads - 1) / threads);
+    if (in_dtype == IMPARO_F32 && out_dtype == IMPARO_F32)
+        k_silu_mul<float, float><<<blocks, threads, 0, s>>>((const float*)gu, (float*)out, total, hidden);
+    else if (in_dtype == IMPARO_F32 && out_dtype == IMPARO_BF16)
+        k_silu_mul<float, bf16_t><<<blocks, threads, 0, s>>>((const float*)gu, (bf16_t*)out, total, hidden);
+    else if (in_dtype == IMPARO_BF16 && out_dtype == IMPARO_BF16)
+        k_silu_mul<bf16_t, bf16_t><<<blocks, threads, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, total, hidden);
+    else
+        return IMPARO_BAD_ARGUMENT;
+    return launch_status();
+}
+
+// ---------------------------------------------------------------- bias, fill
+__global__ void k_add_bias(float* __restrict__ y, const float* __restrict__ bias, int64_t total, int n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total) y[i] += bias[i % n];
+}
+
+extern "C" int imparo_add_bias(float* y, const float* bias, int m, int n, imparo_stream stream) {
+    if (!y || !bias || m < 0 || n <= 0) return IMPARO_BAD_ARGUMENT;
+    if (m == 0) return IMPARO_OK;
+    const int64_t total = (int64_t)m * n;
+    k_add_bias<<<(unsigned)((total + 255) / 256), 256, 0, (hipStream_t)stream>>>(y, bias, total, n);
+    return launch_status();
+}
+
+__global__ void k_fill_f32(float* __restrict__ p, float value, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = value;
+}
+
+extern "C" int imparo_fill_f32(float* p, float value, int64_t n, imparo_stream stream) {
+    if (!p || n < 0) return IMPARO_BAD_ARGUMENT;
+    if (n == 0) return IMPARO_OK;
+    k_fill_f32<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(p, value, n);
+    return launch_status();
+}
+
+// ---------------------------------------------------------------- short conv
+// One thread per (token, channel). seq index e = (t - seg_start) + k runs over
+// state (e < taps-1) then this segment's B*x values; tap 0 multiplies the
+// oldest value. The state is only read here; the state kernel runs after.
+template <typename TOut>
+__global__ void k_short_conv(const float* __restrict__ bcx, const float* __restrict__ weight,
+                             const float* __restrict__ bias, const float* __restrict__ state,
+                             const int32_t* __restrict__ row_of_token, const int32_t* __restrict__ seg_start,
+                             const int32_t* __restrict__ slot, TOut* __restrict__ out,
+                             int n_tokens, int width, int taps) {
+    const int ch = blockIdx.x * blockDim.x + threadIdx.x;
+    const int t = blockIdx.y;
+    if (ch >= width) return;
+    const int r = row_of_token[t];
+    const int local = t - seg_start[r];
+    const int history = taps - 1;
+    const float* st = state + (size_t)slot[r] * history * width;
+    float acc = 0.f;
+    for (int k = 0; k < taps; ++k) {
+        const int e = local + k;            // index into state ++ values
+        float v;
+        if (e < history) {
+            v = st[(size_t)e * width + ch];
+        } else {
+            const size_t row = (size_t)(t - (history - k)) * 3 * width;
+            v = bcx[row + ch] * bcx[row + 2 * width + ch];
+        }
+        acc += weight[(size_t)ch * taps + k] * v;
+    }
+    if (bias) acc += bias[ch];
+    const float c = bcx[(size_t)t * 3 * width + width + ch];
+    store_f32<TOut>(out, (size_t)t * width + ch, c * acc);
+}
+
+extern "C" int imparo_short_conv(const float* bcx, const float* weight, const float* bias, const float* state,
+                                 const int32_t* row_of_token, const int32_t* seg_start, const int32_t* slot,
+                                 void* out, int out_dtype, int n_tokens, int width, int taps, int n_slots,
+                                 int n_rows, imparo_stream stream) {
+    if (!bcx || !weight || !state || !row_of_token || !seg_start || !slot || !out) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens < 0 || width <= 0 || taps < 2 || taps > 64 || n_slots <= 0 || n_rows < 0) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens == 0) return IMPARO_OK;
+    if (n_tokens > 65535) return IMPARO_BAD_ARGUMENT;
+    hipStream_t s = (hipStream_t)stream;
+    const int threads = width >= 256 ? 256 : 64;
+    dim3 grid((width + threads - 1) / threads, n_tokens);
+    if (out_dtype == IMPARO_F32)
+        k_short_conv<float><<<grid, threads, 0, s>>>(bcx, weight, bias, state, row_of_token, seg_start, slot,
+                                                      (float*)out, n_tokens, width, taps);
+    else if (out_dtype == IMPARO_BF16)
+        k_short_conv<bf16_t><<<grid, threads, 0, s>>>(bcx, weight, bias, state, row_of_token, seg_start, slot,
+                                                       (bf16_t*)out, n_tokens, width, taps);
+    else
+        return IMPARO_BAD_ARGUMENT;
+    return launch_status();
+}
+
+// One thread per (request, channel) owns that channel's whole shift, so the
+// update is race-free in place: it reads every value it needs before it
+// writes. Works for segments shorter than the history.
+#define IMPARO_MAX_TAPS 64
+__global__ void k_short_conv_state(const float* __restrict__ bcx, float* __restrict__ state,
+                                   const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len,
+                                   const int32_t* __restrict__ slot, int width, int taps) {
+    const int ch = blockIdx.x * blockDim.x + threadIdx.x;
+    const int r = blockIdx.y;
+    if (ch >= width) return;
+    const int history = taps - 1;
+    const int n = seg_len[r];
+    const int t0 = seg_start[r];
+    float* st = state + (size_t)slot[r] * history * width;
+    float next[IMPARO_MAX_TAPS - 1];
+    for (int s = 0; s < history; ++s) {
+        const int e = n + s;                // index into state ++ values
+        if (e < history) {
+            next[s] = st[(size_t)e * width + ch];
+        } else {
+            const size_t row = (size_t)(t0 + e - history) * 3 * width;
+            next[s] = bcx[row + ch] * bcx[row + 2 * width + ch];
+        }
+    }
+    for (int s = 0; s < history; ++s) st[(size_t)s * width + ch] = next[s];
+}
+
+extern "C" int imparo_short_conv_state(const float* bcx, float* state, const int32_t* seg_start,
+                                       const int32_t* seg_len, const int32_t* slot, int n_rows, int n_tokens,
+                                       int width, int taps, int n_slots, imparo_stream stream) {
+    if (!bcx || !state || !seg_start || !seg_len || !slot) return IMPARO_BAD_ARGUMENT;
+    if (n_rows < 0 || width <= 0 || taps < 2 || taps > IMPARO_MAX_TAPS || n_slots <= 0) return IMPARO_BAD_ARGUMENT;
+    if (n_rows == 0) return IMPARO_OK;
+    if (n_rows > 65535) return IMPARO_BAD_ARGUMENT;
+    const int threads = width >= 256 ? 256 : 64;
+    dim3 grid((width + threads - 1) / threads, n_rows);
+    k_short_conv_state<<<grid, threads, 0, (hipStream_t)stream>>>(bcx, state, seg_start, seg_len, slot, width, taps);
+    return launch_status();
+}

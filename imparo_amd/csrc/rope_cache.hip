@@ -1,0 +1,109 @@
+// Per-head RMS norm + NeoX rotation of q and k, and the write of k and v into
+// the paged cache, in one launch over every (token, head) of the fused qkv row.
+#include "common.h"
+#include "api.h"
+
+#define ROPE_MAX_HEAD_DIM 512
+#define ROPE_WAVES 4
+
+// One wave per (token, unit), unit in [0, heads + 2*kv_heads): q heads, then k
+// heads, then v heads. The row is staged in LDS as float32; the sum of squares
+// is a wave reduction; angles are pos * inv_freq[i] with the product taken in
+// float64 and rounded to float32, sin/cos in float32.
+template <typename T>
+__global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float* __restrict__ q_weight,
+                                     const float* __restrict__ k_weight, float eps,
+                                     const float* __restrict__ inv_freq, int n_freq,
+                                     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_of_token,
+                                     const int32_t* __restrict__ block_table, int table_stride, int page_size,
+                                     T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                     int write_kv, int n_tokens, int heads, int kv_heads, int head_dim, int n_pages) {
+    __shared__ float rows[ROPE_WAVES][ROPE_MAX_HEAD_DIM];
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x / WAVE;
+    const int units = heads + 2 * kv_heads;
+    const long long id = (long long)blockIdx.x * ROPE_WAVES + wave;
+    if (id >= (long long)n_tokens * units) return;
+    const int t = (int)(id / units);
+    const int u = (int)(id - (long long)t * units);
+    const float* src = qkv + (size_t)t * units * head_dim + (size_t)u * head_dim;
+    float* row = rows[wave];
+    const bool is_q = u < heads;
+    const bool is_v = u >= heads + kv_heads;
+    const float* weight = is_q ? q_weight : k_weight;
+
+    float ss = 0.f;
+    for (int i = lane; i < head_dim; i += WAVE) {
+        const float a = src[i];
+        row[i] = a;
+        ss += a * a;
+    }
+    if (!is_v) {
+        if (weight) {
+            ss = wave_sum(ss);
+            const float scale = 1.0f / sqrtf(ss / (float)head_dim + eps);
+            for (int i = lane; i < head_dim; i += WAVE) row[i] = row[i] * scale * weight[i];
+        }
+        wave_lds_sync();   // a pair's second element may have been written by another lane
+        if (n_freq > 0) {
+            const int pos = positions[t];
+            // each lane owns pair (i, i + n_freq): reads both, then writes both
+            for (int i = lane; i < n_freq; i += WAVE) {
+                const float theta = (float)((double)pos * (double)inv_freq[i]);
+                float sn, cs;
+                sincosf(theta, &sn, &cs);
+                const float x0 = row[i], x1 = row[i + n_freq];
+                row[i] = x0 * cs - x1 * sn;
+                row[i + n_freq] = x0 * sn + x1 * cs;
+            }
+        }
+    }
+    wave_lds_sync();
+
+    if (is_q) {
+        T* dst = q_out + ((size_t)t * heads + u) * head_dim;
+        for (int i = lane; i < head_dim; i += WAVE) store_f32<T>(dst, i, row[i]);
+        return;
+    }
+    if (!write_kv) return;
+    const int kvh = is_v ? u - heads - kv_heads : u - heads;
+    const int pos = positions[t];
+    const int page = block_table[(size_t)row_of_token[t] * table_stride + pos / page_size];
+    if (page < 0 || page >= n_pages) return;   // never write outside the pool
+    T* cache = is_v ? v_cache : k_cache;
+    T* dst = cache + (((size_t)page * kv_heads + kvh) * page_size + (pos % page_size)) * head_dim;
+    for (int i = lane; i < head_dim; i += WAVE) store_f32<T>(dst, i, row[i]);
+}
+
+extern "C" int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight, const float* k_weight, float eps,
+                                         const float* inv_freq, int n_freq,
+                                         const int32_t* positions, const int32_t* row_of_token,
+                                         const int32_t* block_table, int table_stride, int page_size,
+                                         void* q_out, void* k_cache, void* v_cache, int dtype, int write_kv,
+                                         int n_tokens, int heads, int kv_heads, int head_dim, int n_pages,
+                                         imparo_stream stream) {
+    if (!qkv || !positions || !q_out) return IMPARO_BAD_ARGUMENT;
+    if (write_kv && (!row_of_token || !block_table || !k_cache || !v_cache)) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens < 0 || heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim > ROPE_MAX_HEAD_DIM)
+        return IMPARO_BAD_ARGUMENT;
+    if (n_freq < 0 || 2 * n_freq > head_dim || (n_freq > 0 && !inv_freq)) return IMPARO_BAD_ARGUMENT;
+    if (page_size <= 0 || table_stride < 0 || n_pages < 0) return IMPARO_BAD_ARGUMENT;
+    if ((q_weight == nullptr) != (k_weight == nullptr)) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens == 0) return IMPARO_OK;
+    const long long total = (long long)n_tokens * (heads + 2 * kv_heads);
+    const unsigned blocks = (unsigned)((total + ROPE_WAVES - 1) / ROPE_WAVES);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == IMPARO_F32)
+        k_qk_norm_rope_store<float><<<blocks, ROPE_WAVES * WAVE, 0, s>>>(
+            qkv, q_weight, k_weight, eps, inv_freq, n_freq, positions, row_of_token, block_table, table_stride,
+            page_size, (float*)q_out, (float*)k_cache, (float*)v_cache, write_kv, n_tokens, heads, kv_heads,
+            head_dim, n_pages);
+    else if (dtype == IMPARO_BF16)
+        k_qk_norm_rope_store<bf16_t><<<blocks, ROPE_WAVES * WAVE, 0, s>>>(
+            qkv, q_weight, k_weight, eps, inv_freq, n_freq, positions, row_of_token, block_table, table_stride,
+            page_size, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, write_kv, n_tokens, heads, kv_heads,
+            head_dim, n_pages);
+    else
+        return IMPARO_BAD_ARGUMENT;
+    return launch_status();
+}

@@ -1,0 +1,108 @@
+"""Plan + weights -> a runnable stack of parts.
+
+The builder knows roles and registries, not architectures: every layer's
+norms, mixer and feed-forward are looked up by the kind its PartSpec names and
+built from the tensors they declared. The run order is the plan's list of
+calls; each call that owns a cache gets a cache site of its own, a call that
+reads another call's cache is bound to that call's site.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ..cache.pages import StateSpec
+from ..config.plan import LayerPlan, ModelPlan, PartSpec
+from ..parts import part_class
+from ..parts.base import Declared, Residual, StepContext
+from ..weights.loader import TensorDecl
+
+
+def _declare(role: str, spec: PartSpec) -> Declared:
+    return part_class(role, spec.kind).declare(spec)
+
+
+def declared_tensors(plan: ModelPlan) -> Declared:
+    """Every tensor the model reads, by name: what the parts declare, united.
+    A name two parts declare (a tied head) must agree in shape."""
+    out: Declared = {}
+
+    def add(d: Declared) -> None:
+        for name, (decl, init) in d.items():
+            if name in out and out[name][0].shape != decl.shape:
+                raise ValueError(f"tensor {name} is declared with shapes {out[name][0].shape} and {decl.shape}")
+            out[name] = (decl, init)
+
+    add(_declare("embedding", plan.embedding))
+    for layer in plan.layers:
+        add(_declare("norm", layer.mixer_norm))
+        add(_declare("mixer", layer.mixer))
+        add(_declare("norm", layer.ffn_norm))
+        add(_declare("feed_forward", layer.ffn))
+    add(_declare("norm", plan.final_norm))
+    add(_declare("head", plan.head))
+    return out
+
+
+class Model:
+    def __init__(self, plan: ModelPlan, tensors: Dict[str, torch.Tensor], device: torch.device,
+                 dtype: torch.dtype):
+        plan.validate()
+        self.plan = plan
+        self.device = device
+        self.dtype = dtype
+        placed: Dict[str, torch.Tensor] = {}
+        self.embedding = part_class("embedding", plan.embedding.kind)(plan.embedding, tensors, device, dtype, placed)
+        self.blocks = []
+        for layer in plan.layers:
+            mk = lambda role, spec: part_class(role, spec.kind)(spec, tensors, device, dtype)
+            block_cls = part_class("block", layer.arrangement)
+            self.blocks.append(block_cls(mk("norm", layer.mixer_norm), mk("mixer", layer.mixer),
+                                         mk("norm", layer.ffn_norm), mk("feed_forward", layer.ffn)))
+        self.final_norm = part_class("norm", plan.final_norm.kind)(plan.final_norm, tensors, device, dtype)
+        self.head = part_class("head", plan.head.kind)(plan.head, tensors, device, dtype, placed)
+        # cache sites: one per entry of the run order; None where the call borrows
+        self.site_of_call: List[int] = []
+        self.site_specs: List[StateSpec] = []
+        for i, call in enumerate(plan.order):
+            mixer = self.blocks[call.layer].mixer
+            if call.cache_of is None:
+                self.site_of_call.append(i)
+                self.site_specs.append(mixer.cache_spec())
+            else:
+                self.site_of_call.append(call.cache_of)
+                self.site_specs.append(None)
+                owner = self.site_specs[call.cache_of]
+                if owner != mixer.cache_spec():
+                    raise ValueError(f"run order entry {i} reads the cache of entry {call.cache_of}, "
+                                     f"whose state has another shape")
+
+    def forward(self, ctx: StepContext, token_ids: torch.Tensor, want_rows: Optional[torch.Tensor]
+                ) -> Optional[torch.Tensor]:
+        """Runs the batch through every call of the order. Returns float32
+        logits [wanted, vocab] for `want_rows` (indices into the packed
+        batch), or None if nothing is wanted; the head is skipped then."""
+        res = Residual(self.embedding.forward(ctx, token_ids))
+        for i, call in enumerate(self.plan.order):
+            self.blocks[call.layer].forward(ctx, res, self.site_of_call[i], call.cache_of is None)
+        if want_rows is None or want_rows.shape[0] == 0:
+            return None
+        h = self.final_norm.forward_rows(ctx, res, want_rows, self.head.in_dtype)
+        return self.head.forward(ctx, h)
+
+    def weight_bytes(self) -> int:
+        seen, total = set(), 0
+        def walk(obj):
+            nonlocal total
+            for v in vars(obj).values():
+                if isinstance(v, torch.Tensor):
+                    if v.data_ptr() not in seen:
+                        seen.add(v.data_ptr())
+                        total += v.numel() * v.element_size()
+                elif hasattr(v, "__dict__") and not isinstance(v, type):
+                    walk(v)
+        walk(self.embedding); walk(self.final_norm); walk(self.head)
+        for b in self.blocks:
+            walk(b)
+        return total

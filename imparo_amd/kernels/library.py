@@ -1,0 +1,74 @@
+"""Loads the gfx950 kernel library and declares its C entry points.
+
+The library is loaded once per process. If it has not been built yet it is
+built at the first call (hipcc must be present); there is no fallback: without
+the library every op raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from ctypes import c_int, c_int64, c_float, c_void_p
+
+from ..csrc import build as _build
+
+_lock = threading.Lock()
+_lib = None
+
+P = c_void_p
+I = c_int
+F = c_float
+
+_SIGNATURES = {
+    "imparo_embed_gather": [P, I, P, P, I, I, I, P],
+    "imparo_rms_norm": [P, P, P, P, P, I, I, I, F, I, P],
+    "imparo_silu_mul": [P, I, P, I, I, I, P],
+    "imparo_add_bias": [P, P, I, I, P],
+    "imparo_gemm": [P, P, P, I, I, I, I, I, P],
+    "imparo_qk_norm_rope_store": [P, P, P, F, P, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, P],
+    "imparo_attention": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P],
+    "imparo_short_conv": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
+    "imparo_short_conv_state": [P, P, P, P, P, I, I, I, I, I, P],
+    "imparo_argmax_rows": [P, P, I, I, P],
+    "imparo_sample_rows": [P, P, P, P, I, I, P],
+    "imparo_fill_f32": [P, F, c_int64, P],
+}
+
+
+class KernelLibraryError(RuntimeError):
+    pass
+
+
+def library() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        path = _build.library_path()
+        if not os.path.isfile(path):
+            try:
+                path = _build.build(verbose=True)
+            except Exception as e:  # no silent fallback: say why there is no library
+                raise KernelLibraryError(f"the gfx950 kernel library is not built and building it failed: {e}") from e
+        try:
+            lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelLibraryError(f"cannot load {path}: {e}") from e
+        for name, argtypes in _SIGNATURES.items():
+            try:
+                fn = getattr(lib, name)
+            except AttributeError:
+                raise KernelLibraryError(f"{path} lacks the entry point {name}; rebuild it "
+                                         f"(python -m imparo_amd.csrc.build)") from None
+            fn.argtypes = argtypes
+            fn.restype = c_int
+        _lib = lib
+        return _lib
+
+
+def loaded_path() -> str:
+    library()
+    return _build.library_path()

@@ -1,0 +1,221 @@
+"""Python faces of the gfx950 kernels.
+
+Each function checks on the host what its kernel assumes (device, dtype,
+contiguity, shapes, index ranges that the host knows), then launches on the
+current stream. There is no CPU path: a tensor that is not on the GPU is an
+error, and so is a missing kernel library.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .library import library
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelArgumentError(ValueError):
+    pass
+
+
+def _code(t: torch.Tensor, what: str) -> int:
+    if t.dtype not in _CODES:
+        raise KernelArgumentError(f"{what} has dtype {t.dtype}; kernels take float32 or bfloat16")
+    return _CODES[t.dtype]
+
+
+def _dev(t: Optional[torch.Tensor], what: str, dtype=None, shape=None) -> int:
+    """Checks a tensor and returns its device address (0 for None)."""
+    if t is None:
+        return 0
+    if not isinstance(t, torch.Tensor):
+        raise KernelArgumentError(f"{what} is not a tensor")
+    if t.device.type != "cuda":
+        raise KernelArgumentError(f"{what} is on {t.device}; the kernels run on the GPU only")
+    if not t.is_contiguous():
+        raise KernelArgumentError(f"{what} is not contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelArgumentError(f"{what} has dtype {t.dtype}, expected {dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelArgumentError(f"{what} has shape {list(t.shape)}, expected {list(shape)}")
+    return t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(status: int, name: str) -> None:
+    if status == 0:
+        return
+    why = {1: "an argument was refused (size or pointer the kernel cannot take)",
+           2: "the launch failed"}.get(status, f"status {status}")
+    raise KernelArgumentError(f"{name}: {why}")
+
+
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    vocab, width = table.shape
+    n = ids.shape[0]
+    _check(library().imparo_embed_gather(
+        _dev(table, "embedding table"), _code(table, "embedding table"),
+        _dev(ids, "token ids", torch.int32, (n,)), _dev(out, "embedding output", torch.float32, (n, width)),
+        n, width, vocab, _stream()), "embed_gather")
+    return out
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+             delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
+             write_back: bool = False) -> torch.Tensor:
+    """out[i] = norm(x[src] (+ delta[src])) * weight, src = rows[i] or i.
+    write_back stores x + delta into x (only without rows)."""
+    width = x.shape[-1]
+    n_out = out.shape[0]
+    if rows is None and n_out != x.shape[0]:
+        raise KernelArgumentError(f"rms_norm: out has {n_out} rows, x has {x.shape[0]}")
+    if rows is not None and rows.shape[0] != n_out:
+        raise KernelArgumentError("rms_norm: one source row index per output row is needed")
+    if write_back and (rows is not None or delta is None):
+        raise KernelArgumentError("rms_norm: write_back needs a delta and no row selection")
+    _check(library().imparo_rms_norm(
+        _dev(x, "rms_norm x", torch.float32), _dev(delta, "rms_norm delta", torch.float32, x.shape),
+        _dev(rows, "rms_norm rows", torch.int32), _dev(weight, "rms_norm weight", torch.float32, (width,)),
+        _dev(out, "rms_norm out", None, (n_out, width)), _code(out, "rms_norm out"),
+        n_out, width, float(eps), int(write_back), _stream()), "rms_norm")
+    return out
+
+
+def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    n, two_h = gu.shape
+    hidden = two_h // 2
+    if two_h != 2 * hidden:
+        raise KernelArgumentError("silu_mul: the input row must hold gate and up halves")
+    _check(library().imparo_silu_mul(_dev(gu, "silu_mul input"), _code(gu, "silu_mul input"),
+                                     _dev(out, "silu_mul output", None, (n, hidden)), _code(out, "silu_mul output"),
+                                     n, hidden, _stream()), "silu_mul")
+    return out
+
+
+def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    m, n = y.shape
+    _check(library().imparo_add_bias(_dev(y, "add_bias y", torch.float32), _dev(bias, "bias", torch.float32, (n,)),
+                                     m, n, _stream()), "add_bias")
+    return y
+
+
+def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[m, n] = x[m, k] . w[n, k]^T; x and w share a dtype; float32 accumulate."""
+    m, k = x.shape
+    n, kw = w.shape
+    if kw != k:
+        raise KernelArgumentError(f"gemm: x has {k} columns but the weight has {kw}")
+    if x.dtype != w.dtype:
+        raise KernelArgumentError(f"gemm: x is {x.dtype} but the weight is {w.dtype}")
+    if x.dtype == torch.bfloat16 and k % 8 != 0:
+        raise KernelArgumentError(f"gemm: the bfloat16 kernels need the inner size to be a multiple of 8, got {k}")
+    _check(library().imparo_gemm(_dev(x, "gemm x"), _dev(w, "gemm weight"), _dev(out, "gemm out", None, (m, n)),
+                                 _code(x, "gemm x"), _code(out, "gemm out"), m, n, k, _stream()), "gemm")
+    return out
+
+
+def qk_norm_rope_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+                       eps: float, inv_freq: Optional[torch.Tensor], positions: torch.Tensor,
+                       row_of_token: torch.Tensor, block_table: Optional[torch.Tensor], page_size: int,
+                       q_out: torch.Tensor, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                       heads: int, kv_heads: int, head_dim: int) -> torch.Tensor:
+    n = qkv.shape[0]
+    units = heads + 2 * kv_heads
+    write_kv = k_cache is not None
+    n_freq = 0 if inv_freq is None else inv_freq.shape[0]
+    n_pages = 0
+    table_stride = 0
+    if write_kv:
+        n_pages = k_cache.shape[0]
+        want = (n_pages, kv_heads, page_size, head_dim)
+        _dev(k_cache, "k cache", q_out.dtype, want)
+        _dev(v_cache, "v cache", q_out.dtype, want)
+        if block_table is None or block_table.dim() != 2:
+            raise KernelArgumentError("qk_norm_rope_store: a [rows, pages] block table is needed to write the cache")
+        table_stride = block_table.shape[1]
+    _check(library().imparo_qk_norm_rope_store(
+        _dev(qkv, "qkv", torch.float32, (n, units * head_dim)),
+        _dev(q_weight, "q norm weight", torch.float32, (head_dim,)),
+        _dev(k_weight, "k norm weight", torch.float32, (head_dim,)), float(eps),
+        _dev(inv_freq, "inverse frequencies", torch.float32), n_freq,
+        _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
+        _dev(block_table, "block table", torch.int32), table_stride, page_size,
+        _dev(q_out, "q out", None, (n, heads, head_dim)), _dev(k_cache, "k cache"), _dev(v_cache, "v cache"),
+        _code(q_out, "q out"), int(write_kv), n, heads, kv_heads, head_dim, n_pages, _stream()),
+        "qk_norm_rope_store")
+    return q_out
+
+
+def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+              positions: torch.Tensor, row_of_token: torch.Tensor, block_table: torch.Tensor,
+              scale: float, window: Optional[int]) -> torch.Tensor:
+    n, heads, head_dim = q.shape
+    n_pages, kv_heads, page_size, hd = k_cache.shape
+    if hd != head_dim:
+        raise KernelArgumentError(f"attention: q has head size {head_dim}, the cache {hd}")
+    if head_dim % 16 != 0:
+        raise KernelArgumentError(f"attention: head size must be a multiple of 16, got {head_dim}")
+    if heads % kv_heads != 0:
+        raise KernelArgumentError(f"attention: {heads} heads cannot share {kv_heads} kv heads evenly")
+    _check(library().imparo_attention(
+        _dev(q, "q"), _dev(k_cache, "k cache", q.dtype), _dev(v_cache, "v cache", q.dtype, k_cache.shape),
+        _dev(out, "attention out", q.dtype, (n, heads * head_dim)), _code(q, "q"),
+        _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
+        _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size,
+        n, heads, kv_heads, head_dim, n_pages, float(scale), int(window or 0), _stream()), "attention")
+    return out
+
+
+def short_conv(bcx: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
+               row_of_token: torch.Tensor, seg_start: torch.Tensor, seg_len: torch.Tensor, slot: torch.Tensor,
+               out: torch.Tensor) -> torch.Tensor:
+    """Gated short convolution of every request's segment, then the state
+    update; the two launches are ordered by the stream."""
+    n, three_w = bcx.shape
+    width, taps = weight.shape
+    if three_w != 3 * width:
+        raise KernelArgumentError(f"short_conv: rows of {three_w} values do not hold B, C and x of width {width}")
+    n_slots = state.shape[0]
+    n_rows = seg_start.shape[0]
+    lib = library()
+    common = dict()
+    _check(lib.imparo_short_conv(
+        _dev(bcx, "bcx", torch.float32), _dev(weight, "conv weight", torch.float32),
+        _dev(bias, "conv bias", torch.float32, (width,)),
+        _dev(state, "conv state", torch.float32, (n_slots, taps - 1, width)),
+        _dev(row_of_token, "row_of_token", torch.int32, (n,)), _dev(seg_start, "seg_start", torch.int32, (n_rows,)),
+        _dev(slot, "slot", torch.int32, (n_rows,)), _dev(out, "conv out", None, (n, width)), _code(out, "conv out"),
+        n, width, taps, n_slots, n_rows, _stream()), "short_conv")
+    _check(lib.imparo_short_conv_state(
+        bcx.data_ptr(), state.data_ptr(), seg_start.data_ptr(), _dev(seg_len, "seg_len", torch.int32, (n_rows,)),
+        slot.data_ptr(), n_rows, n, width, taps, n_slots, _stream()), "short_conv_state")
+    return out
+
+
+def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    n, vocab = logits.shape
+    _check(library().imparo_argmax_rows(_dev(logits, "logits", torch.float32), _dev(out, "picks", torch.int32, (n,)),
+                                        n, vocab, _stream()), "argmax_rows")
+    return out
+
+
+def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor,
+                out: torch.Tensor) -> torch.Tensor:
+    n, vocab = logits.shape
+    _check(library().imparo_sample_rows(
+        _dev(logits, "logits", torch.float32), _dev(temperature, "temperature", torch.float32, (n,)),
+        _dev(uniform, "uniform", torch.float32, (n,)), _dev(out, "picks", torch.int32, (n,)),
+        n, vocab, _stream()), "sample_rows")
+    return out
+
+
+def fill_f32(t: torch.Tensor, value: float) -> torch.Tensor:
+    _check(library().imparo_fill_f32(_dev(t, "fill target", torch.float32), float(value), t.numel(), _stream()),
+           "fill_f32")
+    return t

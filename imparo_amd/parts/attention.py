@@ -1,0 +1,103 @@
+"""Grouped-query attention over the paged cache.
+
+q = Wq h, k = Wk h, v = Wv h (one fused projection), per-head RMS norm of q
+and k, rotation, k and v appended to the cache at the tokens' positions before
+attention of the same batch, causal softmax attention bounded by position,
+then the output projection
+(/root/reference/crates/imparo-model/src/lfm2/workflow_cpu.rs:203-250,
+/root/reference/crates/imparo-model/src/cpu_support.rs:361-445)."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..cache.pages import PagedSpec
+from ..config.plan import PartSpec
+from ..kernels import ops
+from ..weights.loader import TensorDecl
+from .base import Declared, StepContext
+from .linear import Linear, place_matrix, place_vector
+from .registry import part_class, register_part
+
+_DEFAULT_NAMES = dict(q="q_proj", k="k_proj", v="v_proj", o="o_proj", q_norm="q_norm", k_norm="k_norm")
+
+
+class Attention:
+    role = "mixer"
+
+    @staticmethod
+    def _names(spec: PartSpec) -> Dict[str, str]:
+        names = dict(_DEFAULT_NAMES)
+        names.update(spec.get("names") or {})
+        return {k: f"{spec.prefix}.{v}" for k, v in names.items()}
+
+    @classmethod
+    def declare(cls, spec: PartSpec) -> Declared:
+        n = cls._names(spec)
+        E, H, Hk, D = spec["width"], spec["heads"], spec["kv_heads"], spec["head_dim"]
+        out: Declared = {
+            n["q"] + ".weight": (TensorDecl((H * D, E)), "matrix"),
+            n["k"] + ".weight": (TensorDecl((Hk * D, E)), "matrix"),
+            n["v"] + ".weight": (TensorDecl((Hk * D, E)), "matrix"),
+            n["o"] + ".weight": (TensorDecl((E, H * D)), "matrix"),
+        }
+        if spec.get("qk_norm") is not None:
+            out[n["q_norm"] + ".weight"] = (TensorDecl((D,), "vector"), "norm")
+            out[n["k_norm"] + ".weight"] = (TensorDecl((D,), "vector"), "norm")
+        return out
+
+    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
+                 engine_dtype: torch.dtype):
+        n = self._names(spec)
+        self.width, self.heads, self.kv_heads, self.head_dim = (spec["width"], spec["heads"], spec["kv_heads"],
+                                                                spec["head_dim"])
+        if self.head_dim % 16:
+            raise ValueError(f"attention kernels take head sizes in steps of 16, got {self.head_dim}")
+        if self.heads % self.kv_heads:
+            raise ValueError(f"{self.heads} heads cannot share {self.kv_heads} kv heads evenly")
+        self.scale = float(spec["scale"])
+        self.window: Optional[int] = spec.get("window")
+        ws = [tensors[n[x] + ".weight"] for x in ("q", "k", "v")]
+        if len({w.dtype for w in ws}) > 1:
+            ws = [w.to(torch.float32) for w in ws]
+        # one projection for q | k | v: the same dot products, one launch
+        self.qkv = Linear(place_matrix(torch.cat(ws, dim=0), engine_dtype, device))
+        self.out = Linear(place_matrix(tensors[n["o"] + ".weight"], engine_dtype, device))
+        norm = spec.get("qk_norm")
+        if norm is not None:
+            self.norm_eps = float(norm["eps"])
+            self.q_norm = place_vector(tensors[n["q_norm"] + ".weight"], device)
+            self.k_norm = place_vector(tensors[n["k_norm"] + ".weight"], device)
+        else:
+            self.norm_eps, self.q_norm, self.k_norm = 0.0, None, None
+        pos = spec.get("position") or PartSpec("none")
+        self.position = part_class("position", pos.kind)(pos, device)
+        if self.position.rotary_dim > self.head_dim:
+            raise ValueError("the rotated part of a head cannot be wider than the head")
+
+    @property
+    def in_dtype(self) -> torch.dtype:
+        return self.qkv.in_dtype
+
+    def cache_spec(self) -> PagedSpec:
+        return PagedSpec(self.kv_heads, self.head_dim, self.window)
+
+    def forward(self, ctx: StepContext, site: int, owns_cache: bool, h: torch.Tensor) -> torch.Tensor:
+        T = h.shape[0]
+        qkv = self.qkv(ctx, h, torch.float32, "qkv")
+        k_cache, v_cache, table = ctx.kv(site)
+        q = ctx.workspace.get("q", (T, self.heads, self.head_dim), ctx.dtype)
+        ops.qk_norm_rope_store(qkv, self.q_norm, self.k_norm, self.norm_eps, self.position.inv_freq,
+                               ctx.positions, ctx.row_of_token, table if owns_cache else None, ctx.page_size,
+                               q, k_cache if owns_cache else None, v_cache if owns_cache else None,
+                               self.heads, self.kv_heads, self.head_dim)
+        attn_dtype = ctx.dtype
+        o = ctx.workspace.get("attn_out", (T, self.heads * self.head_dim), attn_dtype)
+        ops.attention(q, k_cache, v_cache, o, ctx.positions, ctx.row_of_token, table, self.scale, self.window)
+        if o.dtype != self.out.in_dtype:
+            raise ValueError("the output projection's weight dtype differs from the attention output's")
+        return self.out(ctx, o, torch.float32, "mixer_out")
+
+
+register_part("mixer", "attention", Attention)

@@ -1,0 +1,28 @@
+"""How a layer's parts are arranged.
+
+pre_norm: x += mixer(norm_a(x)); x += ffn(norm_b(x)) -- no post-norms
+(/root/reference/crates/imparo-model/src/lfm2/workflow_cpu.rs:8-15). Each
+delta is left pending on the residual stream so that the next norm, whichever
+block it belongs to, adds it while reading the row."""
+from __future__ import annotations
+
+import torch
+
+from .base import Residual, StepContext
+from .registry import register_part
+
+
+class PreNormBlock:
+    role = "block"
+
+    def __init__(self, mixer_norm, mixer, ffn_norm, ffn):
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+
+    def forward(self, ctx: StepContext, res: Residual, site: int, owns_cache: bool) -> None:
+        h = self.mixer_norm.forward(ctx, res, self.mixer.in_dtype)
+        res.pending = self.mixer.forward(ctx, site, owns_cache, h)
+        n = self.ffn_norm.forward(ctx, res, self.ffn.in_dtype)
+        res.pending = self.ffn.forward(ctx, n)
+
+
+register_part("block", "pre_norm", PreNormBlock)

@@ -1,0 +1,61 @@
+"""Dense SwiGLU feed-forward: f = W2 ( silu(W1 n) * (W3 n) ), SiLU on the gate
+(/root/reference/crates/imparo-model/src/lfm2/workflow_cpu.rs:298-316)."""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from ..config.plan import PartSpec
+from ..kernels import ops
+from ..weights.loader import TensorDecl
+from .base import Declared, StepContext
+from .linear import Linear, place_matrix
+from .registry import register_part
+
+_DEFAULT_NAMES = dict(gate="gate_proj", up="up_proj", down="down_proj")
+
+
+class SwiGlu:
+    role = "feed_forward"
+
+    @staticmethod
+    def _names(spec: PartSpec) -> Dict[str, str]:
+        names = dict(_DEFAULT_NAMES)
+        names.update(spec.get("names") or {})
+        return {k: f"{spec.prefix}.{v}" for k, v in names.items()}
+
+    @classmethod
+    def declare(cls, spec: PartSpec) -> Declared:
+        n = cls._names(spec)
+        E, F = spec["width"], spec["hidden"]
+        return {
+            n["gate"] + ".weight": (TensorDecl((F, E)), "matrix"),
+            n["up"] + ".weight": (TensorDecl((F, E)), "matrix"),
+            n["down"] + ".weight": (TensorDecl((E, F)), "matrix"),
+        }
+
+    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
+                 engine_dtype: torch.dtype):
+        n = self._names(spec)
+        self.width, self.hidden = spec["width"], spec["hidden"]
+        gate, up = tensors[n["gate"] + ".weight"], tensors[n["up"] + ".weight"]
+        if gate.dtype != up.dtype:
+            gate, up = gate.to(torch.float32), up.to(torch.float32)
+        # gate | up as one projection: the same dot products, one launch
+        self.gate_up = Linear(place_matrix(torch.cat([gate, up], dim=0), engine_dtype, device))
+        self.down = Linear(place_matrix(tensors[n["down"] + ".weight"], engine_dtype, device))
+
+    @property
+    def in_dtype(self) -> torch.dtype:
+        return self.gate_up.in_dtype
+
+    def forward(self, ctx: StepContext, n: torch.Tensor) -> torch.Tensor:
+        T = n.shape[0]
+        gu = self.gate_up(ctx, n, torch.float32, "gate_up")
+        g = ctx.workspace.get("gated", (T, self.hidden), self.down.in_dtype)
+        ops.silu_mul(gu, g)
+        return self.down(ctx, g, torch.float32, "ffn_out")
+
+
+register_part("feed_forward", "swiglu", SwiGlu)

@@ -1,0 +1,52 @@
+"""A dense projection y = x . W^T (+ b) on the GEMM kernels.
+
+Not a part of its own: mixers, feed-forwards and the head are made of these.
+The weight decides the kernel: a bfloat16 weight runs the MFMA kernels, a
+float32 weight the float32 kernel; the input must already be in that dtype
+(`in_dtype`), which the producer of the input asks for.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+from .base import StepContext
+
+
+class Linear:
+    def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor] = None):
+        if weight.dim() != 2:
+            raise ValueError(f"a projection weight is [out, in], got shape {list(weight.shape)}")
+        self.weight = weight.contiguous()
+        self.bias = None if bias is None else bias.to(torch.float32).contiguous()
+        self.out_features, self.in_features = weight.shape
+
+    @property
+    def in_dtype(self) -> torch.dtype:
+        return self.weight.dtype
+
+    def __call__(self, ctx: StepContext, x: torch.Tensor, out_dtype: torch.dtype, name: str) -> torch.Tensor:
+        if self.bias is not None and out_dtype != torch.float32:
+            raise ValueError("a projection with a bias writes float32")
+        out = ctx.workspace.get(name, (x.shape[0], self.out_features), out_dtype)
+        ops.gemm(x, self.weight, out)
+        if self.bias is not None:
+            ops.add_bias(out, self.bias)
+        return out
+
+
+def place_matrix(t: torch.Tensor, engine_dtype: torch.dtype, device: torch.device) -> torch.Tensor:
+    """A matrix as the engine keeps it on the device: bfloat16 stays bfloat16
+    under a bfloat16 engine, everything is float32 under a float32 engine, and
+    a tensor stored in float32 stays float32 either way."""
+    if engine_dtype == torch.float32 or t.dtype == torch.float32:
+        return t.to(device=device, dtype=torch.float32).contiguous()
+    return t.to(device=device, dtype=torch.bfloat16).contiguous()
+
+
+def place_vector(t: torch.Tensor, device: torch.device) -> torch.Tensor:
+    """Norm weights, conv taps and biases are read as float32 by the kernels;
+    widening bfloat16 to float32 is exact."""
+    return t.to(device=device, dtype=torch.float32).contiguous()
