@@ -28,6 +28,8 @@ class PagePool:
         if n_pages < 0:
             raise ValueError("a pool cannot have a negative number of pages")
         self.n_pages = n_pages
+        self._place: Optional[List[int]] = None   # rank -> page, when placement is scrambled
+        self._rank: Optional[List[int]] = None
         self._heap = list(range(n_pages))
         self._free = [True] * n_pages
         self.n_free = n_pages
@@ -37,6 +39,8 @@ class PagePool:
         if self.n_free == 0:
             raise OutOfPages("no free page")
         page = heapq.heappop(self._heap)
+        if self._place is not None:
+            page = self._place[page]
         self._free[page] = False
         self.n_free -= 1
         self.high_water = max(self.high_water, page + 1)
@@ -49,7 +53,22 @@ class PagePool:
             raise CacheError(f"page {page} freed twice")
         self._free[page] = True
         self.n_free += 1
-        heapq.heappush(self._heap, page)
+        heapq.heappush(self._heap, page if self._rank is None else self._rank[page])
+
+    def scramble(self, seed: int) -> None:
+        """Permutes which physical page each allocation rank maps to, so that
+        block tables are not the identity. Only on an untouched pool. Output
+        must not depend on it: placement is invisible
+        (/root/reference/crates/imparo-kv/src/resident.rs:56-99)."""
+        if self.n_free != self.n_pages:
+            raise CacheError("placement can only be scrambled while every page is free")
+        import random
+        place = list(range(self.n_pages))
+        random.Random(seed).shuffle(place)
+        self._place = place
+        self._rank = [0] * self.n_pages
+        for rank, page in enumerate(place):
+            self._rank[page] = rank
 
     def is_free(self, page: int) -> bool:
         return self._free[page]
@@ -212,6 +231,10 @@ class CacheManager:
                 if table[idx] >= 0:
                     g.pool.free(table[idx])
                     table[idx] = -1
+
+    def scramble(self, seed: int) -> None:
+        for i, g in enumerate(self.groups):
+            g.pool.scramble(seed + i)
 
     # ------------------------------------------------------------ views
     def table(self, group: int, req: Hashable) -> List[int]:

@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import json
 import mmap
+import os
 import struct
 from typing import Dict, Iterable, List, Tuple
 
@@ -105,9 +106,13 @@ def save_file(tensors: Dict[str, torch.Tensor], path: str) -> None:
         offset += nbytes
     blob = json.dumps(header, separators=(",", ":")).encode("utf-8")
     blob += b" " * ((8 - len(blob) % 8) % 8)
-    with open(path, "wb") as f:
+    # written beside the target and renamed over it: a file that is mapped
+    # somewhere (even as the source of these tensors) is never truncated
+    tmp = f"{path}.tmp{os.getpid()}"
+    with open(tmp, "wb") as f:
         f.write(struct.pack("<Q", len(blob)))
         f.write(blob)
         for name in order:
             t = tensors[name].detach().contiguous().cpu()
             f.write(t.view(torch.uint8).reshape(-1).numpy().tobytes() if t.numel() else b"")
+    os.replace(tmp, path)

@@ -1,0 +1,89 @@
+"""Shared pieces of the GPU tests: engines, cached reference logits, a batch
+context built by hand for tests of single kernels and parts."""
+import functools
+from typing import Dict, List, Sequence, Tuple
+
+import numpy as np
+import torch
+
+
+def make_engine(model_dir, dtype, **kw):
+    from imparo_amd.engine import Engine
+    kw.setdefault("max_tokens", 2048)
+    kw.setdefault("page_size", 16)
+    kw.setdefault("max_requests", 8)
+    return Engine(model_dir, dtype=dtype, **kw)
+
+
+class RefCache:
+    """Plain-implementation logits of whole sequences, computed once each."""
+
+    def __init__(self, plain):
+        self.plain = plain
+        self._memo: Dict[Tuple, torch.Tensor] = {}
+
+    def __call__(self, tokens, order=None) -> torch.Tensor:
+        key = (tuple(tokens), None if order is None else tuple(order))
+        if key not in self._memo:
+            self._memo[key] = self.plain.logits(list(tokens), order)
+        return self._memo[key]
+
+
+def step_all(engine, rid, tokens, cuts: Sequence[int]) -> torch.Tensor:
+    """Feeds `tokens` as request `rid` in portions of the sizes in `cuts`
+    (repeated as needed), wanting every position; returns [T, V] on the CPU."""
+    from imparo_amd.engine import StepEntry
+    outs, at, i = [], 0, 0
+    while at < len(tokens):
+        n = min(cuts[i % len(cuts)], len(tokens) - at)
+        outs.append(engine.step([StepEntry(rid, tokens[at:at + n], list(range(n)))]).cpu())
+        at += n
+        i += 1
+    return torch.cat(outs)
+
+
+def hand_context(segments: Sequence[Tuple[int, int]], page_size: int, n_pages: int, dtype, device,
+                 kv_sites: Dict[int, Tuple[int, int]] = None, fixed_sites: Dict[int, Tuple[int, ...]] = None,
+                 n_slots: int = 8, tables: List[List[int]] = None, slots: List[int] = None):
+    """A StepContext for rows given as (start position, number of tokens).
+    kv_sites: site -> (kv_heads, head_dim); fixed_sites: site -> state shape.
+    Pages are handed out in order unless `tables` gives them."""
+    from imparo_amd.parts.base import StepContext, Workspace
+
+    class Storage:
+        pass
+    st = Storage()
+    st.kv, st.fixed = {}, {}
+    for site, (hk, d) in (kv_sites or {}).items():
+        st.kv[site] = (torch.zeros(n_pages, hk, page_size, d, dtype=dtype, device=device),
+                       torch.zeros(n_pages, hk, page_size, d, dtype=dtype, device=device))
+    for site, shape in (fixed_sites or {}).items():
+        st.fixed[site] = torch.zeros((n_slots,) + tuple(shape), dtype=torch.float32, device=device)
+    R = len(segments)
+    pos, row, start, length = [], [], [], []
+    t = 0
+    for r, (p0, n) in enumerate(segments):
+        pos += list(range(p0, p0 + n))
+        row += [r] * n
+        start.append(t)
+        length.append(n)
+        t += n
+    if tables is None:
+        tables, nxt = [], 0
+        for p0, n in segments:
+            k = (p0 + n + page_size - 1) // page_size
+            tables.append(list(range(nxt, nxt + k)))
+            nxt += k
+        assert nxt <= n_pages
+    P = max(len(tb) for tb in tables)
+    tab = np.full((R, P), -1, dtype=np.int32)
+    for r, tb in enumerate(tables):
+        tab[r, :len(tb)] = tb
+    i32 = lambda a: torch.tensor(np.asarray(a, dtype=np.int32), device=device)
+    ctx = StepContext(
+        n_tokens=t, n_rows=R, positions=i32(pos), row_of_token=i32(row), seg_start=i32(start),
+        seg_len=i32(length), slot=i32(slots if slots is not None else list(range(R))),
+        block_tables={0: i32(tab)}, page_size=page_size, dtype=dtype, workspace=Workspace(device),
+        storage=st, group_of_site={s: 0 for s in (kv_sites or {})},
+        max_seg_len=max(length), max_context=max(p0 + n for p0, n in segments))
+    return ctx

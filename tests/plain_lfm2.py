@@ -159,17 +159,22 @@ class PlainLfm2:
         self.theta = c.get("rope_theta", 1000000.0)
         self.bias = c.get("conv_bias", False)
 
-    def mixer_attention(self, i, h, positions, window):
+    def mixer_attention(self, i, h, positions, window, shared_kv=None):
+        """Returns the mixer's output and the (k, v) it attended over; with
+        `shared_kv` the layer projects only q and reads another call's k, v."""
         p = f"model.layers.{i}.self_attn."
         T = h.shape[0]
         q = linear(h, self.w[p + "q_proj.weight"]).reshape(T, self.H, self.D)
-        k = linear(h, self.w[p + "k_proj.weight"]).reshape(T, self.Hk, self.D)
-        v = linear(h, self.w[p + "v_proj.weight"]).reshape(T, self.Hk, self.D)
         # per-head norm, then rotation, on q and k; v untouched (cpu_support.rs:361-376)
         q = rope_neox(rms_norm(q, self.w[p + "q_layernorm.weight"], self.eps), positions, self.theta, self.D)
-        k = rope_neox(rms_norm(k, self.w[p + "k_layernorm.weight"], self.eps), positions, self.theta, self.D)
+        if shared_kv is None:
+            k = linear(h, self.w[p + "k_proj.weight"]).reshape(T, self.Hk, self.D)
+            v = linear(h, self.w[p + "v_proj.weight"]).reshape(T, self.Hk, self.D)
+            k = rope_neox(rms_norm(k, self.w[p + "k_layernorm.weight"], self.eps), positions, self.theta, self.D)
+        else:
+            k, v = shared_kv
         o = attend(q, k, v, positions, 1.0 / math.sqrt(self.D), window)
-        return linear(o.reshape(T, self.H * self.D), self.w[p + "out_proj.weight"])
+        return linear(o.reshape(T, self.H * self.D), self.w[p + "out_proj.weight"]), (k, v)
 
     def mixer_conv(self, i, h):
         p = f"model.layers.{i}.conv."
@@ -178,28 +183,35 @@ class PlainLfm2:
         y, _ = short_conv(bcx, self.w[p + "conv.weight"], b("conv.bias"))
         return linear(y, self.w[p + "out_proj.weight"], b("out_proj.bias"))
 
-    def hidden(self, tokens):
+    def hidden(self, tokens, order=None):
+        """`order`: list of (layer, cache_of) calls; None runs every layer once.
+        cache_of names an earlier call whose k, v this call reads."""
         tokens = torch.as_tensor(tokens, dtype=torch.long)
         T = tokens.shape[0]
         positions = np.arange(T)
         x = self.w["model.embed_tokens.weight"][tokens]
-        for i, kind in enumerate(self.cfg["layer_types"]):
+        if order is None:
+            order = [(i, None) for i in range(len(self.cfg["layer_types"]))]
+        kv_of_call = {}
+        for c, (i, cache_of) in enumerate(order):
+            kind = self.cfg["layer_types"][i]
             p = f"model.layers.{i}."
             h = rms_norm(x, self.w[p + "operator_norm.weight"], self.eps)
             if kind == "conv":
                 m = self.mixer_conv(i, h)
             else:
                 window = self.cfg.get("sliding_window") if kind == "sliding_attention" else None
-                m = self.mixer_attention(i, h, positions, window)
+                m, kv_of_call[c] = self.mixer_attention(i, h, positions, window,
+                                                        None if cache_of is None else kv_of_call[cache_of])
             x = x + m
             n = rms_norm(x, self.w[p + "ffn_norm.weight"], self.eps)
             x = x + swiglu(n, self.w[p + "feed_forward.w1.weight"], self.w[p + "feed_forward.w3.weight"],
                            self.w[p + "feed_forward.w2.weight"])
         return x
 
-    def logits(self, tokens):
+    def logits(self, tokens, order=None):
         """Logits [T, V] of one whole sequence from position 0."""
-        x = self.hidden(tokens)
+        x = self.hidden(tokens, order)
         head = self.w["model.embed_tokens.weight"] if self.cfg.get("tie_embedding", True) \
             else self.w["lm_head.weight"]
         return linear(rms_norm(x, self.w["model.embedding_norm.weight"], self.eps), head)

@@ -1,0 +1,181 @@
+"""The cache manager on the host: no page lost, held twice or freed twice,
+under random orders of requests; lowest-free allocation; windows; rollback."""
+import random
+
+import pytest
+
+from imparo_amd.cache import (PagePool, CacheManager, PagedSpec, FixedSpec, OutOfPages, CacheError)
+
+
+def test_lowest_free_page_always():
+    # the reference's sequence (/root/reference/crates/imparo-kv/src/alloc.rs:147-276 as the survey
+    # records it): 0,1,2,3; free 2 and 0; next 0, 2, 4
+    p = PagePool(8)
+    assert [p.alloc() for _ in range(4)] == [0, 1, 2, 3]
+    p.free(2)
+    p.free(0)
+    assert [p.alloc() for _ in range(3)] == [0, 2, 4]
+    assert p.high_water == 5
+
+
+def test_ascending_after_churn_and_purity():
+    rng = random.Random(0)
+    p = PagePool(64)
+    held = set()
+    for _ in range(2000):
+        if held and (rng.random() < 0.5 or p.n_free == 0):
+            page = rng.choice(sorted(held))
+            p.free(page)
+            held.remove(page)
+        else:
+            page = p.alloc()
+            assert page == min(set(range(64)) - held)      # a function of the free set only
+            held.add(page)
+    for page in sorted(held):
+        p.free(page)
+    assert [p.alloc() for _ in range(64)] == list(range(64))
+
+
+def test_double_free_and_exhaustion():
+    p = PagePool(2)
+    a = p.alloc()
+    p.alloc()
+    with pytest.raises(OutOfPages):
+        p.alloc()
+    p.free(a)
+    with pytest.raises(CacheError, match="freed twice"):
+        p.free(a)
+    with pytest.raises(CacheError):
+        p.free(9)
+
+
+def test_scrambled_placement_is_a_permutation():
+    p = PagePool(16)
+    p.scramble(3)
+    got = [p.alloc() for _ in range(16)]
+    assert sorted(got) == list(range(16)) and got != list(range(16))
+    p.free(got[5])
+    assert p.alloc() == got[5]
+
+
+SITES = [FixedSpec((2, 8)), PagedSpec(2, 16), FixedSpec((2, 8)), PagedSpec(2, 16), PagedSpec(2, 16, window=10), None]
+
+
+def test_groups_follow_the_specs():
+    m = CacheManager(SITES, page_size=4, n_pages=10, n_slots=3)
+    assert len(m.groups) == 2
+    assert m.groups[0].sites == [1, 3] and m.groups[1].sites == [4]
+    assert m.fixed_sites == [0, 2] and m.group_of_site == {1: 0, 3: 0, 4: 1}
+
+
+def test_reserve_commit_release():
+    m = CacheManager(SITES, page_size=4, n_pages=10, n_slots=3)
+    assert m.admit("a") == 0 and m.admit("b") == 1
+    m.reserve("a", 9)
+    m.commit("a", 9)
+    assert m.table(0, "a") == [0, 1, 2] and m.length["a"] == 9
+    m.reserve("b", 4)
+    m.commit("b", 4)
+    assert m.table(0, "b") == [3]
+    m.reserve("a", 10)           # still inside page 2
+    m.commit("a", 10)
+    assert m.table(0, "a") == [0, 1, 2]
+    m.release("a")
+    assert m.free_pages()[0] == 9
+    assert m.admit("c") == 0      # slot reused
+    m.reserve("c", 5)
+    assert m.table(0, "c") == [0, 1]    # pages reused, lowest first
+    m.check()
+    with pytest.raises(CacheError):
+        m.release("zzz")
+    with pytest.raises(CacheError):
+        m.admit("b")
+
+
+def test_reserve_is_all_or_nothing():
+    m = CacheManager(SITES, page_size=4, n_pages=4, n_slots=2)
+    m.admit("a")
+    m.reserve("a", 8)
+    m.commit("a", 8)
+    m.admit("b")
+    before = (m.free_pages(), list(m.table(0, "b")), list(m.table(1, "b")))
+    with pytest.raises(OutOfPages):
+        m.reserve("b", 12)       # needs 3 pages, 2 are free
+    assert (m.free_pages(), m.table(0, "b"), m.table(1, "b")) == before
+    got = m.reserve("b", 8)
+    m.rollback("b", got)
+    assert (m.free_pages(), m.table(0, "b"), m.table(1, "b")) == before
+    m.check()
+
+
+def test_slots_run_out():
+    m = CacheManager(SITES, page_size=4, n_pages=4, n_slots=1)
+    m.admit("a")
+    with pytest.raises(OutOfPages, match="slots"):
+        m.admit("b")
+
+
+def test_a_window_gives_pages_back_as_it_passes_them():
+    m = CacheManager([PagedSpec(1, 16, window=10), PagedSpec(1, 16)], page_size=4, n_pages=64, n_slots=1)
+    m.admit("a")
+    for n in range(1, 41):
+        m.reserve("a", n)
+        m.commit("a", n)
+        win, full = m.table(0, "a"), m.table(1, "a")
+        # the next query sits at position n and reads keys n+1-10 .. n
+        lo = max(0, n + 1 - 10)
+        for idx, page in enumerate(win):
+            needed = (idx + 1) * 4 > lo
+            assert (page >= 0) == needed, (n, idx, win)
+        assert all(p >= 0 for p in full)
+        assert m.held_pages("a")[0] <= 10 // 4 + 2
+        m.check()
+    # a long portion keeps what its own first query needs
+    m.release("a")
+    m.admit("b")
+    m.reserve("b", 30)
+    assert all(p >= 0 for p in m.table(0, "b"))
+    m.commit("b", 30)
+    assert m.table(0, "b")[:5] == [-1] * 5      # keys below 21 are behind the window of position 30
+    m.reserve("b", 50)
+    assert m.table(0, "b")[5] >= 0
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_random_orders_never_lose_or_share_a_page(seed):
+    rng = random.Random(seed)
+    m = CacheManager(SITES, page_size=4, n_pages=24, n_slots=4)
+    live = {}
+    next_id = 0
+    for _ in range(1500):
+        action = rng.random()
+        if action < 0.25 and len(live) < 4:
+            rid = f"r{next_id}"
+            next_id += 1
+            m.admit(rid)
+            live[rid] = 0
+        elif action < 0.85 and live:
+            rid = rng.choice(sorted(live))
+            grow = rng.choice([1, 1, 1, 2, 7, 19])
+            try:
+                got = m.reserve(rid, live[rid] + grow)
+            except OutOfPages:
+                m.check()
+                continue
+            if rng.random() < 0.1:
+                m.rollback(rid, got)
+            else:
+                live[rid] += grow
+                m.commit(rid, live[rid])
+        elif live:
+            rid = rng.choice(sorted(live))
+            m.release(rid)
+            del live[rid]
+        m.check()
+        for rid, n in live.items():
+            assert m.length[rid] == n
+            assert len(m.table(0, rid)) == (n + 3) // 4 or len(m.table(0, rid)) >= (n + 3) // 4
+    for rid in list(live):
+        m.release(rid)
+    m.check()
+    assert m.free_pages() == [24, 24] and m.slots.n_free == 4

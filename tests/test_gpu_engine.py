@@ -1,0 +1,309 @@
+"""The engine against the plain implementation, in float32 and in bfloat16:
+each request alone and whole; most of it in one step and the last 32 tokens one
+by one; portions of changing size down to two tokens; mixed batches of up to
+four live requests with so few pages that they are used again; long decoding;
+the first tokens of a sequence. Variants with sharpened attention make a
+single wrong or missing key visible, which random weights would average away.
+"""
+import os
+import random
+
+import pytest
+import torch
+
+from conftest import prompt_tokens
+from gpu_helpers import make_engine, RefCache, step_all
+from tolerances import check_logits, BF16_REL
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+MODELS = ["A", "B", "C", "A_sharp", "C_sharp"]
+
+
+@pytest.fixture(scope="module")
+def zoo(model_dirs, tmp_path_factory):
+    """Model folders (with the sharpened variants), plain models, reference caches."""
+    from safetensors.torch import load_file
+    from imparo_amd.weights import save_file
+    from plain_lfm2 import PlainLfm2
+    import json, shutil
+    dirs = dict(model_dirs)
+    for base in ("A", "C"):
+        d = str(tmp_path_factory.mktemp(f"tiny_{base}_sharp"))
+        shutil.copy(os.path.join(model_dirs[base], "config.json"), d)
+        t = load_file(os.path.join(model_dirs[base], "model.safetensors"))
+        for k in list(t):
+            # scores scale with |q||k|: with both norms times 3 their spread is 9 instead of 1 and
+            # the softmax picks out single keys. (Not more: a score of size s carries a bfloat16
+            # rounding of s * 2^-8 from q and k, which at times 5 alone would move weights by 10%.)
+            if k.endswith("q_layernorm.weight") or k.endswith("k_layernorm.weight"):
+                t[k] = (t[k].float() * 3.0).to(t[k].dtype)
+        save_file(t, os.path.join(d, "model.safetensors"))
+        dirs[base + "_sharp"] = d
+    plains = {k: PlainLfm2(v) for k, v in dirs.items()}
+    return dirs, {k: RefCache(p) for k, p in plains.items()}
+
+
+@pytest.fixture(scope="module")
+def engines(zoo):
+    cache = {}
+
+    def get(name, dtype, **kw):
+        key = (name, dtype, tuple(sorted(kw.items())))
+        if key not in cache:
+            cache[key] = make_engine(zoo[0][name], dtype, **kw)
+        return cache[key]
+    return get
+
+
+def vocab_of(zoo, name):
+    return zoo[1][name].plain.cfg["vocab_size"]
+
+
+@pytest.fixture(scope="module")
+def yardstick(zoo, engines):
+    """What a run is held to: the plain implementation, except for sharpened
+    models in bfloat16, which are held to the same engine's whole-prompt run
+    (see tolerances.py)."""
+    memo = {}
+
+    def get(name, dtype, toks, order=None):
+        if not (name.endswith("_sharp") and dtype == "bfloat16"):
+            return zoo[1][name](toks, order), None
+        key = (name, tuple(toks))
+        if key not in memo:
+            eng = engines(name, dtype)
+            memo[key] = step_all(eng, "yardstick", toks, [len(toks)])
+            eng.release("yardstick")
+        return memo[key], BF16_REL
+    return get
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", MODELS)
+def test_each_request_alone_and_whole(zoo, engines, yardstick, name, dtype):
+    eng = engines(name, dtype)
+    for n, seed in ((5, 1), (17, 2), (31, 3), (150, 4)):
+        toks = prompt_tokens(vocab_of(zoo, name), n, seed)
+        ref, rel = yardstick(name, dtype, toks)
+        # (a sharpened model in bfloat16 is its own yardstick whole: decode it instead)
+        got = step_all(eng, "w", toks, [n] if rel is None else [1])
+        eng.release("w")
+        check_logits(got, ref, dtype, f"{name} whole {n}", rel)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", MODELS)
+def test_last_32_tokens_one_by_one(zoo, engines, yardstick, name, dtype):
+    eng = engines(name, dtype)
+    toks = prompt_tokens(vocab_of(zoo, name), 150, 4)
+    got = step_all(eng, "s", toks, [118] + [1] * 32)
+    eng.release("s")
+    ref, rel = yardstick(name, dtype, toks)
+    check_logits(got, ref, dtype, f"{name} stepwise", rel)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", MODELS)
+def test_portions_of_changing_size(zoo, engines, yardstick, name, dtype):
+    eng = engines(name, dtype)
+    toks = prompt_tokens(vocab_of(zoo, name), 150, 4)
+    ref, rel = yardstick(name, dtype, toks)
+    for cuts in ([2, 3, 7, 2, 16, 5, 33, 2, 1, 64], [4], [7], [2], [63, 1, 2, 17]):
+        got = step_all(eng, "p", toks, cuts)
+        eng.release("p")
+        check_logits(got, ref, dtype, f"{name} portions {cuts}", rel)
+
+
+def _mixed_schedule(rng, lengths, max_live=4):
+    """A schedule of steps: each step gives some live requests a portion or
+    one token. Returns [(step entries [(rid, lo, hi)], ends [rid])]."""
+    waiting = list(range(len(lengths)))
+    fed = {}
+    steps = []
+    while waiting or fed:
+        while waiting and len(fed) < max_live and (not fed or rng.random() < 0.6):
+            fed[waiting.pop(0)] = 0
+        entries, ends = [], []
+        for rid in sorted(fed):
+            if rng.random() < 0.25 and len(fed) > 1:
+                continue                                  # left out of this step, goes on later
+            left = lengths[rid] - fed[rid]
+            n = min(left, rng.choice([1, 1, 1, 2, 2, 3, 5, 9, 16, 40]))
+            entries.append((rid, fed[rid], fed[rid] + n))
+            fed[rid] += n
+            if fed[rid] == lengths[rid]:
+                ends.append(rid)
+        for rid in ends:
+            del fed[rid]
+        if entries:
+            steps.append((entries, ends))
+    return steps
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", MODELS)
+def test_mixed_batches_with_pages_used_again(zoo, engines, yardstick, name, dtype):
+    from imparo_amd.engine import StepEntry
+    rng = random.Random(11)
+    lengths = [70, 33, 121, 9, 64, 50, 97, 18]
+    V = vocab_of(zoo, name)
+    prompts = [prompt_tokens(V, n, 100 + i) for i, n in enumerate(lengths)]
+    # pages of 8; four live requests of up to 121 tokens need at most 4*16 pages: 40 forces reuse
+    eng = engines(name, dtype, page_size=8, max_tokens=40 * 8, max_requests=4)
+    steps = _mixed_schedule(rng, lengths)
+    got = {i: [] for i in range(len(lengths))}
+    used = set()
+    for entries, ends in steps:
+        batch = [StepEntry(f"m{rid}", prompts[rid][lo:hi], list(range(hi - lo))) for rid, lo, hi in entries]
+        out = eng.step(batch).cpu()
+        for g in eng.cache.groups:
+            for tab in g.tables.values():
+                used.update(p for p in tab if p >= 0)
+        at = 0
+        for rid, lo, hi in entries:
+            got[rid].append(out[at:at + hi - lo])
+            at += hi - lo
+        for rid in ends:
+            eng.release(f"m{rid}")
+        eng.cache.check()
+    total_pages_asked = sum((n + 7) // 8 for n in lengths)
+    assert total_pages_asked > 40 >= len(used), "the schedule must make requests share pages over time"
+    assert eng.free_pages() == [40] * len(eng.cache.groups)
+    for rid, n in enumerate(lengths):
+        ref, rel = yardstick(name, dtype, prompts[rid])
+        check_logits(torch.cat(got[rid]), ref, dtype, f"{name} mixed request {rid}", rel)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C_sharp"])
+def test_long_decoding(zoo, engines, yardstick, name, dtype):
+    eng = engines(name, dtype)
+    toks = prompt_tokens(vocab_of(zoo, name), 330, 7)
+    got = step_all(eng, "l", toks, [4] + [1] * 326)
+    eng.release("l")
+    ref, rel = yardstick(name, dtype, toks)
+    check_logits(got, ref, dtype, f"{name} long decoding", rel)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_first_tokens(zoo, engines, name, dtype):
+    eng = engines(name, dtype)
+    for n in (1, 2, 3, 4):
+        toks = prompt_tokens(vocab_of(zoo, name), n, 20 + n)
+        for cuts in ([n], [1]):
+            got = step_all(eng, "f", toks, cuts)
+            eng.release("f")
+            check_logits(got, zoo[1][name](toks), dtype, f"{name} first {n} tokens cut {cuts}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_wanted_places_only(zoo, engines, dtype):
+    """`want` picks rows; a step that wants nothing returns nothing but still fills the cache."""
+    from imparo_amd.engine import StepEntry
+    eng = engines("B", dtype)
+    toks = prompt_tokens(vocab_of(zoo, "B"), 40, 5)
+    ref = zoo[1]["B"](toks)
+    assert eng.step([StepEntry("x", toks[:20], [])]) is None
+    out = eng.step([StepEntry("x", toks[20:], [19, 0, 7]), StepEntry("y", toks[:9], [8])]).cpu()
+    eng.release("x"), eng.release("y")
+    check_logits(out, torch.stack([ref[39], ref[20], ref[27], ref[8]]), dtype, "wanted places")
+
+
+def test_placement_is_invisible(zoo, engines):
+    """Permuted page placement gives the same bits (float32 and bfloat16)."""
+    for dtype in DTYPES:
+        toks = prompt_tokens(vocab_of(zoo, "C_sharp"), 100, 9)
+        base = step_all(engines("C_sharp", dtype), "q", toks, [13, 1, 1, 40])
+        engines("C_sharp", dtype).release("q")
+        eng = make_engine(zoo[0]["C_sharp"], dtype)
+        eng.cache.scramble(5)
+        got = step_all(eng, "q", toks, [13, 1, 1, 40])
+        assert any(t != sorted(t) or t[0] != 0 for g in eng.cache.groups for t in g.tables.values())
+        assert torch.equal(got, base)
+
+
+def test_cutting_and_batching_leave_float32_bits_alone(zoo, engines):
+    """In float32 every sum runs in an order fixed by the position, so the way
+    of cutting changes nothing at all."""
+    eng = engines("B", "float32")
+    toks = prompt_tokens(vocab_of(zoo, "B"), 90, 12)
+    a = step_all(eng, "a", toks, [90])
+    eng.release("a")
+    b = step_all(eng, "a", toks, [3, 1, 20, 2])
+    eng.release("a")
+    assert torch.equal(a, b)
+
+
+def test_a_step_that_does_not_fit_changes_nothing(zoo):
+    from imparo_amd.engine import StepEntry
+    from imparo_amd.cache import OutOfPages
+    eng = make_engine(zoo[0]["A"], "float32", page_size=8, max_tokens=64, max_requests=2)
+    toks = prompt_tokens(vocab_of(zoo, "A"), 60, 3)
+    ref = zoo[1]["A"](toks)
+    first = eng.step([StepEntry("a", toks[:30], list(range(30)))]).cpu()
+    free = eng.free_pages()
+    with pytest.raises(OutOfPages):      # a's 10 more fit, b's 40 do not: neither advances
+        eng.step([StepEntry("a", toks[30:40], [0]), StepEntry("b", toks[:40], [0])])
+    assert eng.free_pages() == free and eng.length("a") == 30 and not eng.is_live("b")
+    rest = eng.step([StepEntry("a", toks[30:], list(range(30)))]).cpu()
+    check_logits(torch.cat([first, rest]), ref, "float32", "after a refused step")
+    with pytest.raises(OutOfPages):      # the pool holds 64 positions
+        eng.step([StepEntry("a", toks[:10], [])])
+    eng.release("a")
+    assert eng.free_pages() == [8]
+
+
+def test_refused_batches(zoo, engines):
+    from imparo_amd.engine import StepEntry, StepError
+    eng = engines("A", "float32")
+    with pytest.raises(StepError, match="outside the vocabulary"):
+        eng.step([StepEntry("r", [1, 256], [0])])
+    with pytest.raises(StepError, match="twice"):
+        eng.step([StepEntry("r", [1], [0]), StepEntry("r", [2], [0])])
+    with pytest.raises(StepError, match="wanted place"):
+        eng.step([StepEntry("r", [1, 2], [2])])
+    with pytest.raises(StepError, match="no tokens"):
+        eng.step([StepEntry("r", [], [])])
+    assert not eng.is_live("r")
+
+
+def test_run_order_with_a_layer_twice_and_a_borrowed_cache(zoo, tmp_path):
+    """The order layers run in is data: a plan that runs layer 1 twice, the
+    second time reading the first call's keys and values, and layer 0 twice
+    with a state of its own each time."""
+    import dataclasses, json, shutil
+    from imparo_amd.config import register_architecture, Lfm2Config, LayerCall
+    from imparo_amd.config import lfm2
+    order = [(0, None), (1, None), (1, 1), (2, None), (0, None), (3, None)]
+
+    def build(cfg):
+        plan = lfm2.build_plan(cfg)
+        return dataclasses.replace(plan, architecture="TestLfm2Reordered",
+                                   order=[LayerCall(l, c) for l, c in order])
+    register_architecture("TestLfm2Reordered", Lfm2Config.from_dict, build)
+    d = str(tmp_path / "reordered")
+    shutil.copytree(zoo[0]["A_sharp"], d)
+    cfg = json.load(open(os.path.join(d, "config.json")))
+    cfg["architectures"] = ["TestLfm2Reordered"]
+    json.dump(cfg, open(os.path.join(d, "config.json"), "w"))
+    toks = prompt_tokens(256, 80, 31)
+    ref = zoo[1]["A_sharp"](toks, order)
+    assert not torch.allclose(ref, zoo[1]["A_sharp"](toks), atol=1e-3)
+    for dtype in DTYPES:
+        eng = make_engine(d, dtype)
+        assert len(eng.cache.fixed_sites) == 3 and len(eng.cache.groups[0].sites) == 2
+        got = step_all(eng, "o", toks, [9, 1, 1, 30, 2])
+        if dtype == "float32":
+            check_logits(got, ref, dtype, "reordered float32")
+        else:       # a sharpened model: in bfloat16 it is held to its own whole-prompt run
+            eng.release("o")
+            check_logits(got, step_all(eng, "o", toks, [80]), dtype, "reordered bfloat16", BF16_REL)
+    # the same order on the unsharpened weights, against the plain implementation in bfloat16
+    d2 = str(tmp_path / "reordered_plain")
+    shutil.copytree(zoo[0]["A"], d2)
+    json.dump(cfg, open(os.path.join(d2, "config.json"), "w"))
+    check_logits(step_all(make_engine(d2, "bfloat16"), "o", toks, [9, 1, 1, 30, 2]), zoo[1]["A"](toks, order),
+                 "bfloat16", "reordered bfloat16 against plain")

@@ -1,0 +1,296 @@
+"""Each kernel alone beside a plain reference, at sizes other than the
+engine's: odd row counts, widths and vocabularies that are no power of two,
+head sizes in steps of 16, several head/group counts, windows, short segments.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_lfm2 as P
+from gpu_helpers import hand_context
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def ops():
+    from imparo_amd.kernels import ops as o
+    return o
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * scale
+
+
+# ---------------------------------------------------------------- GEMM
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 33, 64, 65, 130, 300])
+@pytest.mark.parametrize("n,k", [(16, 8), (40, 96), (136, 264), (200, 1032), (1000, 64)])
+def test_gemm(m, n, k):
+    x, w = rnd(m, k, seed=m), rnd(n, k, seed=n + 1)
+    # float32: exact products, sums of at most 1032 terms
+    out = torch.empty(m, n, dtype=torch.float32, device=DEV)
+    ops().gemm(x.to(DEV), w.to(DEV), out)
+    ref = x.double() @ w.double().t()
+    assert (out.cpu().double() - ref).abs().max() <= 1e-6 * math.sqrt(k) * ref.abs().max()
+    # bfloat16 operands: products are exact in float32, accumulation is float32
+    xb, wb = x.to(torch.bfloat16), w.to(torch.bfloat16)
+    ref = xb.double() @ wb.double().t()
+    out = torch.empty(m, n, dtype=torch.float32, device=DEV)
+    ops().gemm(xb.to(DEV), wb.to(DEV), out)
+    assert (out.cpu().double() - ref).abs().max() <= 1e-6 * math.sqrt(k) * ref.abs().max()
+    outb = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    ops().gemm(xb.to(DEV), wb.to(DEV), outb)
+    assert torch.equal(outb.cpu(), out.cpu().to(torch.bfloat16))      # only the final rounding differs
+
+
+def test_gemm_refuses_what_it_cannot_take():
+    from imparo_amd.kernels import KernelArgumentError
+    x, w = rnd(4, 12).to(torch.bfloat16).to(DEV), rnd(8, 12).to(torch.bfloat16).to(DEV)
+    with pytest.raises(KernelArgumentError, match="multiple of 8"):
+        ops().gemm(x, w, torch.empty(4, 8, dtype=torch.float32, device=DEV))
+    with pytest.raises(KernelArgumentError, match="columns"):
+        ops().gemm(rnd(4, 16).to(DEV), rnd(8, 24).to(DEV), torch.empty(4, 8, device=DEV))
+    with pytest.raises(KernelArgumentError, match="GPU only"):
+        ops().gemm(rnd(4, 16), rnd(8, 16), torch.empty(4, 8))
+    # float32 takes any inner size
+    out = torch.empty(3, 5, device=DEV)
+    ops().gemm(rnd(3, 7).to(DEV), rnd(5, 7, seed=1).to(DEV), out)
+    torch.testing.assert_close(out.cpu(), rnd(3, 7) @ rnd(5, 7, seed=1).t(), rtol=1e-5, atol=1e-5)
+
+
+# ---------------------------------------------------------------- rows
+@pytest.mark.parametrize("width", [16, 100, 2048, 2500])
+def test_rms_norm(width):
+    x, d, w = rnd(7, width, seed=1), rnd(7, width, seed=2), 1 + 0.1 * rnd(width, seed=3)
+    for eps in (1e-5, 1e-2):
+        out = torch.empty(7, width, device=DEV)
+        ops().rms_norm(x.to(DEV), w.to(DEV), eps, out)
+        torch.testing.assert_close(out.cpu(), P.rms_norm(x, w, eps), rtol=2e-6, atol=2e-6)
+    # fused add, written back
+    xd = x.to(DEV).clone()
+    out = torch.empty(7, width, dtype=torch.bfloat16, device=DEV)
+    ops().rms_norm(xd, w.to(DEV), 1e-5, out, delta=d.to(DEV), write_back=True)
+    assert torch.equal(xd.cpu(), x + d)
+    ref = P.rms_norm(x + d, w, 1e-5)
+    assert (out.cpu().float() - ref).abs().max() <= 2 ** -8 * ref.abs().max()
+    # selected rows, with a delta, nothing written back
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32, device=DEV)
+    xd = x.to(DEV).clone()
+    out = torch.empty(3, width, device=DEV)
+    ops().rms_norm(xd, w.to(DEV), 1e-5, out, delta=d.to(DEV), rows=rows)
+    assert torch.equal(xd.cpu(), x)
+    torch.testing.assert_close(out.cpu(), P.rms_norm((x + d)[[5, 0, 5]], w, 1e-5), rtol=2e-6, atol=2e-6)
+
+
+def test_embed_gather_and_silu_mul():
+    table = rnd(37, 24, seed=4)
+    ids = torch.tensor([36, 0, 5, 5], dtype=torch.int32, device=DEV)
+    for t in (table, table.to(torch.bfloat16)):
+        out = torch.empty(4, 24, device=DEV)
+        ops().embed_gather(t.to(DEV), ids, out)
+        assert torch.equal(out.cpu(), t.float()[[36, 0, 5, 5]])
+    gu = rnd(5, 2 * 88, seed=5, scale=3.0)
+    out = torch.empty(5, 88, device=DEV)
+    ops().silu_mul(gu.to(DEV), out)
+    torch.testing.assert_close(out.cpu(), P.silu(gu[:, :88]) * gu[:, 88:], rtol=2e-6, atol=1e-6)
+    out = torch.empty(5, 88, dtype=torch.bfloat16, device=DEV)
+    ops().silu_mul(gu.to(DEV), out)
+    assert torch.equal(out.cpu(), (P.silu(gu[:, :88]) * gu[:, 88:]).to(torch.bfloat16)) or \
+        (out.cpu().float() - P.silu(gu[:, :88]) * gu[:, 88:]).abs().max() < 0.05
+
+
+# ---------------------------------------------------------------- norm + rotation + cache write
+@pytest.mark.parametrize("H,Hk,D,rot", [(4, 2, 16, 16), (3, 1, 48, 48), (6, 3, 64, 32), (2, 2, 80, 80), (5, 1, 128, 0)])
+@pytest.mark.parametrize("page_size", [4, 16])
+def test_qk_norm_rope_store(H, Hk, D, rot, page_size):
+    segments = [(0, 5), (37, 1), (9, 3)]
+    tables = [[3, 1], list(range(4, 4 + 40 // page_size + 1)), [0, 2, 14][: (12 + page_size - 1) // page_size]]
+    n_pages = 16
+    for dtype in (torch.float32, torch.bfloat16):
+        ctx = hand_context(segments, page_size, n_pages, dtype, DEV, kv_sites={0: (Hk, D)}, tables=tables)
+        T = ctx.n_tokens
+        qkv = rnd(T, (H + 2 * Hk) * D, seed=D)
+        qw, kw = 1 + 0.1 * rnd(D, seed=1), 1 + 0.1 * rnd(D, seed=2)
+        base = 10000.0
+        inv = None
+        if rot:
+            i = np.arange(rot // 2, dtype=np.float32)
+            inv = torch.from_numpy(np.power(np.float32(base), (np.float32(-2.0) * i / np.float32(rot))).astype(np.float32)).to(DEV)
+        k_cache, v_cache, table = ctx.kv(0)
+        q_out = torch.empty(T, H, D, dtype=dtype, device=DEV)
+        ops().qk_norm_rope_store(qkv.to(DEV), qw.to(DEV), kw.to(DEV), 1e-5, inv, ctx.positions, ctx.row_of_token,
+                                 table, page_size, q_out, k_cache, v_cache, H, Hk, D)
+        positions = ctx.positions.cpu().tolist()
+        q = qkv[:, :H * D].reshape(T, H, D)
+        k = qkv[:, H * D:(H + Hk) * D].reshape(T, Hk, D)
+        v = qkv[:, (H + Hk) * D:].reshape(T, Hk, D)
+        q_ref, k_ref = P.rms_norm(q, qw, 1e-5), P.rms_norm(k, kw, 1e-5)
+        if rot:
+            q_ref, k_ref = P.rope_neox(q_ref, positions, base, rot), P.rope_neox(k_ref, positions, base, rot)
+        tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -7)
+        torch.testing.assert_close(q_out.cpu().float(), q_ref, **tol)
+        rows = ctx.row_of_token.cpu().tolist()
+        written = torch.zeros(n_pages, page_size, dtype=torch.bool)
+        for t, (pos, r) in enumerate(zip(positions, rows)):
+            page = tables[r][pos // page_size]
+            written[page, pos % page_size] = True
+            torch.testing.assert_close(k_cache[page, :, pos % page_size].cpu().float(), k_ref[t], **tol)
+            torch.testing.assert_close(v_cache[page, :, pos % page_size].cpu().float(), v[t], **tol)
+        # nothing else was touched
+        untouched = ~written
+        assert k_cache.cpu().float().permute(0, 2, 1, 3)[untouched].abs().sum() == 0
+        assert v_cache.cpu().float().permute(0, 2, 1, 3)[untouched].abs().sum() == 0
+
+
+# ---------------------------------------------------------------- attention
+def _attention_case(H, Hk, D, page_size, window, dtype, sharpen=None, seed=0):
+    """Rows at different depths of their contexts; the cache is filled by hand
+    from whole-sequence k, v; the reference attends over the whole sequences."""
+    ctx_lens = [70, 1, 200, 33]
+    q_lens = [5, 1, 1, 33]                      # the last q_len positions of each context are queried
+    n_pages = sum((c + page_size - 1) // page_size for c in ctx_lens) + 3
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(seed)).tolist()
+    tables, nxt = [], 0
+    for c in ctx_lens:
+        k = (c + page_size - 1) // page_size
+        tables.append(perm[nxt:nxt + k])
+        nxt += k
+    segments = [(c - ql, ql) for c, ql in zip(ctx_lens, q_lens)]
+    ctx = hand_context(segments, page_size, n_pages, dtype, DEV, kv_sites={0: (Hk, D)}, tables=tables)
+    k_cache, v_cache, table = ctx.kv(0)
+    k_cache.fill_(float("nan"))                # a key read from outside the context poisons the output
+    v_cache.fill_(float("nan"))
+    qs, refs = [], []
+    for r, (c, ql) in enumerate(zip(ctx_lens, q_lens)):
+        q, k, v = rnd(c, H, D, seed=seed + 10 * r), rnd(c, Hk, D, seed=seed + 10 * r + 1), rnd(c, Hk, D, seed=seed + 10 * r + 2)
+        if sharpen is not None:                # one far key stands out for the last query
+            far = sharpen(c)
+            k[far] = 0
+            k[far, :, 0] = 12.0
+            q[-1] = 0
+            q[-1, :, 0] = 12.0
+        q, k, v = (t.to(dtype).float() for t in (q, k, v))
+        for p in range(c):
+            page = tables[r][p // page_size]
+            k_cache[page, :, p % page_size] = k[p].to(dtype).to(DEV)
+            v_cache[page, :, p % page_size] = v[p].to(dtype).to(DEV)
+        ref = P.attend(q, k, v, range(c), 1.0 / math.sqrt(D), window)
+        qs.append(q[c - ql:])
+        refs.append(ref[c - ql:])
+    q_all = torch.cat(qs).to(dtype).to(DEV)
+    out = torch.empty(ctx.n_tokens, H * D, dtype=dtype, device=DEV)
+    ops().attention(q_all, k_cache, v_cache, out, ctx.positions, ctx.row_of_token, table, 1.0 / math.sqrt(D), window)
+    return out.cpu().float().reshape(-1, H, D), torch.cat(refs)
+
+
+@pytest.mark.parametrize("H,Hk,D", [(1, 1, 16), (6, 2, 48), (5, 5, 64), (8, 1, 128), (4, 2, 80)])
+@pytest.mark.parametrize("page_size,window", [(4, None), (16, None), (64, None), (8, 19), (16, 64), (4, 1)])
+def test_attention(H, Hk, D, page_size, window):
+    got, ref = _attention_case(H, Hk, D, page_size, window, torch.float32)
+    torch.testing.assert_close(got, ref, rtol=1e-5, atol=1e-5)
+    got, ref = _attention_case(H, Hk, D, page_size, window, torch.bfloat16)
+    torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)      # one rounding of the output, P in float32
+
+
+@pytest.mark.parametrize("where", ["first", "page_edge", "middle"])
+def test_attention_finds_one_far_key_among_hundreds(where):
+    pick = {"first": lambda c: 0, "page_edge": lambda c: (c // 2 // 16) * 16, "middle": lambda c: c // 3}[where]
+    for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 2 ** -6)):
+        got, ref = _attention_case(4, 2, 64, 16, None, dtype, sharpen=pick)
+        torch.testing.assert_close(got, ref, rtol=tol, atol=tol)
+        # the test means something: with the far key the last query's output is that key's value
+    # the last row's query sits at 199 and its far key at 66: a window of 133 starts at 67 and
+    # leaves it out, one of 134 starts at 66 and takes it in; the edge decides the output
+    for window, dtype in ((133, torch.float32), (134, torch.float32), (133, torch.bfloat16), (134, torch.bfloat16)):
+        got, ref = _attention_case(2, 1, 32, 8, window, dtype, sharpen=lambda c: c // 3)
+        torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)
+
+
+# ---------------------------------------------------------------- short conv
+@pytest.mark.parametrize("width,taps", [(8, 2), (100, 3), (300, 4), (64, 7)])
+def test_short_conv(width, taps):
+    segments = [(0, 1), (0, 9), (0, 2), (0, 40)]            # segments shorter than the history too
+    slots = [3, 0, 5, 1]
+    w = rnd(width, 1, taps, seed=1, scale=0.3)
+    bias = rnd(width, seed=2, scale=0.1)
+    for use_bias in (False, True):
+        ctx = hand_context(segments, 16, 16, torch.float32, DEV, fixed_sites={0: (taps - 1, width)}, slots=slots)
+        state = ctx.fixed_state(0)
+        state0 = rnd(8, taps - 1, width, seed=3)
+        state.copy_(state0)
+        bcx = rnd(ctx.n_tokens, 3 * width, seed=4)
+        for out_dtype in (torch.float32, torch.bfloat16):
+            state.copy_(state0)
+            out = torch.empty(ctx.n_tokens, width, dtype=out_dtype, device=DEV)
+            ops().short_conv(bcx.to(DEV), w.reshape(width, taps).to(DEV), bias.to(DEV) if use_bias else None, state,
+                             ctx.row_of_token, ctx.seg_start, ctx.seg_len, ctx.slot, out)
+            at = 0
+            for (p0, n), slot in zip(segments, slots):
+                y, s = P.short_conv(bcx[at:at + n], w, bias if use_bias else None, state=state0[slot])
+                tol = dict(rtol=1e-5, atol=1e-5) if out_dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -7)
+                torch.testing.assert_close(out[at:at + n].cpu().float(), y, **tol)
+                torch.testing.assert_close(state[slot].cpu(), s, rtol=1e-6, atol=1e-6)
+                at += n
+            for slot in set(range(8)) - set(slots):          # other requests' state is left alone
+                assert torch.equal(state[slot].cpu(), state0[slot])
+
+
+def test_short_conv_exact_vectors_from_the_reference():
+    # /root/reference/crates/imparo-cpu/src/ops.rs:1207-1254 on the GPU kernel
+    ctx = hand_context([(0, 2)], 16, 4, torch.float32, DEV, fixed_sites={0: (2, 1)})
+    state = ctx.fixed_state(0)
+    state[0] = torch.tensor([[5.0], [7.0]])
+    out = torch.empty(2, 1, device=DEV)
+    ops().short_conv(torch.ones(2, 3, device=DEV), torch.tensor([[1.0, 0.0, 0.0]], device=DEV), None, state,
+                     ctx.row_of_token, ctx.seg_start, ctx.seg_len, ctx.slot, out)
+    assert out.flatten().tolist() == [5.0, 7.0] and state[0].flatten().tolist() == [1.0, 1.0]
+
+
+# ---------------------------------------------------------------- sampling
+@pytest.mark.parametrize("vocab", [7, 200, 1000, 65536, 70001])
+def test_argmax_rows(vocab):
+    x = rnd(6, vocab, seed=vocab)
+    x[1, vocab // 2] = x[1].max() + 1
+    x[1, vocab - 1] = x[1, vocab // 2]               # a tie: the smaller index wins
+    x[2, 0] = float("nan")
+    x[3] = float("nan")                               # all NaN -> 0
+    x[4, :] = -float("inf")
+    x[5, vocab - 1] = 50.0
+    out = torch.empty(6, dtype=torch.int32, device=DEV)
+    ops().argmax_rows(x.to(DEV), out)
+    assert out.cpu().tolist() == [P.argmax_first(r.numpy()) for r in x]
+    assert out[1].item() == vocab // 2 and out[3].item() == 0 and out[5].item() == vocab - 1
+
+
+@pytest.mark.parametrize("vocab", [7, 384, 65536])
+def test_sample_rows(vocab):
+    n = 64
+    logits = rnd(n, vocab, seed=1, scale=2.0)
+    temps = torch.tensor([0.8] * (n - 2) + [0.0, 1.7])
+    g = torch.Generator().manual_seed(2)
+    u = torch.rand(n, generator=g)
+    u[0], u[1] = 0.0, 0.99999994
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    ops().sample_rows(logits.to(DEV), temps.to(DEV), u.to(DEV), out)
+    got = out.cpu().tolist()
+    for r in range(n):
+        if temps[r] <= 0:
+            assert got[r] == P.argmax_first(logits[r].numpy())
+            continue
+        p = torch.softmax(logits[r].double() / temps[r].double(), dim=0)
+        cdf = torch.cumsum(p, 0)
+        target = float(u[r])
+        lo = float(cdf[got[r] - 1]) if got[r] > 0 else 0.0
+        hi = float(cdf[got[r]])
+        # the pick's interval of the CDF holds the target, up to float32 rounding of the sums
+        assert lo - 1e-5 <= target <= hi + 1e-5, (r, got[r], lo, target, hi)
+    # draws follow the distribution: a row repeated with many uniforms
+    row = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5]]).repeat(4000, 1)
+    uu = torch.rand(4000, generator=g)
+    out = torch.empty(4000, dtype=torch.int32, device=DEV)
+    ops().sample_rows(row.to(DEV), torch.full((4000,), 1.0, device=DEV), uu.to(DEV), out)
+    freq = torch.bincount(out.cpu().long(), minlength=5).float() / 4000
+    assert (freq - torch.softmax(row[0], 0)).abs().max() < 0.03

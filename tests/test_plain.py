@@ -1,0 +1,207 @@
+"""Pins the plain implementation by what fixes it beside the reference's text:
+vectors the reference's own tests hold, special cases that reduce to a library
+routine, and invariants. Each is chosen so that a plausible mistake fails it.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_lfm2 as P
+
+
+# ---------------------------------------------------------------- short conv
+def _bcx(b, c, x):
+    return torch.tensor([list(bb) + list(cc) + list(xx) for bb, cc, xx in zip(b, c, x)], dtype=torch.float32)
+
+
+def test_conv_tap_zero_is_the_oldest_value():
+    # /root/reference/crates/imparo-cpu/src/ops.rs:1207-1254: width 1, kernel 3, state [5,7],
+    # b = x = c = 1 for two tokens; tap-0-only -> out [5,7], state' [1,1]; last-tap-only -> [1,1]
+    bcx = _bcx([[1.0]] * 2, [[1.0]] * 2, [[1.0]] * 2)
+    state = torch.tensor([[5.0], [7.0]])
+    y, s = P.short_conv(bcx, torch.tensor([[[1.0, 0.0, 0.0]]]), state=state)
+    assert y.flatten().tolist() == [5.0, 7.0] and s.flatten().tolist() == [1.0, 1.0]
+    y, _ = P.short_conv(bcx, torch.tensor([[[0.0, 0.0, 1.0]]]), state=state)
+    assert y.flatten().tolist() == [1.0, 1.0]
+
+
+def test_conv_reference_native_vectors():
+    # /root/reference/crates/imparo-cuda/native/tests/lfm2_ops_test.cpp:46-62: width 1, kernel 4,
+    # state {11,13,17}, bcx {2,0,3, 2,0,5}, oldest-tap weights {1,0,0,0} -> out {0,0}, state' {17,6,10}
+    oldest = torch.tensor([[[1.0, 0.0, 0.0, 0.0]]])
+    bcx = _bcx([[2.0], [2.0]], [[0.0], [0.0]], [[3.0], [5.0]])
+    y, s = P.short_conv(bcx, oldest, state=torch.tensor([[11.0], [13.0], [17.0]]))
+    assert y.flatten().tolist() == [0.0, 0.0]
+    assert s.flatten().tolist() == [17.0, 6.0, 10.0]
+    # same file: all-ones rows over state {5,7,9} with the oldest tap -> out {5,7}
+    y, _ = P.short_conv(torch.ones(2, 3), oldest, state=torch.tensor([[5.0], [7.0], [9.0]]))
+    assert y.flatten().tolist() == [5.0, 7.0]
+    # lfm2_ops_test.cpp:64-72: history 2, one token {b2, c1, x3} over {5,7} -> {7,6}
+    _, s = P.short_conv(_bcx([[2.0]], [[1.0]], [[3.0]]), torch.tensor([[[0.0, 0.0, 0.0]]]),
+                        state=torch.tensor([[5.0], [7.0]]))
+    assert s.flatten().tolist() == [7.0, 6.0]
+
+
+def test_conv_c_gates_the_output_and_the_state_still_advances():
+    # ops.rs:1258-1285: c = 0, b = 2, x = 3 -> out 0, state holds b*x = 6
+    y, s = P.short_conv(_bcx([[2.0]], [[0.0]], [[3.0]]), torch.tensor([[[1.0, 1.0]]]),
+                        state=torch.tensor([[9.0]]))
+    assert y.item() == 0.0 and s.item() == 6.0
+
+
+def test_conv_batch_equals_one_token_at_a_time():
+    # ops.rs:1161-1203: width 4, kernel 3, 5 tokens; exact binary fractions so equality is exact
+    g = torch.Generator().manual_seed(0)
+    bcx = torch.randint(-8, 8, (5, 12), generator=g).float() / 4
+    w = torch.randint(-8, 8, (4, 1, 3), generator=g).float() / 4
+    y_all, s_all = P.short_conv(bcx, w)
+    state = None
+    ys = []
+    for t in range(5):
+        y, state = P.short_conv(bcx[t:t + 1], w, state=state)
+        ys.append(y)
+    assert torch.equal(torch.cat(ys), y_all) and torch.equal(state, s_all)
+
+
+def test_conv_reduces_to_a_depthwise_conv1d():
+    g = torch.Generator().manual_seed(1)
+    T, E, L = 9, 6, 4
+    bcx = torch.randn(T, 3 * E, generator=g)
+    w = torch.randn(E, 1, L, generator=g)
+    bias = torch.randn(E, generator=g)
+    u = (bcx[:, :E] * bcx[:, 2 * E:]).t().unsqueeze(0)                    # [1, E, T]
+    lib = torch.nn.functional.conv1d(torch.nn.functional.pad(u, (L - 1, 0)), w, bias, groups=E)[0].t()
+    y, _ = P.short_conv(bcx, w, bias)
+    torch.testing.assert_close(y, bcx[:, E:2 * E] * lib, rtol=1e-5, atol=1e-5)
+
+
+# ---------------------------------------------------------------- attention
+def test_attention_is_causal_and_scaled():
+    # /root/reference/crates/imparo-model/src/cpu_support.rs:485-512
+    q = torch.tensor([[[1.0, 0.0]], [[1.0, 0.0]]])
+    k = torch.tensor([[[0.0, 1.0]], [[1.0, 0.0]]])
+    v = torch.tensor([[[1.0, 0.0]], [[0.0, 1.0]]])
+    out = P.attend(q, k, v, [0, 1], 1.0)
+    assert out[0, 0].tolist() == [1.0, 0.0]
+    assert abs(out[1, 0].sum().item() - 1.0) < 1e-6 and out[1, 0, 1] > out[1, 0, 0]
+    # scores 0 and 1 at scale 1: weights 1/(1+e), e/(1+e); scale 0.5 changes them
+    assert abs(out[1, 0, 1].item() - math.e / (1 + math.e)) < 1e-6
+    half = P.attend(q, k, v, [0, 1], 0.5)
+    assert abs(half[1, 0, 1].item() - math.exp(0.5) / (1 + math.exp(0.5))) < 1e-6
+
+
+def test_a_window_of_one_leaves_each_token_alone():
+    # cpu_support.rs:516-535
+    q = torch.tensor([[[1.0, 0.0]], [[1.0, 0.0]]])
+    k = torch.tensor([[[0.0, 1.0]], [[1.0, 0.0]]])
+    v = torch.tensor([[[1.0, 0.0]], [[0.0, 1.0]]])
+    out = P.attend(q, k, v, [0, 1], 1.0, window=1)
+    assert out[0, 0].tolist() == [1.0, 0.0] and out[1, 0].tolist() == [0.0, 1.0]
+
+
+def test_grouped_query_heads_map_contiguously():
+    # cpu_support.rs:538-557: 4 heads, 2 kv heads, v = [10, 20] -> [10, 10, 20, 20]
+    q = torch.ones(1, 4, 1)
+    k = torch.ones(1, 2, 1)
+    v = torch.tensor([[[10.0], [20.0]]])
+    assert P.attend(q, k, v, [0], 1.0).flatten().tolist() == [10.0, 10.0, 20.0, 20.0]
+
+
+def test_attention_reduces_to_the_library_routine():
+    g = torch.Generator().manual_seed(2)
+    T, H, Hk, D = 11, 6, 2, 8
+    q, k, v = torch.randn(T, H, D, generator=g), torch.randn(T, Hk, D, generator=g), torch.randn(T, Hk, D, generator=g)
+    lib = torch.nn.functional.scaled_dot_product_attention(
+        q.transpose(0, 1), k.transpose(0, 1).repeat_interleave(H // Hk, 0),
+        v.transpose(0, 1).repeat_interleave(H // Hk, 0), is_causal=True).transpose(0, 1)
+    torch.testing.assert_close(P.attend(q, k, v, range(T), 1.0 / math.sqrt(D)), lib, rtol=1e-5, atol=1e-5)
+
+
+# ---------------------------------------------------------------- rotation
+def test_rope_position_zero_is_identity_and_pairs_keep_their_norm():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(4, 2, 8, generator=g)
+    assert torch.equal(P.rope_neox(x[:1], [0], 10000.0, 8), x[:1])
+    y = P.rope_neox(x, [3, 17, 100, 4000], 10000.0, 8)
+    torch.testing.assert_close(x[..., :4] ** 2 + x[..., 4:] ** 2, y[..., :4] ** 2 + y[..., 4:] ** 2,
+                               rtol=1e-5, atol=1e-5)
+
+
+def test_rope_pairs_i_with_i_plus_half_and_turns_the_right_way():
+    # one pair (i=0, inv=1): position p turns (1, 0) to (cos p, sin p); an interleaved pairing or a
+    # flipped sign fails this
+    x = torch.zeros(1, 1, 4)
+    x[0, 0, 0] = 1.0
+    y = P.rope_neox(x, [1], 10000.0, 4)
+    assert abs(y[0, 0, 0].item() - math.cos(1.0)) < 1e-6 and abs(y[0, 0, 2].item() - math.sin(1.0)) < 1e-6
+    assert y[0, 0, 1].item() == 0.0 and y[0, 0, 3].item() == 0.0
+    # second pair turns by base^(-2/4) = 0.01 per position
+    x = torch.zeros(1, 1, 4)
+    x[0, 0, 1] = 1.0
+    y = P.rope_neox(x, [50], 10000.0, 4)
+    assert abs(y[0, 0, 1].item() - math.cos(0.5)) < 1e-6 and abs(y[0, 0, 3].item() - math.sin(0.5)) < 1e-6
+
+
+def test_rope_scores_depend_on_distance_only():
+    g = torch.Generator().manual_seed(4)
+    q, k = torch.randn(1, 1, 16, generator=g), torch.randn(1, 1, 16, generator=g)
+    def score(m, n):
+        return (P.rope_neox(q, [m], 10000.0, 16) * P.rope_neox(k, [n], 10000.0, 16)).sum().item()
+    assert abs(score(5, 2) - score(105, 102)) < 1e-4 and abs(score(5, 2) - score(9, 2)) > 1e-3
+
+
+# ---------------------------------------------------------------- the rest
+def test_rms_norm():
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(3, 10, generator=g)
+    w = torch.ones(10)
+    y = P.rms_norm(x, w, 0.0)
+    torch.testing.assert_close((y * y).mean(-1), torch.ones(3), rtol=1e-5, atol=1e-5)      # unit rms
+    torch.testing.assert_close(P.rms_norm(7 * x, w, 0.0), y, rtol=1e-5, atol=1e-5)        # scale free
+    w2 = torch.arange(10).float()
+    torch.testing.assert_close(P.rms_norm(x, w2, 1e-5), x / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-5) * w2)
+    # the weight multiplies: no +1 offset (a zero weight gives zero)
+    assert torch.equal(P.rms_norm(x, torch.zeros(10), 1e-5), torch.zeros(3, 10))
+    # eps is inside the root: a zero row stays zero and finite
+    assert torch.equal(P.rms_norm(torch.zeros(1, 10), w, 1e-5), torch.zeros(1, 10))
+
+
+def test_silu_values_and_gate_side():
+    # lfm2_ops_test.cpp:83-84
+    assert abs(P.silu(torch.tensor(1.0)).item() - 0.7310586) < 1e-6 and P.silu(torch.tensor(0.0)).item() == 0.0
+    torch.testing.assert_close(P.silu(torch.linspace(-5, 5, 11)), torch.nn.functional.silu(torch.linspace(-5, 5, 11)))
+    # SiLU is on the gate (w1): with w3 x = 1 the result is silu(w1 x); swapping the roles changes it
+    n = torch.tensor([[2.0]])
+    w1, w3, w2 = torch.tensor([[1.0]]), torch.tensor([[0.5]]), torch.tensor([[1.0]])
+    assert abs(P.swiglu(n, w1, w3, w2).item() - (2.0 / (1 + math.exp(-2.0))) * 1.0) < 1e-6
+
+
+def test_linear_is_out_by_in():
+    w = torch.tensor([[1.0, 2.0, 3.0], [0.0, 1.0, 0.0]])
+    assert P.linear(torch.tensor([[1.0, 1.0, 1.0]]), w).tolist() == [[6.0, 1.0]]
+
+
+def test_argmax_first_max_and_nan():
+    assert P.argmax_first([1.0, 3.0, 3.0, 2.0]) == 1
+    assert P.argmax_first([float("nan"), 1.0, float("nan")]) == 1
+    assert P.argmax_first([float("nan")] * 3) == 0
+    assert P.argmax_first(np.arange(5.0)) == int(np.argmax(np.arange(5.0)))
+
+
+def test_ff_dim():
+    for ff, mult, want in ((12288, 256, 8192), (10240, 256, 6912), (6656, 256, 4608), (480, 64, 320)):
+        assert P.ff_dim_from_config(dict(block_auto_adjust_ff_dim=True, block_ff_dim=ff, block_multiple_of=mult)) == want
+    assert P.ff_dim_from_config(dict(block_auto_adjust_ff_dim=False, block_ff_dim=192)) == 192
+
+
+def test_whole_model_is_causal_and_one_expert_head_cases(plain_models):
+    """A later token never changes an earlier logit; and the model's greedy
+    continuation is a function of the prefix."""
+    m = plain_models["A"]
+    toks = list(range(3, 23))
+    a = m.logits(toks)
+    b = m.logits(toks[:12] + [200] * 8)
+    torch.testing.assert_close(a[:12], b[:12], rtol=1e-5, atol=1e-6)
+    assert not torch.allclose(a[12:], b[12:], atol=1e-4)
