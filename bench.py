@@ -1,0 +1,189 @@
+#!/usr/bin/env python3
+"""Benchmark: decode tokens per second of the LFM2-1.2B shape on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the whole batch through the engine's own loop:
+step function, sampling kernel, the sampled tokens read back and fed again.
+Default: batch 8, every request's context ending at 4096 tokens, random
+bfloat16 weights (seed 2), synthetic token ids uniform over the vocabulary.
+The JSON line also carries a 2,048-token prefill, the decode step's HBM
+roofline, and decode at batch 1 and 64.
+"""
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
+MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+LFM2_1_2B = dict(
+    architectures=["Lfm2ForCausalLM"], model_type="lfm2", vocab_size=65536, hidden_size=2048,
+    num_hidden_layers=16, num_attention_heads=32, num_key_value_heads=8,
+    layer_types=["full_attention" if i in (2, 5, 8, 10, 12, 14) else "conv" for i in range(16)],
+    block_auto_adjust_ff_dim=True, block_ff_dim=12288, block_multiple_of=256, block_ffn_dim_multiplier=1.0,
+    conv_L_cache=3, conv_bias=False, rope_theta=1000000.0, tie_embedding=True, norm_eps=1e-5,
+    max_position_embeddings=128000,
+)
+
+
+def model_numbers(cfg):
+    """Matrix parameters per token (layers, head) and cache bytes per token, from the configuration."""
+    from imparo_amd.config import Lfm2Config
+    c = Lfm2Config.from_dict(cfg)
+    E, F, D, H, Hk, L = c.hidden_size, c.ff_dim, c.head_dim, c.num_attention_heads, c.num_key_value_heads, c.conv_L_cache
+    n_attn = sum(t != "conv" for t in c.layer_types)
+    n_conv = len(c.layer_types) - n_attn
+    attn = (H + 2 * Hk) * D * E + E * H * D
+    conv = 3 * E * E + E * E
+    ffn = 3 * E * F
+    layer_params = n_attn * (attn + ffn) + n_conv * (conv + ffn)
+    head_params = c.vocab_size * E
+    return dict(cfg=c, layer_params=layer_params, head_params=head_params, n_attn=n_attn, n_conv=n_conv,
+                kv_bytes_per_token=n_attn * 2 * Hk * D * 2, conv_state_bytes=n_conv * (L - 1) * E * 4,
+                attn_flops_per_pair=n_attn * 4 * H * D)
+
+
+def decode_run(engine, sampler, batch, context, steps, warmup, vocab, seed):
+    """Fills `batch` requests up to context - steps - warmup tokens, then times `steps` decode steps."""
+    import torch
+    from imparo_amd.engine import StepEntry
+    g = torch.Generator().manual_seed(seed)
+    start = context - steps - warmup
+    ids = [f"d{i}" for i in range(batch)]
+    last = None
+    for i, rid in enumerate(ids):                      # prompts in 2,048-token portions
+        prompt = torch.randint(0, vocab, (start,), generator=g).tolist()
+        for lo in range(0, start, 2048):
+            hi = min(start, lo + 2048)
+            out = engine.step([StepEntry(rid, prompt[lo:hi], [hi - lo - 1] if hi == start else [])])
+        last = out if last is None else torch.cat([last, out])
+    temps, unis = [0.0] * batch, [0.0] * batch
+    tokens = sampler.pick(last, temps, unis)
+
+    def one_step(tokens):
+        logits = engine.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, tokens)])
+        return sampler.pick(logits, temps, unis)
+
+    for _ in range(warmup):
+        tokens = one_step(tokens)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        tokens = one_step(tokens)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    for rid in ids:
+        engine.release(rid)
+    return dt
+
+
+def prefill_run(engine, tokens, vocab, reps, seed):
+    import torch
+    from imparo_amd.engine import StepEntry
+    g = torch.Generator().manual_seed(seed)
+    best = None
+    for r in range(reps + 1):
+        prompt = torch.randint(0, vocab, (tokens,), generator=g).tolist()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step([StepEntry("p", prompt, [tokens - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        engine.release("p")
+        if r > 0:                                      # the first run sizes the workspace
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from imparo_amd import write_random_model
+    from imparo_amd.engine import Engine
+    from imparo_amd.sampling import Sampler
+
+    cfg = dict(LFM2_1_2B)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers is not None and args.layers < full_layers:
+        cfg["num_hidden_layers"] = args.layers
+        cfg["layer_types"] = cfg["layer_types"][:args.layers]
+    nums = model_numbers(cfg)
+    c = nums["cfg"]
+    tmp = tempfile.mkdtemp(prefix="imparo_bench_")
+    print(f"[bench] writing random weights ({(nums['layer_params'] + nums['head_params']) / 1e9:.2f} B parameters) ...",
+          file=sys.stderr, flush=True)
+    write_random_model(cfg, 2, tmp)
+    biggest = max(args.batch, 1 if args.no_points else 64)
+    engine = Engine(tmp, dtype=args.dtype, max_tokens=biggest * (args.context + 64), page_size=64,
+                    max_requests=biggest)
+    for f in os.listdir(tmp):
+        os.remove(os.path.join(tmp, f))
+    os.rmdir(tmp)
+    sampler = Sampler(engine.device)
+    elem = 2 if args.dtype == "bfloat16" else 4
+    print("[bench] decode ...", file=sys.stderr, flush=True)
+    dt = decode_run(engine, sampler, args.batch, args.context, args.steps, args.warmup, c.vocab_size, 2)
+    ms = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    # bytes one decode step has to read: every weight once, the cache of the live requests
+    mean_ctx = args.context - args.steps / 2
+    step_bytes = ((nums["layer_params"] + nums["head_params"]) * elem
+                  + args.batch * (mean_ctx * nums["kv_bytes_per_token"] * elem / 2 + nums["conv_state_bytes"]))
+    achieved = step_bytes / (dt / args.steps) / 1e9
+    line = {
+        "metric": "decode tok/s (LFM2-1.2B shape, batch 8, context 4096)",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic token ids, random weights (seed 2)",
+        "config": {
+            "model": "LFM2-1.2B shape", "global_batch": args.batch, "seq_len": args.context, "parallelism": "single GPU",
+            "layers": c.num_hidden_layers, "layers_full": full_layers,
+            "attention_layers": nums["n_attn"], "conv_layers": nums["n_conv"],
+            "hidden_size": c.hidden_size, "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads,
+            "head_dim": c.head_dim, "ff_dim": c.ff_dim, "vocab_size": c.vocab_size, "conv_L_cache": c.conv_L_cache,
+            "tie_embedding": c.tie_embedding, "page_size": engine.page_size, "decode_tokens": args.steps + args.warmup,
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_points:
+        print("[bench] prefill of 2,048 tokens ...", file=sys.stderr, flush=True)
+        T = 2048
+        pt = prefill_run(engine, T, c.vocab_size, 3, 3)
+        flops = 2.0 * T * nums["layer_params"] + 2.0 * nums["head_params"] + nums["attn_flops_per_pair"] * T * (T + 1) / 2
+        peak = MFMA_PEAK["bf16" if args.dtype == "bfloat16" else "fp32"]
+        line["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
+                           "frac": round(flops / pt / peak, 4)}
+        points = {}
+        for b in (1, 64):
+            print(f"[bench] decode at batch {b} ...", file=sys.stderr, flush=True)
+            k = max(8, args.steps // 2)
+            d = decode_run(engine, sampler, b, args.context, k, 4, c.vocab_size, 10 + b)
+            points[f"decode_b{b}"] = round(b * k / d, 1)
+        line["points"] = points
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,8 +1,10 @@
 """The device memory behind the cache manager's pages and slots.
 
-Per cache site with a paged spec: a K and a V pool laid out
-[n_pages, kv_heads, page_size, head_dim], so one kv head's rows of a page are
-contiguous. Per site with a fixed spec: [n_slots, *shape] float32.
+Per cache site with a paged spec: a K pool [n_pages, kv_heads, page_size,
+head_dim], so one kv head's rows of a page are contiguous, and a V pool of the
+same layout or, where the matrix-core attention kernels apply (bfloat16, pages
+of at least 16), transposed inside the page: [n_pages, kv_heads, head_dim,
+page_size]. Per site with a fixed spec: [n_slots, *shape] float32.
 """
 from __future__ import annotations
 
@@ -20,13 +22,17 @@ class CacheStorage:
         self.dtype = dtype
         self.device = device
         self.kv: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
+        self.v_transposed: Dict[int, bool] = {}
         self.fixed: Dict[int, torch.Tensor] = {}
         for site, spec in enumerate(manager.site_specs):
             if isinstance(spec, PagedSpec):
                 g = manager.groups[manager.group_of_site[site]]
                 shape = (g.pool.n_pages, spec.kv_heads, manager.page_size, spec.head_dim)
+                vt = ops.mfma_attention_supported(dtype, manager.page_size, spec.head_dim)
+                v_shape = (shape[0], shape[1], shape[3], shape[2]) if vt else shape
+                self.v_transposed[site] = vt
                 self.kv[site] = (torch.zeros(shape, dtype=dtype, device=device),
-                                 torch.zeros(shape, dtype=dtype, device=device))
+                                 torch.zeros(v_shape, dtype=dtype, device=device))
             elif isinstance(spec, FixedSpec):
                 self.fixed[site] = torch.zeros((manager.n_slots,) + tuple(spec.shape),
                                                dtype=torch.float32, device=device)

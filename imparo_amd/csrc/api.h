@@ -38,14 +38,15 @@ int imparo_gemm(const void* x, const void* w, void* y, int dtype, int out_dtype,
 // qkv is float32 [n_tokens, (heads + 2*kv_heads) * head_dim]; q goes to q_out
 // [n_tokens, heads, head_dim], k and v into the paged cache at each token's
 // position: page = table[row_of_token[t] * table_stride + pos / page_size].
-// Cache layout [n_pages, kv_heads, page_size, head_dim]. write_kv 0 skips the cache.
+// Cache layout [n_pages, kv_heads, page_size, head_dim]; with v_transposed the V
+// cache is [n_pages, kv_heads, head_dim, page_size]. write_kv 0 skips the cache.
 int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight, const float* k_weight, float eps,
                               const float* inv_freq, int n_freq,
                               const int32_t* positions, const int32_t* row_of_token,
                               const int32_t* block_table, int table_stride, int page_size,
                               void* q_out, void* k_cache, void* v_cache, int dtype, int write_kv,
                               int n_tokens, int heads, int kv_heads, int head_dim, int n_pages,
-                              imparo_stream stream);
+                              int v_transposed, imparo_stream stream);
 
 // Causal grouped-query attention over the paged cache; one query per (token,
 // head); keys lo..pos with lo = max(0, pos + 1 - window) (window 0: all keys).
@@ -53,7 +54,29 @@ int imparo_attention(const void* q, const void* k_cache, const void* v_cache, vo
                      const int32_t* positions, const int32_t* row_of_token,
                      const int32_t* block_table, int table_stride, int page_size,
                      int n_tokens, int heads, int kv_heads, int head_dim, int n_pages,
-                     float scale, int window, imparo_stream stream);
+                     float scale, int window, int v_transposed, imparo_stream stream);
+
+// Matrix-core attention, bfloat16, V cache transposed, page_size a power of two
+// >= 16, head_dim a multiple of 16 up to 128.
+// Decode: one query token per listed row (rows[i] indexes seg_start); the key
+// range is split in pieces of 256 keys whose partial results go through
+// part_o [n_rows, heads, n_splits, head_dim] and part_ml [n_rows, heads,
+// n_splits, 2]; n_splits >= ceil(longest context / 256).
+int imparo_attention_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
+                            float* part_o, float* part_ml, const int32_t* rows, int n_rows,
+                            const int32_t* seg_start, const int32_t* positions,
+                            const int32_t* block_table, int table_stride, int page_size,
+                            int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
+                            int n_splits, imparo_stream stream);
+
+// Prompt portions: the listed rows' segments in tiles of 64 queries;
+// n_tiles = sum over the rows of ceil(seg_len / 64).
+int imparo_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
+                             const int32_t* rows, int n_rows, int n_tiles,
+                             const int32_t* seg_start, const int32_t* seg_len, const int32_t* positions,
+                             const int32_t* block_table, int table_stride, int page_size,
+                             int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
+                             imparo_stream stream);
 
 // Gated short convolution over each request's segment, continuing from its
 // state slot. bcx float32 [n_tokens, 3*width] = [B | C | x]. state float32

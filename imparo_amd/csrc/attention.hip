@@ -51,7 +51,7 @@ __global__ void k_attention_wave(const T* __restrict__ q, const T* __restrict__ 
                                  T* __restrict__ out, const int32_t* __restrict__ positions,
                                  const int32_t* __restrict__ row_of_token, const int32_t* __restrict__ block_table,
                                  int table_stride, int page_size, int n_tokens, int heads, int kv_heads, int head_dim,
-                                 int n_pages, float scale, int window) {
+                                 int n_pages, float scale, int window, int v_transposed) {
     __shared__ float q_rows[ATT_WAVES][ATT_MAX_HEAD_DIM];
     __shared__ float probs[ATT_WAVES][WAVE];
     __shared__ long long v_off[ATT_WAVES][WAVE];
@@ -87,6 +87,8 @@ __global__ void k_attention_wave(const T* __restrict__ q, const T* __restrict__ 
             if (page >= 0 && page < n_pages) {
                 off = (((long long)page * kv_heads + kvh) * page_size + (p % page_size)) * head_dim;
                 s = dot_row<T>(qr, k_cache + off, head_dim) * scale;
+                if (v_transposed)
+                    off = ((long long)page * kv_heads + kvh) * page_size * head_dim + (p % page_size);
             }
         }
         const float m_new = fmaxf(m, wave_max(s));
@@ -108,7 +110,7 @@ __global__ void k_attention_wave(const T* __restrict__ q, const T* __restrict__ 
 #pragma unroll
             for (int j = 0; j < DPL; ++j) {
                 const int d = lane + j * WAVE;
-                if (d < head_dim) acc[j] += pk * load_f32<T>(vrow, d);
+                if (d < head_dim) acc[j] += pk * load_f32<T>(vrow, v_transposed ? (size_t)d * page_size : (size_t)d);
             }
         }
         wave_lds_sync();
@@ -137,7 +139,7 @@ extern "C" int imparo_attention(const void* q, const void* k_cache, const void* 
                                 const int32_t* positions, const int32_t* row_of_token,
                                 const int32_t* block_table, int table_stride, int page_size,
                                 int n_tokens, int heads, int kv_heads, int head_dim, int n_pages,
-                                float scale, int window, imparo_stream stream) {
+                                float scale, int window, int v_transposed, imparo_stream stream) {
     const int bad = check_attention_args(q, k_cache, v_cache, out, positions, row_of_token, block_table, table_stride,
                                          page_size, n_tokens, heads, kv_heads, head_dim, n_pages, window);
     if (bad) return bad;
@@ -148,11 +150,12 @@ extern "C" int imparo_attention(const void* q, const void* k_cache, const void* 
     if (dtype == IMPARO_F32)
         k_attention_wave<float><<<blocks, ATT_WAVES * WAVE, 0, s>>>(
             (const float*)q, (const float*)k_cache, (const float*)v_cache, (float*)out, positions, row_of_token,
-            block_table, table_stride, page_size, n_tokens, heads, kv_heads, head_dim, n_pages, scale, window);
+            block_table, table_stride, page_size, n_tokens, heads, kv_heads, head_dim, n_pages, scale, window, v_transposed);
     else if (dtype == IMPARO_BF16)
         k_attention_wave<bf16_t><<<blocks, ATT_WAVES * WAVE, 0, s>>>(
             (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, positions, row_of_token,
-            block_table, table_stride, page_size, n_tokens, heads, kv_heads, head_dim, n_pages, scale, window);
+            block_table, table_stride, page_size, n_tokens, heads, kv_heads, head_dim, n_pages, scale, window,
+            v_transposed);
     else
         return IMPARO_BAD_ARGUMENT;
     return launch_status();

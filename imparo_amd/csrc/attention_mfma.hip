@@ -1,0 +1,340 @@
+// Matrix-core attention over the paged bfloat16 cache: a split-KV kernel for
+// single decoded tokens and a tiled kernel for prompt portions.
+//
+// Both are built on one wave-level step over a tile of 16 keys for up to 16
+// queries, arranged so that nothing has to move between lanes:
+//   S^T[key][query] = K . Q^T      A = K rows (8-byte loads), B = Q^T in registers
+//   O^T[dim][query] += V^T . P^T   A = V^T (the cache keeps V transposed inside a
+//                                  page, so 4 consecutive keys of one dimension
+//                                  are one 8-byte load), B = P^T
+// In the 16x16 result layout a lane holds column lane%16 and rows 4*(lane/16)+i:
+// every value a lane holds belongs to query lane%16, and that is also the B
+// operand layout, so the softmax weights feed the second product as they are.
+// Cache layouts: K [page, kv head, slot, dim], V [page, kv head, dim, slot].
+#include "common.h"
+#include "api.h"
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define DEC_SPLIT 256     // keys per decode split, aligned at absolute multiples
+#define MFMA_WAVES 4
+
+template <int ND>
+struct WaveState {
+    f32x4 o[ND];   // O^T rows dt*16 + 4*(lane/16) + i of query lane%16
+    s16x4 q[ND];   // Q^T operand: dims dk*16 + 4*(lane/16) + i of query lane%16
+    float m, l;
+};
+
+struct Paged {
+    const bf16_t* __restrict__ k;
+    const bf16_t* __restrict__ v;
+    const int32_t* __restrict__ table;
+    int page_size, kv_heads, kvh, n_pages;
+};
+
+__device__ __forceinline__ short pack_bf16(float f) { return (short)f32_to_bf16(f); }
+
+// One tile of 16 keys starting at key_base (a multiple of 16). [lo_q, hi_q] is
+// the key range of this lane's query, [lo_all, hi_all] the live keys any query
+// of the wave may read (addresses are clamped into it; values outside it are
+// forced to zero, never multiplied). `full`: every key of the tile is inside
+// every query's range, so no masking is needed.
+template <int ND>
+__device__ __forceinline__ void attn_tile(WaveState<ND>& st, const Paged& kv, int key_base, int lo_q, int hi_q,
+                                          int lo_all, int hi_all, bool full, float scale, int lane) {
+    constexpr int D = ND * 16;
+    const int c = lane & 15, g = lane >> 4;
+    // ---- scores
+    const int key = min(max(key_base + c, lo_all), hi_all);
+    int page = kv.table[key / kv.page_size];
+    page = min(max(page, 0), kv.n_pages - 1);
+    const bf16_t* krow = kv.k + (((size_t)page * kv.kv_heads + kv.kvh) * kv.page_size + (key % kv.page_size)) * D + 4 * g;
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int dk = 0; dk < ND; ++dk) {
+        const s16x4 a = *reinterpret_cast<const s16x4*>(krow + dk * 16);
+        s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, st.q[dk], s, 0, 0, 0);
+    }
+    const int kg = key_base + 4 * g;          // this lane's 4 keys: kg .. kg+3
+    float sv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const bool ok = full || (kg + i >= lo_q && kg + i <= hi_q);
+        sv[i] = ok ? s[i] * scale : -INFINITY;
+    }
+    float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = fmaxf(st.m, mx);
+    const float corr = (st.m == -INFINITY) ? 0.f : __expf(st.m - m_new);
+    s16x4 pb;
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float p = (sv[i] == -INFINITY) ? 0.f : __expf(sv[i] - m_new);
+        const bf16_t r = f32_to_bf16(p);
+        pb[i] = (short)r;
+        psum += bf16_to_f32(r);               // the denominator sums what the product uses
+    }
+    psum += __shfl_xor(psum, 16, WAVE);
+    psum += __shfl_xor(psum, 32, WAVE);
+    st.l = st.l * corr + psum;
+    st.m = m_new;
+    // ---- weighted values
+    const int kgc = min(max(kg, lo_all & ~3), hi_all & ~3);
+    int vpage = kv.table[kgc / kv.page_size];
+    vpage = min(max(vpage, 0), kv.n_pages - 1);
+    const bf16_t* vbase = kv.v + ((size_t)vpage * kv.kv_heads + kv.kvh) * kv.page_size * D + (kgc % kv.page_size);
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) {
+        s16x4 a = *reinterpret_cast<const s16x4*>(vbase + (size_t)(dt * 16 + c) * kv.page_size);
+        if (!full) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (kg + i < lo_all || kg + i > hi_all) a[i] = 0;   // stale or foreign memory: never multiplied
+        }
+        st.o[dt] = st.o[dt] * corr;
+        st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, st.o[dt], 0, 0, 0);
+    }
+}
+
+template <int ND>
+__device__ __forceinline__ void load_q(WaveState<ND>& st, const bf16_t* __restrict__ qrow, bool valid, int lane) {
+    const int g = lane >> 4;
+#pragma unroll
+    for (int dk = 0; dk < ND; ++dk) {
+        st.q[dk] = valid ? *reinterpret_cast<const s16x4*>(qrow + dk * 16 + 4 * g) : s16x4{0, 0, 0, 0};
+        st.o[dk] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    st.m = -INFINITY;
+    st.l = 0.f;
+}
+
+// ---------------------------------------------------------------- decode
+// grid (split, kv head x passes of 16 query heads, decode row). The four waves
+// of a block take the split's key tiles in turn; their partial results meet in
+// LDS and are merged in wave order; one partial (max, sum, O) per split goes to
+// scratch for the merge kernel.
+template <int ND>
+__global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_decode(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    float* __restrict__ part_o, float* __restrict__ part_ml, const int32_t* __restrict__ rows,
+    const int32_t* __restrict__ seg_start, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int n_pages,
+    float scale, int window, int n_splits) {
+    constexpr int D = ND * 16;
+    __shared__ float sm[MFMA_WAVES][16], sl[MFMA_WAVES][16];
+    __shared__ float so[MFMA_WAVES][16][D + 1];
+    const int split = blockIdx.x, ri = blockIdx.z;
+    const int G = heads / kv_heads, passes = (G + 15) / 16;
+    const int kvh = blockIdx.y / passes, pass = blockIdx.y % passes;
+    const int row = rows[ri];
+    const int t = seg_start[row];
+    const int pos = positions[t];
+    const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+    const int k_begin = max(split * DEC_SPLIT, lo & ~15);
+    const int k_end = min((split + 1) * DEC_SPLIT, pos + 1);
+    if (k_begin >= k_end) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 15, g = lane >> 4;
+    const int hq = pass * 16 + c;               // query head inside the group
+    const bool qvalid = hq < G;
+    const int head = kvh * G + min(hq, G - 1);
+    WaveState<ND> st;
+    load_q<ND>(st, q + ((size_t)t * heads + head) * D, qvalid, lane);
+    Paged kv{k_cache, v_cache, block_table + (size_t)row * table_stride, page_size, kv_heads, kvh, n_pages};
+    const int hi_q = qvalid ? pos : -1;
+    for (int kb = k_begin + wave * 16; kb < k_end; kb += MFMA_WAVES * 16) {
+        const bool full = kb >= lo && kb + 15 <= pos;
+        attn_tile<ND>(st, kv, kb, lo, hi_q, lo, pos, full, scale, lane);
+    }
+    if (g == 0) {
+        sm[wave][c] = st.m;
+        sl[wave][c] = st.l;
+    }
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) so[wave][c][dt * 16 + 4 * g + i] = st.o[dt][i];
+    __syncthreads();
+    for (int e = threadIdx.x; e < 16 * D; e += MFMA_WAVES * 64) {
+        const int qc = e / D, d = e - qc * D;
+        if (pass * 16 + qc >= G) continue;
+        float ms = sm[0][qc];
+#pragma unroll
+        for (int w = 1; w < MFMA_WAVES; ++w) ms = fmaxf(ms, sm[w][qc]);
+        float acc = 0.f, ls = 0.f;
+#pragma unroll
+        for (int w = 0; w < MFMA_WAVES; ++w) {
+            const float f = (sm[w][qc] == -INFINITY) ? 0.f : __expf(sm[w][qc] - ms);
+            acc += so[w][qc][d] * f;
+            ls += sl[w][qc] * f;
+        }
+        const size_t slot = ((size_t)ri * heads + kvh * G + pass * 16 + qc) * n_splits + split;
+        part_o[slot * D + d] = acc;
+        if (d == 0) {
+            part_ml[slot * 2] = ms;
+            part_ml[slot * 2 + 1] = ls;
+        }
+    }
+}
+
+// One wave per (decode row, head): merges the splits in order.
+__global__ void k_attn_decode_merge(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                    bf16_t* __restrict__ out, const int32_t* __restrict__ rows,
+                                    const int32_t* __restrict__ seg_start, const int32_t* __restrict__ positions,
+                                    int heads, int head_dim, int n_splits, int window) {
+    const int ri = blockIdx.x / heads, head = blockIdx.x % heads;
+    const int t = seg_start[rows[ri]];
+    const int pos = positions[t];
+    const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+    const int s_lo = (lo & ~15) / DEC_SPLIT, s_hi = pos / DEC_SPLIT;
+    const size_t base = ((size_t)ri * heads + head) * n_splits;
+    float ms = -INFINITY;
+    for (int s = s_lo; s <= s_hi; ++s) ms = fmaxf(ms, part_ml[(base + s) * 2]);
+    float ls = 0.f;
+    for (int s = s_lo; s <= s_hi; ++s) {
+        const float m = part_ml[(base + s) * 2];
+        ls += (m == -INFINITY) ? 0.f : part_ml[(base + s) * 2 + 1] * __expf(m - ms);
+    }
+    const float inv = ls > 0.f ? 1.0f / ls : 0.f;
+    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+        float acc = 0.f;
+        for (int s = s_lo; s <= s_hi; ++s) {
+            const float m = part_ml[(base + s) * 2];
+            if (m != -INFINITY) acc += part_o[(base + s) * head_dim + d] * __expf(m - ms);
+        }
+        out[((size_t)t * heads + head) * head_dim + d] = f32_to_bf16(acc * inv);
+    }
+}
+
+// ---------------------------------------------------------------- prompt portions
+// grid (tile of 64 queries, head). A block's four waves take 16 consecutive
+// queries each and walk the keys from the lowest any of them may read up to
+// the last query's own position.
+template <int ND>
+__global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    bf16_t* __restrict__ out, const int32_t* __restrict__ rows, int n_rows,
+    const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int n_pages,
+    float scale, int window) {
+    constexpr int D = ND * 16;
+    int tile = blockIdx.x, row = -1;
+    for (int i = 0; i < n_rows; ++i) {
+        const int r = rows[i];
+        const int nt = (seg_len[r] + 63) >> 6;
+        if (tile < nt) {
+            row = r;
+            break;
+        }
+        tile -= nt;
+    }
+    if (row < 0) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 15, g = lane >> 4;
+    const int len = seg_len[row];
+    const int q_first = tile * 64 + wave * 16;
+    if (q_first >= len) return;
+    const int head = blockIdx.y;
+    const int kvh = head / (heads / kv_heads);
+    const int t0 = seg_start[row];
+    const int pos0 = positions[t0];
+    const int qi = q_first + c;
+    const bool qvalid = qi < len;
+    const int pos_q = pos0 + qi;
+    const int pos_first = pos0 + q_first;
+    const int pos_last = pos0 + min(len, q_first + 16) - 1;
+    const int lo_q = window > 0 ? max(0, pos_q + 1 - window) : 0;
+    const int hi_q = qvalid ? pos_q : -1;
+    const int lo_all = window > 0 ? max(0, pos_first + 1 - window) : 0;
+    const int lo_max = window > 0 ? max(0, pos_last + 1 - window) : 0;
+    WaveState<ND> st;
+    load_q<ND>(st, q + ((size_t)(t0 + min(qi, len - 1)) * heads + head) * D, qvalid, lane);
+    Paged kv{k_cache, v_cache, block_table + (size_t)row * table_stride, page_size, kv_heads, kvh, n_pages};
+    for (int kb = lo_all & ~15; kb <= pos_last; kb += 16) {
+        const bool full = kb >= lo_max && kb + 15 <= pos_first;
+        attn_tile<ND>(st, kv, kb, lo_q, hi_q, lo_all, pos_last, full, scale, lane);
+    }
+    if (!qvalid) return;
+    const float inv = st.l > 0.f ? 1.0f / st.l : 0.f;
+    bf16_t* dst = out + ((size_t)(t0 + qi) * heads + head) * D + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) {
+        s16x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = pack_bf16(st.o[dt][i] * inv);
+        *reinterpret_cast<s16x4*>(dst + dt * 16) = v;
+    }
+}
+
+// ---------------------------------------------------------------- entry points
+static int check_common(const void* q, const void* k_cache, const void* v_cache, const void* out, const int32_t* rows,
+                        const int32_t* seg_start, const int32_t* positions, const int32_t* block_table,
+                        int table_stride, int page_size, int heads, int kv_heads, int head_dim, int n_pages, int window) {
+    if (!q || !k_cache || !v_cache || !out || !rows || !seg_start || !positions || !block_table)
+        return IMPARO_BAD_ARGUMENT;
+    if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0) return IMPARO_BAD_ARGUMENT;
+    if (head_dim <= 0 || head_dim % 16 != 0 || head_dim > 128) return IMPARO_BAD_ARGUMENT;
+    if (page_size < 16 || (page_size & (page_size - 1)) != 0) return IMPARO_BAD_ARGUMENT;
+    if (table_stride <= 0 || n_pages <= 0 || window < 0) return IMPARO_BAD_ARGUMENT;
+    return IMPARO_OK;
+}
+
+#define DISPATCH_ND(nd, CALL)                                                                                        \
+    switch (nd) {                                                                                                    \
+        case 1: { constexpr int ND = 1; CALL; } break;                                                               \
+        case 2: { constexpr int ND = 2; CALL; } break;                                                               \
+        case 3: { constexpr int ND = 3; CALL; } break;                                                               \
+        case 4: { constexpr int ND = 4; CALL; } break;                                                               \
+        case 5: { constexpr int ND = 5; CALL; } break;                                                               \
+        case 6: { constexpr int ND = 6; CALL; } break;                                                               \
+        case 7: { constexpr int ND = 7; CALL; } break;                                                               \
+        case 8: { constexpr int ND = 8; CALL; } break;                                                               \
+        default: return IMPARO_BAD_ARGUMENT;                                                                         \
+    }
+
+extern "C" int imparo_attention_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                       float* part_o, float* part_ml, const int32_t* rows, int n_rows,
+                                       const int32_t* seg_start, const int32_t* positions,
+                                       const int32_t* block_table, int table_stride, int page_size,
+                                       int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
+                                       int n_splits, imparo_stream stream) {
+    const int bad = check_common(q, k_cache, v_cache, out, rows, seg_start, positions, block_table, table_stride,
+                                 page_size, heads, kv_heads, head_dim, n_pages, window);
+    if (bad) return bad;
+    if (!part_o || !part_ml || n_rows < 0 || n_splits <= 0 || n_splits > 65535) return IMPARO_BAD_ARGUMENT;
+    if (n_rows == 0) return IMPARO_OK;
+    if (n_rows > 65535) return IMPARO_BAD_ARGUMENT;
+    hipStream_t s = (hipStream_t)stream;
+    const int G = heads / kv_heads;
+    dim3 grid(n_splits, kv_heads * ((G + 15) / 16), n_rows);
+    DISPATCH_ND(head_dim / 16, (k_attn_decode<ND><<<grid, MFMA_WAVES * 64, 0, s>>>(
+        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, part_o, part_ml, rows, seg_start, positions,
+        block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, n_splits)));
+    if (launch_status()) return IMPARO_LAUNCH_FAILED;
+    k_attn_decode_merge<<<n_rows * heads, 64, 0, s>>>(part_o, part_ml, (bf16_t*)out, rows, seg_start, positions, heads,
+                                                      head_dim, n_splits, window);
+    return launch_status();
+}
+
+extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                        const int32_t* rows, int n_rows, int n_tiles,
+                                        const int32_t* seg_start, const int32_t* seg_len, const int32_t* positions,
+                                        const int32_t* block_table, int table_stride, int page_size,
+                                        int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
+                                        imparo_stream stream) {
+    const int bad = check_common(q, k_cache, v_cache, out, rows, seg_start, positions, block_table, table_stride,
+                                 page_size, heads, kv_heads, head_dim, n_pages, window);
+    if (bad) return bad;
+    if (!seg_len || n_rows < 0 || n_tiles < 0 || heads > 65535) return IMPARO_BAD_ARGUMENT;
+    if (n_rows == 0 || n_tiles == 0) return IMPARO_OK;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid(n_tiles, heads);
+    DISPATCH_ND(head_dim / 16, (k_attn_prefill<ND><<<grid, MFMA_WAVES * 64, 0, s>>>(
+        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, rows, n_rows, seg_start,
+        seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window)));
+    return launch_status();
+}

@@ -17,7 +17,8 @@ __global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float*
                                      const int32_t* __restrict__ positions, const int32_t* __restrict__ row_of_token,
                                      const int32_t* __restrict__ block_table, int table_stride, int page_size,
                                      T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                     int write_kv, int n_tokens, int heads, int kv_heads, int head_dim, int n_pages) {
+                                     int write_kv, int n_tokens, int heads, int kv_heads, int head_dim, int n_pages,
+                                     int v_transposed) {
     __shared__ float rows[ROPE_WAVES][ROPE_MAX_HEAD_DIM];
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = threadIdx.x / WAVE;
@@ -70,6 +71,12 @@ __global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float*
     const int pos = positions[t];
     const int page = block_table[(size_t)row_of_token[t] * table_stride + pos / page_size];
     if (page < 0 || page >= n_pages) return;   // never write outside the pool
+    if (is_v && v_transposed) {
+        // [page, kv head, dim, slot]: the keys of one dimension lie side by side
+        T* dst = v_cache + ((size_t)page * kv_heads + kvh) * page_size * head_dim + (pos % page_size);
+        for (int i = lane; i < head_dim; i += WAVE) store_f32<T>(dst, (size_t)i * page_size, row[i]);
+        return;
+    }
     T* cache = is_v ? v_cache : k_cache;
     T* dst = cache + (((size_t)page * kv_heads + kvh) * page_size + (pos % page_size)) * head_dim;
     for (int i = lane; i < head_dim; i += WAVE) store_f32<T>(dst, i, row[i]);
@@ -81,7 +88,7 @@ extern "C" int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight
                                          const int32_t* block_table, int table_stride, int page_size,
                                          void* q_out, void* k_cache, void* v_cache, int dtype, int write_kv,
                                          int n_tokens, int heads, int kv_heads, int head_dim, int n_pages,
-                                         imparo_stream stream) {
+                                         int v_transposed, imparo_stream stream) {
     if (!qkv || !positions || !q_out) return IMPARO_BAD_ARGUMENT;
     if (write_kv && (!row_of_token || !block_table || !k_cache || !v_cache)) return IMPARO_BAD_ARGUMENT;
     if (n_tokens < 0 || heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim > ROPE_MAX_HEAD_DIM)
@@ -97,12 +104,12 @@ extern "C" int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight
         k_qk_norm_rope_store<float><<<blocks, ROPE_WAVES * WAVE, 0, s>>>(
             qkv, q_weight, k_weight, eps, inv_freq, n_freq, positions, row_of_token, block_table, table_stride,
             page_size, (float*)q_out, (float*)k_cache, (float*)v_cache, write_kv, n_tokens, heads, kv_heads,
-            head_dim, n_pages);
+            head_dim, n_pages, v_transposed);
     else if (dtype == IMPARO_BF16)
         k_qk_norm_rope_store<bf16_t><<<blocks, ROPE_WAVES * WAVE, 0, s>>>(
             qkv, q_weight, k_weight, eps, inv_freq, n_freq, positions, row_of_token, block_table, table_stride,
             page_size, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, write_kv, n_tokens, heads, kv_heads,
-            head_dim, n_pages);
+            head_dim, n_pages, v_transposed);
     else
         return IMPARO_BAD_ARGUMENT;
     return launch_status();

@@ -174,12 +174,13 @@ class Engine:
         lengths = [self.cache.length[e.request] for e in entries]
         P = max(1, max(len(self.cache.table(g, e.request)) for e in entries for g in range(G)) if G else 1)
         W = sum(len(e.want) for e in entries)
-        # layout: tokens | positions | row_of_token | seg_start | seg_len | slot | want | tables[G][R][P]
-        total = 3 * T + 3 * R + W + G * R * P
+        # layout: tokens | positions | row_of_token | seg_start | seg_len | slot | row lists | want | tables[G][R][P]
+        total = 3 * T + 4 * R + W + G * R * P
         a = np.empty(total, dtype=np.int32)
         o_tok, o_pos, o_row = 0, T, 2 * T
         o_start, o_len, o_slot = 3 * T, 3 * T + R, 3 * T + 2 * R
-        o_want = 3 * T + 3 * R
+        o_lists = 3 * T + 3 * R
+        o_want = 3 * T + 4 * R
         o_tab = o_want + W
         t = 0
         w = 0
@@ -195,6 +196,10 @@ class Engine:
                 a[o_want + w] = t + int(wi)
                 w += 1
             t += n
+        # rows with one token first, rows with a portion after them
+        dec = [r for r, e in enumerate(entries) if len(e.tokens) == 1]
+        pre = [r for r, e in enumerate(entries) if len(e.tokens) > 1]
+        a[o_lists:o_lists + R] = np.asarray(dec + pre, dtype=np.int32)
         tables = a[o_tab:].reshape(G, R, P) if G else None
         if G:
             tables.fill(-1)
@@ -212,6 +217,9 @@ class Engine:
             workspace=self.workspace, storage=self.storage, group_of_site=self.cache.group_of_site,
             max_seg_len=max(len(e.tokens) for e in entries),
             max_context=max(lengths[r] + len(e.tokens) for r, e in enumerate(entries)),
+            decode_rows=dev[o_lists:o_lists + len(dec)], n_decode_rows=len(dec),
+            prefill_rows=dev[o_lists + len(dec):o_lists + R], n_prefill_rows=len(pre),
+            n_prefill_tiles=sum((len(entries[r].tokens) + 63) // 64 for r in pre),
         )
         want_rows = dev[o_want:o_want + W] if W else None
         return ctx, dev[o_tok:o_tok + T], want_rows

@@ -124,7 +124,7 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_we
                        eps: float, inv_freq: Optional[torch.Tensor], positions: torch.Tensor,
                        row_of_token: torch.Tensor, block_table: Optional[torch.Tensor], page_size: int,
                        q_out: torch.Tensor, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                       heads: int, kv_heads: int, head_dim: int) -> torch.Tensor:
+                       heads: int, kv_heads: int, head_dim: int, v_transposed: bool = False) -> torch.Tensor:
     n = qkv.shape[0]
     units = heads + 2 * kv_heads
     write_kv = k_cache is not None
@@ -133,9 +133,9 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_we
     table_stride = 0
     if write_kv:
         n_pages = k_cache.shape[0]
-        want = (n_pages, kv_heads, page_size, head_dim)
-        _dev(k_cache, "k cache", q_out.dtype, want)
-        _dev(v_cache, "v cache", q_out.dtype, want)
+        _dev(k_cache, "k cache", q_out.dtype, (n_pages, kv_heads, page_size, head_dim))
+        _dev(v_cache, "v cache", q_out.dtype, (n_pages, kv_heads, head_dim, page_size) if v_transposed
+             else (n_pages, kv_heads, page_size, head_dim))
         if block_table is None or block_table.dim() != 2:
             raise KernelArgumentError("qk_norm_rope_store: a [rows, pages] block table is needed to write the cache")
         table_stride = block_table.shape[1]
@@ -147,14 +147,16 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_we
         _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
         _dev(block_table, "block table", torch.int32), table_stride, page_size,
         _dev(q_out, "q out", None, (n, heads, head_dim)), _dev(k_cache, "k cache"), _dev(v_cache, "v cache"),
-        _code(q_out, "q out"), int(write_kv), n, heads, kv_heads, head_dim, n_pages, _stream()),
+        _code(q_out, "q out"), int(write_kv), n, heads, kv_heads, head_dim, n_pages, int(v_transposed), _stream()),
         "qk_norm_rope_store")
     return q_out
 
 
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
               positions: torch.Tensor, row_of_token: torch.Tensor, block_table: torch.Tensor,
-              scale: float, window: Optional[int]) -> torch.Tensor:
+              scale: float, window: Optional[int], v_transposed: bool = False) -> torch.Tensor:
+    """The general kernel: any page size, head sizes in steps of 16 up to 512,
+    float32 or bfloat16; one wave per (token, head)."""
     n, heads, head_dim = q.shape
     n_pages, kv_heads, page_size, hd = k_cache.shape
     if hd != head_dim:
@@ -164,11 +166,68 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out
     if heads % kv_heads != 0:
         raise KernelArgumentError(f"attention: {heads} heads cannot share {kv_heads} kv heads evenly")
     _check(library().imparo_attention(
-        _dev(q, "q"), _dev(k_cache, "k cache", q.dtype), _dev(v_cache, "v cache", q.dtype, k_cache.shape),
+        _dev(q, "q"), _dev(k_cache, "k cache", q.dtype),
+        _dev(v_cache, "v cache", q.dtype, (n_pages, kv_heads, head_dim, page_size) if v_transposed else k_cache.shape),
         _dev(out, "attention out", q.dtype, (n, heads * head_dim)), _code(q, "q"),
         _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
         _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size,
-        n, heads, kv_heads, head_dim, n_pages, float(scale), int(window or 0), _stream()), "attention")
+        n, heads, kv_heads, head_dim, n_pages, float(scale), int(window or 0), int(v_transposed), _stream()),
+        "attention")
+    return out
+
+
+DECODE_SPLIT = 256
+
+
+def mfma_attention_supported(dtype: torch.dtype, page_size: int, head_dim: int) -> bool:
+    return (dtype == torch.bfloat16 and page_size >= 16 and page_size & (page_size - 1) == 0
+            and head_dim % 16 == 0 and head_dim <= 128)
+
+
+def _check_mfma(q, k_cache, v_cache, out):
+    n, heads, head_dim = q.shape
+    n_pages, kv_heads, page_size, hd = k_cache.shape
+    if not mfma_attention_supported(q.dtype, page_size, head_dim) or hd != head_dim:
+        raise KernelArgumentError(f"the matrix-core attention kernels take bfloat16, pages of a power of two >= 16 and "
+                                  f"head sizes in steps of 16 up to 128; got {q.dtype}, pages of {page_size}, "
+                                  f"head size {head_dim}")
+    if heads % kv_heads != 0:
+        raise KernelArgumentError(f"attention: {heads} heads cannot share {kv_heads} kv heads evenly")
+    _dev(k_cache, "k cache", torch.bfloat16)
+    _dev(v_cache, "v cache", torch.bfloat16, (n_pages, kv_heads, head_dim, page_size))
+    _dev(out, "attention out", torch.bfloat16, (n, heads * head_dim))
+    return n, heads, head_dim, n_pages, kv_heads, page_size
+
+
+def attention_decode(q, k_cache, v_cache, out, part_o, part_ml, rows, n_rows: int, seg_start, positions,
+                     block_table, scale: float, window: Optional[int], max_context: int) -> torch.Tensor:
+    """Split-KV attention for rows that bring one token each. `rows` lists
+    them (indices into seg_start); `max_context` bounds every row's position + 1."""
+    n, heads, head_dim, n_pages, kv_heads, page_size = _check_mfma(q, k_cache, v_cache, out)
+    n_splits = max(1, (max_context + DECODE_SPLIT - 1) // DECODE_SPLIT)
+    if part_o.numel() < n_rows * heads * n_splits * head_dim or part_ml.numel() < n_rows * heads * n_splits * 2:
+        raise KernelArgumentError("attention_decode: the scratch for partial results is too small")
+    _check(library().imparo_attention_decode(
+        _dev(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
+        _dev(part_o, "partial outputs", torch.float32), _dev(part_ml, "partial sums", torch.float32),
+        _dev(rows, "decode rows", torch.int32), n_rows, _dev(seg_start, "seg_start", torch.int32),
+        _dev(positions, "positions", torch.int32, (n,)), _dev(block_table, "block table", torch.int32),
+        block_table.shape[1], page_size, heads, kv_heads, head_dim, n_pages, float(scale), int(window or 0),
+        n_splits, _stream()), "attention_decode")
+    return out
+
+
+def attention_prefill(q, k_cache, v_cache, out, rows, n_rows: int, n_tiles: int, seg_start, seg_len, positions,
+                      block_table, scale: float, window: Optional[int]) -> torch.Tensor:
+    """Tiled attention for rows that bring a portion of a prompt. `n_tiles` is
+    the sum over the listed rows of ceil(seg_len / 64)."""
+    n, heads, head_dim, n_pages, kv_heads, page_size = _check_mfma(q, k_cache, v_cache, out)
+    _check(library().imparo_attention_prefill(
+        _dev(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
+        _dev(rows, "prefill rows", torch.int32), n_rows, n_tiles, _dev(seg_start, "seg_start", torch.int32),
+        _dev(seg_len, "seg_len", torch.int32), _dev(positions, "positions", torch.int32, (n,)),
+        _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size, heads, kv_heads, head_dim,
+        n_pages, float(scale), int(window or 0), _stream()), "attention_prefill")
     return out
 
 

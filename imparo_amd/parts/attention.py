@@ -87,14 +87,30 @@ class Attention:
         T = h.shape[0]
         qkv = self.qkv(ctx, h, torch.float32, "qkv")
         k_cache, v_cache, table = ctx.kv(site)
+        vt = ctx.v_transposed(site)
         q = ctx.workspace.get("q", (T, self.heads, self.head_dim), ctx.dtype)
         ops.qk_norm_rope_store(qkv, self.q_norm, self.k_norm, self.norm_eps, self.position.inv_freq,
                                ctx.positions, ctx.row_of_token, table if owns_cache else None, ctx.page_size,
                                q, k_cache if owns_cache else None, v_cache if owns_cache else None,
-                               self.heads, self.kv_heads, self.head_dim)
-        attn_dtype = ctx.dtype
-        o = ctx.workspace.get("attn_out", (T, self.heads * self.head_dim), attn_dtype)
-        ops.attention(q, k_cache, v_cache, o, ctx.positions, ctx.row_of_token, table, self.scale, self.window)
+                               self.heads, self.kv_heads, self.head_dim, v_transposed=vt)
+        o = ctx.workspace.get("attn_out", (T, self.heads * self.head_dim), ctx.dtype)
+        if vt and ctx.decode_rows is not None:
+            # matrix-core kernels: single tokens split over their keys, portions tiled over their queries
+            if ctx.n_decode_rows:
+                n_splits = (ctx.max_context + ops.DECODE_SPLIT - 1) // ops.DECODE_SPLIT
+                part_o = ctx.workspace.get("attn_part_o", (ctx.n_decode_rows * self.heads * n_splits * self.head_dim,),
+                                           torch.float32)
+                part_ml = ctx.workspace.get("attn_part_ml", (ctx.n_decode_rows * self.heads * n_splits * 2,),
+                                            torch.float32)
+                ops.attention_decode(q, k_cache, v_cache, o, part_o, part_ml, ctx.decode_rows, ctx.n_decode_rows,
+                                     ctx.seg_start, ctx.positions, table, self.scale, self.window, ctx.max_context)
+            if ctx.n_prefill_rows:
+                ops.attention_prefill(q, k_cache, v_cache, o, ctx.prefill_rows, ctx.n_prefill_rows,
+                                      ctx.n_prefill_tiles, ctx.seg_start, ctx.seg_len, ctx.positions, table,
+                                      self.scale, self.window)
+        else:
+            ops.attention(q, k_cache, v_cache, o, ctx.positions, ctx.row_of_token, table, self.scale, self.window,
+                          v_transposed=vt)
         if o.dtype != self.out.in_dtype:
             raise ValueError("the output projection's weight dtype differs from the attention output's")
         return self.out(ctx, o, torch.float32, "mixer_out")

@@ -62,10 +62,19 @@ class StepContext:
     group_of_site: Dict[int, int]
     max_seg_len: int = 1                # host copy: longest segment of the batch
     max_context: int = 0                # host copy: longest context after this step
+    # rows that bring one token / more than one, as index lists into seg_start
+    decode_rows: Optional[torch.Tensor] = None
+    n_decode_rows: int = 0
+    prefill_rows: Optional[torch.Tensor] = None
+    n_prefill_rows: int = 0
+    n_prefill_tiles: int = 0            # sum over prefill rows of ceil(seg_len / 64)
 
     def kv(self, site: int):
         k, v = self.storage.kv[site]
         return k, v, self.block_tables[self.group_of_site[site]]
+
+    def v_transposed(self, site: int) -> bool:
+        return bool(getattr(self.storage, "v_transposed", {}).get(site, False))
 
     def fixed_state(self, site: int) -> torch.Tensor:
         return self.storage.fixed[site]

@@ -44,7 +44,8 @@ def step_all(engine, rid, tokens, cuts: Sequence[int]) -> torch.Tensor:
 
 def hand_context(segments: Sequence[Tuple[int, int]], page_size: int, n_pages: int, dtype, device,
                  kv_sites: Dict[int, Tuple[int, int]] = None, fixed_sites: Dict[int, Tuple[int, ...]] = None,
-                 n_slots: int = 8, tables: List[List[int]] = None, slots: List[int] = None):
+                 n_slots: int = 8, tables: List[List[int]] = None, slots: List[int] = None,
+                 v_transposed: bool = False):
     """A StepContext for rows given as (start position, number of tokens).
     kv_sites: site -> (kv_heads, head_dim); fixed_sites: site -> state shape.
     Pages are handed out in order unless `tables` gives them."""
@@ -53,10 +54,12 @@ def hand_context(segments: Sequence[Tuple[int, int]], page_size: int, n_pages: i
     class Storage:
         pass
     st = Storage()
-    st.kv, st.fixed = {}, {}
+    st.kv, st.fixed, st.v_transposed = {}, {}, {}
     for site, (hk, d) in (kv_sites or {}).items():
+        v_shape = (n_pages, hk, d, page_size) if v_transposed else (n_pages, hk, page_size, d)
         st.kv[site] = (torch.zeros(n_pages, hk, page_size, d, dtype=dtype, device=device),
-                       torch.zeros(n_pages, hk, page_size, d, dtype=dtype, device=device))
+                       torch.zeros(v_shape, dtype=dtype, device=device))
+        st.v_transposed[site] = v_transposed
     for site, shape in (fixed_sites or {}).items():
         st.fixed[site] = torch.zeros((n_slots,) + tuple(shape), dtype=torch.float32, device=device)
     R = len(segments)
@@ -86,4 +89,10 @@ def hand_context(segments: Sequence[Tuple[int, int]], page_size: int, n_pages: i
         block_tables={0: i32(tab)}, page_size=page_size, dtype=dtype, workspace=Workspace(device),
         storage=st, group_of_site={s: 0 for s in (kv_sites or {})},
         max_seg_len=max(length), max_context=max(p0 + n for p0, n in segments))
+    dec = [r for r, n in enumerate(length) if n == 1]
+    pre = [r for r, n in enumerate(length) if n > 1]
+    lists = i32(dec + pre)
+    ctx.decode_rows, ctx.n_decode_rows = lists[:len(dec)], len(dec)
+    ctx.prefill_rows, ctx.n_prefill_rows = lists[len(dec):], len(pre)
+    ctx.n_prefill_tiles = sum((length[r] + 63) // 64 for r in pre)
     return ctx

@@ -104,13 +104,14 @@ def test_embed_gather_and_silu_mul():
 
 # ---------------------------------------------------------------- norm + rotation + cache write
 @pytest.mark.parametrize("H,Hk,D,rot", [(4, 2, 16, 16), (3, 1, 48, 48), (6, 3, 64, 32), (2, 2, 80, 80), (5, 1, 128, 0)])
-@pytest.mark.parametrize("page_size", [4, 16])
-def test_qk_norm_rope_store(H, Hk, D, rot, page_size):
+@pytest.mark.parametrize("page_size,vt", [(4, False), (16, False), (16, True)])
+def test_qk_norm_rope_store(H, Hk, D, rot, page_size, vt):
     segments = [(0, 5), (37, 1), (9, 3)]
     tables = [[3, 1], list(range(4, 4 + 40 // page_size + 1)), [0, 2, 14][: (12 + page_size - 1) // page_size]]
     n_pages = 16
     for dtype in (torch.float32, torch.bfloat16):
-        ctx = hand_context(segments, page_size, n_pages, dtype, DEV, kv_sites={0: (Hk, D)}, tables=tables)
+        ctx = hand_context(segments, page_size, n_pages, dtype, DEV, kv_sites={0: (Hk, D)}, tables=tables,
+                           v_transposed=vt)
         T = ctx.n_tokens
         qkv = rnd(T, (H + 2 * Hk) * D, seed=D)
         qw, kw = 1 + 0.1 * rnd(D, seed=1), 1 + 0.1 * rnd(D, seed=2)
@@ -122,7 +123,9 @@ def test_qk_norm_rope_store(H, Hk, D, rot, page_size):
         k_cache, v_cache, table = ctx.kv(0)
         q_out = torch.empty(T, H, D, dtype=dtype, device=DEV)
         ops().qk_norm_rope_store(qkv.to(DEV), qw.to(DEV), kw.to(DEV), 1e-5, inv, ctx.positions, ctx.row_of_token,
-                                 table, page_size, q_out, k_cache, v_cache, H, Hk, D)
+                                 table, page_size, q_out, k_cache, v_cache, H, Hk, D, v_transposed=vt)
+        if vt:
+            v_cache = v_cache.transpose(2, 3)           # viewed [page, kv head, slot, dim] again
         positions = ctx.positions.cpu().tolist()
         q = qkv[:, :H * D].reshape(T, H, D)
         k = qkv[:, H * D:(H + Hk) * D].reshape(T, Hk, D)
@@ -146,11 +149,12 @@ def test_qk_norm_rope_store(H, Hk, D, rot, page_size):
 
 
 # ---------------------------------------------------------------- attention
-def _attention_case(H, Hk, D, page_size, window, dtype, sharpen=None, seed=0):
+def _attention_case(H, Hk, D, page_size, window, dtype, sharpen=None, seed=0, kernel="wave", v_transposed=None,
+                    ctx_lens=(70, 1, 200, 33), q_lens=(5, 1, 1, 33)):
     """Rows at different depths of their contexts; the cache is filled by hand
     from whole-sequence k, v; the reference attends over the whole sequences."""
-    ctx_lens = [70, 1, 200, 33]
-    q_lens = [5, 1, 1, 33]                      # the last q_len positions of each context are queried
+    # the last q_len positions of each context are queried
+    vt = (kernel == "mfma") if v_transposed is None else v_transposed
     n_pages = sum((c + page_size - 1) // page_size for c in ctx_lens) + 3
     perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(seed)).tolist()
     tables, nxt = [], 0
@@ -159,7 +163,8 @@ def _attention_case(H, Hk, D, page_size, window, dtype, sharpen=None, seed=0):
         tables.append(perm[nxt:nxt + k])
         nxt += k
     segments = [(c - ql, ql) for c, ql in zip(ctx_lens, q_lens)]
-    ctx = hand_context(segments, page_size, n_pages, dtype, DEV, kv_sites={0: (Hk, D)}, tables=tables)
+    ctx = hand_context(segments, page_size, n_pages, dtype, DEV, kv_sites={0: (Hk, D)}, tables=tables,
+                       v_transposed=vt)
     k_cache, v_cache, table = ctx.kv(0)
     k_cache.fill_(float("nan"))                # a key read from outside the context poisons the output
     v_cache.fill_(float("nan"))
@@ -176,13 +181,27 @@ def _attention_case(H, Hk, D, page_size, window, dtype, sharpen=None, seed=0):
         for p in range(c):
             page = tables[r][p // page_size]
             k_cache[page, :, p % page_size] = k[p].to(dtype).to(DEV)
-            v_cache[page, :, p % page_size] = v[p].to(dtype).to(DEV)
+            if vt:
+                v_cache[page, :, :, p % page_size] = v[p].to(dtype).to(DEV)
+            else:
+                v_cache[page, :, p % page_size] = v[p].to(dtype).to(DEV)
         ref = P.attend(q, k, v, range(c), 1.0 / math.sqrt(D), window)
         qs.append(q[c - ql:])
         refs.append(ref[c - ql:])
     q_all = torch.cat(qs).to(dtype).to(DEV)
-    out = torch.empty(ctx.n_tokens, H * D, dtype=dtype, device=DEV)
-    ops().attention(q_all, k_cache, v_cache, out, ctx.positions, ctx.row_of_token, table, 1.0 / math.sqrt(D), window)
+    out = torch.full((ctx.n_tokens, H * D), float("nan"), dtype=dtype, device=DEV)
+    scale = 1.0 / math.sqrt(D)
+    if kernel == "wave":
+        ops().attention(q_all, k_cache, v_cache, out, ctx.positions, ctx.row_of_token, table, scale, window,
+                        v_transposed=vt)
+    else:
+        n_splits = (ctx.max_context + 255) // 256
+        part_o = torch.full((ctx.n_decode_rows * H * n_splits * D,), float("nan"), device=DEV)
+        part_ml = torch.full((ctx.n_decode_rows * H * n_splits * 2,), float("nan"), device=DEV)
+        ops().attention_decode(q_all, k_cache, v_cache, out, part_o, part_ml, ctx.decode_rows, ctx.n_decode_rows,
+                               ctx.seg_start, ctx.positions, table, scale, window, ctx.max_context)
+        ops().attention_prefill(q_all, k_cache, v_cache, out, ctx.prefill_rows, ctx.n_prefill_rows,
+                                ctx.n_prefill_tiles, ctx.seg_start, ctx.seg_len, ctx.positions, table, scale, window)
     return out.cpu().float().reshape(-1, H, D), torch.cat(refs)
 
 
@@ -195,17 +214,52 @@ def test_attention(H, Hk, D, page_size, window):
     torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)      # one rounding of the output, P in float32
 
 
+@pytest.mark.parametrize("H,Hk,D", [(1, 1, 16), (6, 2, 48), (5, 5, 64), (8, 1, 128), (4, 2, 80), (40, 2, 32)])
+@pytest.mark.parametrize("page_size,window", [(16, None), (64, None), (32, 19), (16, 64), (16, 1), (128, 300)])
+def test_matrix_core_attention(H, Hk, D, page_size, window):
+    """The split-KV decode kernel and the tiled prefill kernel: contexts that
+    span several splits of 256 keys and several tiles of 64 queries."""
+    got, ref = _attention_case(H, Hk, D, page_size, window, torch.bfloat16, kernel="mfma",
+                               ctx_lens=(70, 1, 700, 33, 300, 513, 256), q_lens=(5, 1, 1, 33, 150, 1, 1))
+    # attention weights are rounded to bfloat16 before the second product: 2^-9 relative each
+    torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)
+    # and the general kernel reads the transposed layout too
+    got, ref = _attention_case(H, Hk, D, page_size, window, torch.bfloat16, kernel="wave", v_transposed=True)
+    torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)
+
+
+def test_matrix_core_attention_refuses_other_sizes():
+    from imparo_amd.kernels import KernelArgumentError
+    assert not ops().mfma_attention_supported(torch.bfloat16, 8, 64)
+    assert not ops().mfma_attention_supported(torch.float32, 16, 64)
+    assert not ops().mfma_attention_supported(torch.bfloat16, 16, 144)
+    assert ops().mfma_attention_supported(torch.bfloat16, 64, 112)
+    q = torch.zeros(1, 2, 144, dtype=torch.bfloat16, device=DEV)
+    kc = torch.zeros(2, 1, 16, 144, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros(2, 1, 144, 16, dtype=torch.bfloat16, device=DEV)
+    i = torch.zeros(1, dtype=torch.int32, device=DEV)
+    with pytest.raises(KernelArgumentError, match="head sizes"):
+        ops().attention_prefill(q, kc, vc, torch.zeros(1, 288, dtype=torch.bfloat16, device=DEV), i, 1, 1, i, i, i,
+                                torch.zeros(1, 1, dtype=torch.int32, device=DEV), 1.0, None)
+
+
+@pytest.mark.parametrize("kernel", ["wave", "mfma"])
 @pytest.mark.parametrize("where", ["first", "page_edge", "middle"])
-def test_attention_finds_one_far_key_among_hundreds(where):
+def test_attention_finds_one_far_key_among_hundreds(where, kernel):
     pick = {"first": lambda c: 0, "page_edge": lambda c: (c // 2 // 16) * 16, "middle": lambda c: c // 3}[where]
     for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 2 ** -6)):
-        got, ref = _attention_case(4, 2, 64, 16, None, dtype, sharpen=pick)
+        if kernel == "mfma" and dtype == torch.float32:
+            continue
+        got, ref = _attention_case(4, 2, 64, 16, None, dtype, sharpen=pick, kernel=kernel)
         torch.testing.assert_close(got, ref, rtol=tol, atol=tol)
         # the test means something: with the far key the last query's output is that key's value
     # the last row's query sits at 199 and its far key at 66: a window of 133 starts at 67 and
     # leaves it out, one of 134 starts at 66 and takes it in; the edge decides the output
     for window, dtype in ((133, torch.float32), (134, torch.float32), (133, torch.bfloat16), (134, torch.bfloat16)):
-        got, ref = _attention_case(2, 1, 32, 8, window, dtype, sharpen=lambda c: c // 3)
+        if kernel == "mfma" and dtype == torch.float32:
+            continue
+        got, ref = _attention_case(2, 1, 32, 16 if kernel == "mfma" else 8, window, dtype, sharpen=lambda c: c // 3,
+                                   kernel=kernel)
         torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)
 
 
