@@ -29,9 +29,12 @@ int imparo_silu_mul(const void* gu, int in_dtype, void* out, int out_dtype, int 
 // y = x (+ bias): adds a float32 bias [n] to every row of a float32 [m, n] in place.
 int imparo_add_bias(float* y, const float* bias, int m, int n, imparo_stream stream);
 
-// Y[m, n] = X[m, k] . W[n, k]^T, float32 accumulate. X and W share `dtype`.
-int imparo_gemm(const void* x, const void* w, void* y, int dtype, int out_dtype,
-                int m, int n, int k, imparo_stream stream);
+// Y[m, n] = X[m, k] . W[n, k]^T (+ bias[n], float32, may be null), float32
+// accumulate. X and W share `dtype`. epilogue 0: Y is [m, n]. epilogue 1
+// (SwiGLU): W's rows alternate gate, up; Y is [m, n/2] with
+// Y[m, j] = silu(y[m, 2j]) * y[m, 2j+1].
+int imparo_gemm(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
+                int m, int n, int k, int epilogue, imparo_stream stream);
 
 // Per (token, head): RMS norm over the head (weight null: none), NeoX rotation
 // with angles pos * inv_freq[i] over the first 2*n_freq dims (n_freq 0: none).
@@ -87,6 +90,12 @@ int imparo_short_conv(const float* bcx, const float* weight, const float* bias, 
                       const int32_t* row_of_token, const int32_t* seg_start, const int32_t* slot,
                       void* out, int out_dtype, int n_tokens, int width, int taps, int n_slots, int n_rows,
                       imparo_stream stream);
+
+// The same for a batch in which every request brings exactly one token, output
+// and state update in one launch: n_tokens == n_rows, token r belongs to row r.
+int imparo_short_conv_decode(const float* bcx, const float* weight, const float* bias, float* state,
+                             const int32_t* slot, void* out, int out_dtype, int n_rows, int width, int taps,
+                             int n_slots, imparo_stream stream);
 
 // state' = the last taps-1 rows of (state ++ B*x) for every request; runs after
 // imparo_short_conv on the same stream.

@@ -177,7 +177,7 @@ __global__ void k_short_conv(const float* __restrict__ bcx, const float* __restr
             const size_t row = (size_t)(t - (history - k)) * 3 * width;
             v = bcx[row + ch] * bcx[row + 2 * width + ch];
         }
-        acc += weight[(size_t)ch * taps + k] * v;
+        acc = fmaf(weight[(size_t)ch * taps + k], v, acc);
     }
     if (bias) acc += bias[ch];
     const float c = bcx[(size_t)t * 3 * width + width + ch];
@@ -201,6 +201,52 @@ extern "C" int imparo_short_conv(const float* bcx, const float* weight, const fl
     else if (out_dtype == IMPARO_BF16)
         k_short_conv<bf16_t><<<grid, threads, 0, s>>>(bcx, weight, bias, state, row_of_token, seg_start, slot,
                                                        (bf16_t*)out, n_tokens, width, taps);
+    else
+        return IMPARO_BAD_ARGUMENT;
+    return launch_status();
+}
+
+// Single-token rows: one thread per (row, channel) reads the history, writes
+// the output and the shifted history. It owns its channel, so nothing races.
+template <typename TOut>
+__global__ void k_short_conv_decode(const float* __restrict__ bcx, const float* __restrict__ weight,
+                                    const float* __restrict__ bias, float* __restrict__ state,
+                                    const int32_t* __restrict__ slot, TOut* __restrict__ out, int width, int taps) {
+    const int ch = blockIdx.x * blockDim.x + threadIdx.x;
+    const int r = blockIdx.y;
+    if (ch >= width) return;
+    const int history = taps - 1;
+    float* st = state + (size_t)slot[r] * history * width;
+    const size_t row = (size_t)r * 3 * width;
+    const float u = bcx[row + ch] * bcx[row + 2 * width + ch];
+    // the taps are summed oldest first, exactly as the general kernel sums them
+    float acc = 0.f;
+    float prev = st[ch];                                  // oldest
+    for (int k = 0; k < history; ++k) {
+        acc = fmaf(weight[(size_t)ch * taps + k], prev, acc);
+        const float next = (k + 1 < history) ? st[(size_t)(k + 1) * width + ch] : u;
+        st[(size_t)k * width + ch] = next;
+        prev = next;
+    }
+    acc = fmaf(weight[(size_t)ch * taps + history], u, acc);
+    if (bias) acc += bias[ch];
+    store_f32<TOut>(out, (size_t)r * width + ch, bcx[row + width + ch] * acc);
+}
+
+extern "C" int imparo_short_conv_decode(const float* bcx, const float* weight, const float* bias, float* state,
+                                        const int32_t* slot, void* out, int out_dtype, int n_rows, int width,
+                                        int taps, int n_slots, imparo_stream stream) {
+    if (!bcx || !weight || !state || !slot || !out) return IMPARO_BAD_ARGUMENT;
+    if (n_rows < 0 || width <= 0 || taps < 2 || taps > 64 || n_slots <= 0) return IMPARO_BAD_ARGUMENT;
+    if (n_rows == 0) return IMPARO_OK;
+    if (n_rows > 65535) return IMPARO_BAD_ARGUMENT;
+    hipStream_t s = (hipStream_t)stream;
+    const int threads = width >= 256 ? 256 : 64;
+    dim3 grid((width + threads - 1) / threads, n_rows);
+    if (out_dtype == IMPARO_F32)
+        k_short_conv_decode<float><<<grid, threads, 0, s>>>(bcx, weight, bias, state, slot, (float*)out, width, taps);
+    else if (out_dtype == IMPARO_BF16)
+        k_short_conv_decode<bf16_t><<<grid, threads, 0, s>>>(bcx, weight, bias, state, slot, (bf16_t*)out, width, taps);
     else
         return IMPARO_BAD_ARGUMENT;
     return launch_status();

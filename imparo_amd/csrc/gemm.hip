@@ -18,6 +18,11 @@ union Frag8 {
     bf16x8 v;
 };
 
+#define EPI_NONE 0
+#define EPI_SWIGLU 1   // weight rows interleaved gate, up, gate, up...: out[m, j] = silu(y[m, 2j]) * y[m, 2j+1]
+
+__device__ __forceinline__ float silu_mul_f(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+
 // ------------------------------------------------------------------ float32
 #define F32_BM 64
 #define F32_BN 64
@@ -25,7 +30,8 @@ union Frag8 {
 
 template <typename TOut>
 __global__ __launch_bounds__(256) void k_gemm_f32(const float* __restrict__ X, const float* __restrict__ W,
-                                                  TOut* __restrict__ Y, int M, int N, int K) {
+                                                  const float* __restrict__ bias, TOut* __restrict__ Y,
+                                                  int M, int N, int K, int epilogue) {
     __shared__ float As[F32_BK][F32_BM + 4];
     __shared__ float Bs[F32_BK][F32_BN + 4];
     const int tid = threadIdx.x;
@@ -67,6 +73,21 @@ __global__ __launch_bounds__(256) void k_gemm_f32(const float* __restrict__ X, c
     for (int i = 0; i < 4; ++i) {
         const int m = m0 + ty * 4 + i;
         if (m >= M) continue;
+        if (bias) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int n = n0 + tx * 4 + j;
+                if (n < N) acc[i][j] += bias[n];
+            }
+        }
+        if (epilogue == EPI_SWIGLU) {
+#pragma unroll
+            for (int j = 0; j < 4; j += 2) {
+                const int n = n0 + tx * 4 + j;
+                if (n + 1 < N) store_f32<TOut>(Y, (size_t)m * (N / 2) + n / 2, silu_mul_f(acc[i][j], acc[i][j + 1]));
+            }
+            continue;
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + tx * 4 + j;
@@ -76,51 +97,72 @@ __global__ __launch_bounds__(256) void k_gemm_f32(const float* __restrict__ X, c
 }
 
 // ------------------------------------------------------------------ bfloat16, many rows
+// 128x128 output tile per block of four waves (2x2, 64x64 each as 2x2 MFMA
+// tiles of 32x32x16), K in steps of 64. Global loads run three K-steps ahead
+// in registers, LDS is double-buffered, one barrier per K-step. Blocks are
+// numbered so that those sharing rows of X and W sit on the same XCD (blocks
+// go to the 8 XCDs round-robin, each XCD has its own L2).
 #define BG_BM 128
 #define BG_BN 128
-#define BG_BK 32
-#define BG_LD 40   // LDS row stride in elements: 80 bytes keeps 16-byte reads of 16 rows on distinct banks
+#define BG_BK 64
+#define BG_LD 72   // LDS row stride in elements: 144 bytes keeps 16-byte reads of 16 rows on distinct banks
+#define BG_PF 3    // K-steps in flight
+#define BG_GROUP_M 8
+#define N_XCD 8
 
 template <typename TOut>
-__global__ __launch_bounds__(256) void k_gemm_bf16_tile(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
-                                                        TOut* __restrict__ Y, int M, int N, int K) {
+__global__ __launch_bounds__(256, 2) void k_gemm_bf16_tile(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+                                                           const float* __restrict__ bias, TOut* __restrict__ Y,
+                                                           int M, int N, int K, int tiles_m, int tiles_n,
+                                                           int epilogue) {
     __shared__ __attribute__((aligned(16))) bf16_t As[2][BG_BM * BG_LD];
     __shared__ __attribute__((aligned(16))) bf16_t Bs[2][BG_BN * BG_LD];
+    // block id -> tile: consecutive logical ids on one XCD, grouped over 8 tile rows
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + N_XCD - 1) / N_XCD;
+    const int logical = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;
+    if (logical >= total) return;
+    const int per_group = BG_GROUP_M * tiles_n;
+    const int first_m = (logical / per_group) * BG_GROUP_M;
+    const int gsize = min(tiles_m - first_m, BG_GROUP_M);
+    const int tile_m = first_m + (logical % per_group) % gsize;
+    const int tile_n = (logical % per_group) / gsize;
+
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * BG_BM, n0 = blockIdx.x * BG_BN;
+    const int m0 = tile_m * BG_BM, n0 = tile_n * BG_BN;
 
-    // this thread's two 16-byte pieces of each operand tile
-    const bf16_t* pa[2];
-    const bf16_t* pb[2];
-    int lds_off[2], kc8[2];
+    // this thread's four 16-byte pieces of each operand tile: rows tid/8 + 32 j, columns (tid%8)*8
+    const int kc8 = (tid & 7) * 8;
+    const bf16_t* pa[4];
+    const bf16_t* pb[4];
+    int lds_off[4];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int c = tid + j * 256;
-        const int row = c >> 2;
-        kc8[j] = (c & 3) * 8;
-        pa[j] = X + (size_t)min(m0 + row, M - 1) * K + kc8[j];
-        pb[j] = W + (size_t)min(n0 + row, N - 1) * K + kc8[j];
-        lds_off[j] = row * BG_LD + kc8[j];
+    for (int j = 0; j < 4; ++j) {
+        const int row = (tid >> 3) + 32 * j;
+        pa[j] = X + (size_t)min(m0 + row, M - 1) * K + kc8;
+        pb[j] = W + (size_t)min(n0 + row, N - 1) * K + kc8;
+        lds_off[j] = row * BG_LD + kc8;
     }
     const int nk = (K + BG_BK - 1) / BG_BK;
-    uint4 ra[2], rb[2];
-    const uint4 zero = make_uint4(0, 0, 0, 0);
+    // three register sets, one per K-step in flight (named apart so that they stay in registers)
+    uint4 a0[4], b0[4], a1[4], b1[4], a2[4], b2[4];
 
-    auto fetch = [&](int kt) {
+    auto fetch = [&](int kt, uint4 (&a)[4], uint4 (&b)[4]) {
+        const bool in = kt * BG_BK + kc8 < K;
+        const size_t off = (size_t)kt * BG_BK;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const bool in = kt * BG_BK + kc8[j] < K;
-            ra[j] = in ? *reinterpret_cast<const uint4*>(pa[j] + (size_t)kt * BG_BK) : zero;
-            rb[j] = in ? *reinterpret_cast<const uint4*>(pb[j] + (size_t)kt * BG_BK) : zero;
+        for (int j = 0; j < 4; ++j) {
+            a[j] = in ? *reinterpret_cast<const uint4*>(pa[j] + off) : make_uint4(0, 0, 0, 0);
+            b[j] = in ? *reinterpret_cast<const uint4*>(pb[j] + off) : make_uint4(0, 0, 0, 0);
         }
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](int buf, const uint4 (&a)[4], const uint4 (&b)[4]) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            *reinterpret_cast<uint4*>(&As[buf][lds_off[j]]) = ra[j];
-            *reinterpret_cast<uint4*>(&Bs[buf][lds_off[j]]) = rb[j];
+        for (int j = 0; j < 4; ++j) {
+            *reinterpret_cast<uint4*>(&As[buf][lds_off[j]]) = a[j];
+            *reinterpret_cast<uint4*>(&Bs[buf][lds_off[j]]) = b[j];
         }
     };
 
@@ -132,30 +174,48 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_tile(const bf16_t* __restrict
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    fetch(0);
-    stash(0);
-    __syncthreads();
     const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) fetch(kt + 1);
+    const int a_base = (wm * 64 + frag_row) * BG_LD + frag_k;
+    const int b_base = (wn * 64 + frag_row) * BG_LD + frag_k;
+    auto compute = [&](int buf) {
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            Frag8 a[2], b[2];
+        for (int ks = 0; ks < BG_BK / 16; ++ks) {
+            Frag8 fa[2], fb[2];
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                a[i].u = *reinterpret_cast<const uint4*>(&As[buf][(wm * 64 + i * 32 + frag_row) * BG_LD + ks * 16 + frag_k]);
+            for (int ii = 0; ii < 2; ++ii)
+                fa[ii].u = *reinterpret_cast<const uint4*>(&As[buf][a_base + ii * 32 * BG_LD + ks * 16]);
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                b[j].u = *reinterpret_cast<const uint4*>(&Bs[buf][(wn * 64 + j * 32 + frag_row) * BG_LD + ks * 16 + frag_k]);
+            for (int jj = 0; jj < 2; ++jj)
+                fb[jj].u = *reinterpret_cast<const uint4*>(&Bs[buf][b_base + jj * 32 * BG_LD + ks * 16]);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int ii = 0; ii < 2; ++ii)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i].v, b[j].v, acc[i][j], 0, 0, 0);
+                for (int jj = 0; jj < 2; ++jj)
+                    acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ii].v, fb[jj].v, acc[ii][jj], 0, 0, 0);
         }
-        if (kt + 1 < nk) stash(buf ^ 1);
+    };
+    // K-step i: the next step's tile goes from its registers to LDS, those registers
+    // take the load of step i+1+BG_PF, then step i is multiplied out of LDS
+    auto step = [&](int i, uint4 (&na)[4], uint4 (&nb)[4]) {
+        const int buf = i & 1;
+        if (i + 1 < nk) {
+            stash(buf ^ 1, na, nb);
+            fetch(i + 1 + BG_PF, na, nb);
+        }
+        compute(buf);
         __syncthreads();
+    };
+
+    fetch(0, a0, b0);
+    fetch(1, a1, b1);
+    fetch(2, a2, b2);
+    stash(0, a0, b0);
+    fetch(3, a0, b0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; kt += BG_PF) {
+        step(kt, a1, b1);
+        if (kt + 1 < nk) step(kt + 1, a2, b2);
+        if (kt + 2 < nk) step(kt + 2, a0, b0);
     }
     // D layout of the 32x32 tile: lane holds column lane%32, rows 8*(r/4) + 4*(lane/32) + r%4
 #pragma unroll
@@ -163,11 +223,24 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_tile(const bf16_t* __restrict
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+            const float bn = (bias && n < N) ? bias[n] : 0.f;
+            if (epilogue == EPI_SWIGLU) {
+                // gate and up of one output sit in neighbouring lanes (n even, n odd)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float mine = acc[i][j][r] + bn;
+                    const float other = __shfl_xor(mine, 1, WAVE);
+                    const int m = m0 + wm * 64 + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                    if (!(lane & 1) && n + 1 < N && m < M)
+                        store_f32<TOut>(Y, (size_t)m * (N / 2) + n / 2, silu_mul_f(mine, other));
+                }
+                continue;
+            }
             if (n >= N) continue;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = m0 + wm * 64 + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-                if (m < M) store_f32<TOut>(Y, (size_t)m * N + n, acc[i][j][r]);
+                if (m < M) store_f32<TOut>(Y, (size_t)m * N + n, acc[i][j][r] + bn);
             }
         }
 }
@@ -182,7 +255,9 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_tile(const bf16_t* __restrict
 template <typename TOut, int MT>
 __global__ __launch_bounds__(SK_WAVES * 64) void k_gemm_bf16_skinny(const bf16_t* __restrict__ X,
                                                                     const bf16_t* __restrict__ W,
-                                                                    TOut* __restrict__ Y, int M, int N, int K) {
+                                                                    const float* __restrict__ bias,
+                                                                    TOut* __restrict__ Y, int M, int N, int K,
+                                                                    int epilogue) {
     __shared__ float red[SK_WAVES][MT][64][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0 = blockIdx.x * 16;
@@ -225,47 +300,67 @@ __global__ __launch_bounds__(SK_WAVES * 64) void k_gemm_bf16_skinny(const bf16_t
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + r16;
+        float v[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            float v = red[0][mt][lane][i];
+            v[i] = red[0][mt][lane][i];
 #pragma unroll
-            for (int w = 1; w < SK_WAVES; ++w) v += red[w][mt][lane][i];
+            for (int w = 1; w < SK_WAVES; ++w) v[i] += red[w][mt][lane][i];
             const int n = n0 + g * 4 + i;
-            if (m < M && n < N) store_f32<TOut>(Y, (size_t)m * N + n, v);
+            if (bias && n < N) v[i] += bias[n];
+        }
+        if (m >= M) continue;
+        if (epilogue == EPI_SWIGLU) {
+#pragma unroll
+            for (int i = 0; i < 4; i += 2) {
+                const int n = n0 + g * 4 + i;
+                if (n + 1 < N) store_f32<TOut>(Y, (size_t)m * (N / 2) + n / 2, silu_mul_f(v[i], v[i + 1]));
+            }
+            continue;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int n = n0 + g * 4 + i;
+            if (n < N) store_f32<TOut>(Y, (size_t)m * N + n, v[i]);
         }
     }
 }
 
 template <typename TOut>
-static int launch_bf16(const bf16_t* x, const bf16_t* w, TOut* y, int m, int n, int k, hipStream_t s) {
+static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
+                       hipStream_t s) {
     if (m <= 64) {
         const unsigned blocks = (unsigned)((n + 15) / 16);
         if (m <= 16)
-            k_gemm_bf16_skinny<TOut, 1><<<blocks, SK_WAVES * 64, 0, s>>>(x, w, y, m, n, k);
+            k_gemm_bf16_skinny<TOut, 1><<<blocks, SK_WAVES * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
         else if (m <= 32)
-            k_gemm_bf16_skinny<TOut, 2><<<blocks, SK_WAVES * 64, 0, s>>>(x, w, y, m, n, k);
+            k_gemm_bf16_skinny<TOut, 2><<<blocks, SK_WAVES * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
         else
-            k_gemm_bf16_skinny<TOut, 4><<<blocks, SK_WAVES * 64, 0, s>>>(x, w, y, m, n, k);
+            k_gemm_bf16_skinny<TOut, 4><<<blocks, SK_WAVES * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
     } else {
-        dim3 grid((n + BG_BN - 1) / BG_BN, (m + BG_BM - 1) / BG_BM);
-        if (grid.y > 65535) return IMPARO_BAD_ARGUMENT;
-        k_gemm_bf16_tile<TOut><<<grid, 256, 0, s>>>(x, w, y, m, n, k);
+        const int tiles_m = (m + BG_BM - 1) / BG_BM, tiles_n = (n + BG_BN - 1) / BG_BN;
+        const long long total = (long long)tiles_m * tiles_n;
+        if (total > 0x7fffff00LL) return IMPARO_BAD_ARGUMENT;
+        const unsigned blocks = (unsigned)(((total + N_XCD - 1) / N_XCD) * N_XCD);
+        k_gemm_bf16_tile<TOut><<<blocks, 256, 0, s>>>(x, w, bias, y, m, n, k, tiles_m, tiles_n, epilogue);
     }
     return launch_status();
 }
 
-extern "C" int imparo_gemm(const void* x, const void* w, void* y, int dtype, int out_dtype,
-                           int m, int n, int k, imparo_stream stream) {
+extern "C" int imparo_gemm(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
+                           int m, int n, int k, int epilogue, imparo_stream stream) {
     if (!x || !w || !y || m < 0 || n <= 0 || k <= 0) return IMPARO_BAD_ARGUMENT;
+    if (epilogue != EPI_NONE && epilogue != EPI_SWIGLU) return IMPARO_BAD_ARGUMENT;
+    if (epilogue == EPI_SWIGLU && (n % 2 != 0)) return IMPARO_BAD_ARGUMENT;
     if (m == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;
     if (dtype == IMPARO_F32) {
         dim3 grid((n + F32_BN - 1) / F32_BN, (m + F32_BM - 1) / F32_BM);
         if (grid.y > 65535) return IMPARO_BAD_ARGUMENT;
         if (out_dtype == IMPARO_F32)
-            k_gemm_f32<float><<<grid, 256, 0, s>>>((const float*)x, (const float*)w, (float*)y, m, n, k);
+            k_gemm_f32<float><<<grid, 256, 0, s>>>((const float*)x, (const float*)w, bias, (float*)y, m, n, k, epilogue);
         else if (out_dtype == IMPARO_BF16)
-            k_gemm_f32<bf16_t><<<grid, 256, 0, s>>>((const float*)x, (const float*)w, (bf16_t*)y, m, n, k);
+            k_gemm_f32<bf16_t><<<grid, 256, 0, s>>>((const float*)x, (const float*)w, bias, (bf16_t*)y, m, n, k, epilogue);
         else
             return IMPARO_BAD_ARGUMENT;
         return launch_status();
@@ -273,7 +368,9 @@ extern "C" int imparo_gemm(const void* x, const void* w, void* y, int dtype, int
     if (dtype != IMPARO_BF16) return IMPARO_BAD_ARGUMENT;
     // 16-byte loads along K: rows must start 16-byte aligned
     if (k % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return IMPARO_BAD_ARGUMENT;
-    if (out_dtype == IMPARO_F32) return launch_bf16<float>((const bf16_t*)x, (const bf16_t*)w, (float*)y, m, n, k, s);
-    if (out_dtype == IMPARO_BF16) return launch_bf16<bf16_t>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, m, n, k, s);
+    if (out_dtype == IMPARO_F32)
+        return launch_bf16<float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)y, m, n, k, epilogue, s);
+    if (out_dtype == IMPARO_BF16)
+        return launch_bf16<bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)y, m, n, k, epilogue, s);
     return IMPARO_BAD_ARGUMENT;
 }

@@ -99,14 +99,19 @@ def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
 
 
 def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """y += bias on every row (the GEMM kernels add a bias themselves; this is
+    for other producers)."""
     m, n = y.shape
     _check(library().imparo_add_bias(_dev(y, "add_bias y", torch.float32), _dev(bias, "bias", torch.float32, (n,)),
                                      m, n, _stream()), "add_bias")
     return y
 
 
-def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[m, n] = x[m, k] . w[n, k]^T; x and w share a dtype; float32 accumulate."""
+def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
+         swiglu: bool = False) -> torch.Tensor:
+    """out[m, n] = x[m, k] . w[n, k]^T (+ bias[n]); x and w share a dtype; float32
+    accumulate. With `swiglu` the rows of w alternate gate and up and out is
+    [m, n/2] = silu(gate) * up."""
     m, k = x.shape
     n, kw = w.shape
     if kw != k:
@@ -115,8 +120,11 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         raise KernelArgumentError(f"gemm: x is {x.dtype} but the weight is {w.dtype}")
     if x.dtype == torch.bfloat16 and k % 8 != 0:
         raise KernelArgumentError(f"gemm: the bfloat16 kernels need the inner size to be a multiple of 8, got {k}")
-    _check(library().imparo_gemm(_dev(x, "gemm x"), _dev(w, "gemm weight"), _dev(out, "gemm out", None, (m, n)),
-                                 _code(x, "gemm x"), _code(out, "gemm out"), m, n, k, _stream()), "gemm")
+    if swiglu and n % 2:
+        raise KernelArgumentError("gemm: a gate/up weight has an even number of rows")
+    _check(library().imparo_gemm(_dev(x, "gemm x"), _dev(w, "gemm weight"), _dev(bias, "gemm bias", torch.float32, (n,)),
+                                 _dev(out, "gemm out", None, (m, n // 2 if swiglu else n)),
+                                 _code(x, "gemm x"), _code(out, "gemm out"), m, n, k, int(swiglu), _stream()), "gemm")
     return out
 
 
@@ -233,9 +241,11 @@ def attention_prefill(q, k_cache, v_cache, out, rows, n_rows: int, n_tiles: int,
 
 def short_conv(bcx: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
                row_of_token: torch.Tensor, seg_start: torch.Tensor, seg_len: torch.Tensor, slot: torch.Tensor,
-               out: torch.Tensor) -> torch.Tensor:
+               out: torch.Tensor, single_tokens: bool = False) -> torch.Tensor:
     """Gated short convolution of every request's segment, then the state
-    update; the two launches are ordered by the stream."""
+    update; the two launches are ordered by the stream. `single_tokens`: the
+    caller knows that every request brings exactly one token; output and
+    update then share one launch."""
     n, three_w = bcx.shape
     width, taps = weight.shape
     if three_w != 3 * width:
@@ -243,7 +253,16 @@ def short_conv(bcx: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     n_slots = state.shape[0]
     n_rows = seg_start.shape[0]
     lib = library()
-    common = dict()
+    if single_tokens:
+        if n != n_rows:
+            raise KernelArgumentError("short_conv: single_tokens needs one token per request")
+        _check(lib.imparo_short_conv_decode(
+            _dev(bcx, "bcx", torch.float32), _dev(weight, "conv weight", torch.float32),
+            _dev(bias, "conv bias", torch.float32, (width,)),
+            _dev(state, "conv state", torch.float32, (n_slots, taps - 1, width)),
+            _dev(slot, "slot", torch.int32, (n_rows,)), _dev(out, "conv out", None, (n, width)), _code(out, "conv out"),
+            n_rows, width, taps, n_slots, _stream()), "short_conv_decode")
+        return out
     _check(lib.imparo_short_conv(
         _dev(bcx, "bcx", torch.float32), _dev(weight, "conv weight", torch.float32),
         _dev(bias, "conv bias", torch.float32, (width,)),

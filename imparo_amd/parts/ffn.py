@@ -42,8 +42,10 @@ class SwiGlu:
         gate, up = tensors[n["gate"] + ".weight"], tensors[n["up"] + ".weight"]
         if gate.dtype != up.dtype:
             gate, up = gate.to(torch.float32), up.to(torch.float32)
-        # gate | up as one projection: the same dot products, one launch
-        self.gate_up = Linear(place_matrix(torch.cat([gate, up], dim=0), engine_dtype, device))
+        # gate and up as one projection with alternating rows (g0, u0, g1, u1, ...): the same dot
+        # products, one launch, and the GEMM's epilogue applies silu(gate) * up before it stores
+        fused = torch.stack([gate, up], dim=1).reshape(2 * self.hidden, self.width)
+        self.gate_up = Linear(place_matrix(fused, engine_dtype, device))
         self.down = Linear(place_matrix(tensors[n["down"] + ".weight"], engine_dtype, device))
 
     @property
@@ -51,10 +53,7 @@ class SwiGlu:
         return self.gate_up.in_dtype
 
     def forward(self, ctx: StepContext, n: torch.Tensor) -> torch.Tensor:
-        T = n.shape[0]
-        gu = self.gate_up(ctx, n, torch.float32, "gate_up")
-        g = ctx.workspace.get("gated", (T, self.hidden), self.down.in_dtype)
-        ops.silu_mul(gu, g)
+        g = self.gate_up(ctx, n, self.down.in_dtype, "gated", swiglu=True)
         return self.down(ctx, g, torch.float32, "ffn_out")
 
 

@@ -27,14 +27,13 @@ class Linear:
     def in_dtype(self) -> torch.dtype:
         return self.weight.dtype
 
-    def __call__(self, ctx: StepContext, x: torch.Tensor, out_dtype: torch.dtype, name: str) -> torch.Tensor:
-        if self.bias is not None and out_dtype != torch.float32:
-            raise ValueError("a projection with a bias writes float32")
-        out = ctx.workspace.get(name, (x.shape[0], self.out_features), out_dtype)
-        ops.gemm(x, self.weight, out)
-        if self.bias is not None:
-            ops.add_bias(out, self.bias)
-        return out
+    def __call__(self, ctx: StepContext, x: torch.Tensor, out_dtype: torch.dtype, name: str,
+                 swiglu: bool = False) -> torch.Tensor:
+        """`swiglu`: the weight's rows alternate gate and up; the output is
+        silu(gate) * up, half as wide."""
+        width = self.out_features // 2 if swiglu else self.out_features
+        out = ctx.workspace.get(name, (x.shape[0], width), out_dtype)
+        return ops.gemm(x, self.weight, out, bias=self.bias, swiglu=swiglu)
 
 
 def place_matrix(t: torch.Tensor, engine_dtype: torch.dtype, device: torch.device) -> torch.Tensor:

@@ -68,7 +68,7 @@ class ShortConv:
         bcx = self.in_proj(ctx, h, torch.float32, "bcx")
         y = ctx.workspace.get("conv_out", (T, self.width), self.out_proj.in_dtype)
         ops.short_conv(bcx, self.conv_weight, self.conv_bias, ctx.fixed_state(site), ctx.row_of_token,
-                       ctx.seg_start, ctx.seg_len, ctx.slot, y)
+                       ctx.seg_start, ctx.seg_len, ctx.slot, y, single_tokens=ctx.max_seg_len == 1)
         return self.out_proj(ctx, y, torch.float32, "mixer_out")
 
 

@@ -46,6 +46,36 @@ def test_gemm(m, n, k):
     assert torch.equal(outb.cpu(), out.cpu().to(torch.bfloat16))      # only the final rounding differs
 
 
+@pytest.mark.parametrize("m", [1, 20, 64, 150])
+def test_gemm_epilogues(m):
+    """A bias, and the SwiGLU epilogue over a weight whose rows alternate gate and up, in the
+    float32 kernel and both bfloat16 kernels."""
+    n, k = 2 * 88, 72
+    x, w, b = rnd(m, k, seed=1), rnd(n, k, seed=2, scale=0.3), rnd(n, seed=3)
+    for dt in (torch.float32, torch.bfloat16):
+        xd, wd = x.to(dt), w.to(dt)
+        y = xd.double() @ wd.double().t() + b.double()
+        out = torch.empty(m, n, device=DEV)
+        ops().gemm(xd.to(DEV), wd.to(DEV), out, bias=b.to(DEV))
+        torch.testing.assert_close(out.cpu().double(), y, rtol=1e-5, atol=1e-5)
+        gate, up = y[:, 0::2], y[:, 1::2]
+        ref = (gate / (1 + torch.exp(-gate)) * up)
+        out = torch.empty(m, n // 2, device=DEV)
+        ops().gemm(xd.to(DEV), wd.to(DEV), out, bias=b.to(DEV), swiglu=True)
+        torch.testing.assert_close(out.cpu().double(), ref, rtol=1e-5, atol=1e-5)
+        outb = torch.empty(m, n // 2, dtype=torch.bfloat16, device=DEV)
+        ops().gemm(xd.to(DEV), wd.to(DEV), outb, bias=b.to(DEV), swiglu=True)
+        assert torch.equal(outb.cpu(), out.cpu().to(torch.bfloat16))
+    # an odd last column never pairs with its neighbour's tile: n = 2 * odd, edge tiles
+    n = 2 * 67
+    w = rnd(n, k, seed=4, scale=0.3).to(torch.bfloat16)
+    y = x.to(torch.bfloat16).double() @ w.double().t()
+    out = torch.empty(m, n // 2, device=DEV)
+    ops().gemm(x.to(torch.bfloat16).to(DEV), w.to(DEV), out, swiglu=True)
+    torch.testing.assert_close(out.cpu().double(), y[:, 0::2] / (1 + torch.exp(-y[:, 0::2])) * y[:, 1::2],
+                               rtol=1e-5, atol=1e-5)
+
+
 def test_gemm_refuses_what_it_cannot_take():
     from imparo_amd.kernels import KernelArgumentError
     x, w = rnd(4, 12).to(torch.bfloat16).to(DEV), rnd(8, 12).to(torch.bfloat16).to(DEV)
@@ -290,6 +320,30 @@ def test_short_conv(width, taps):
                 at += n
             for slot in set(range(8)) - set(slots):          # other requests' state is left alone
                 assert torch.equal(state[slot].cpu(), state0[slot])
+
+
+@pytest.mark.parametrize("width,taps", [(8, 2), (100, 3), (300, 4), (64, 7)])
+def test_short_conv_single_tokens_in_one_launch(width, taps):
+    """The fused kernel for batches of single tokens gives the same bits as the general pair."""
+    segments = [(5, 1), (0, 1), (9, 1)]
+    slots = [4, 1, 6]
+    w = rnd(width, taps, seed=1, scale=0.3).to(DEV)
+    bias = rnd(width, seed=2, scale=0.1).to(DEV)
+    bcx = rnd(3, 3 * width, seed=4).to(DEV)
+    state0 = rnd(8, taps - 1, width, seed=3)
+    results = []
+    for single in (False, True):
+        ctx = hand_context(segments, 16, 16, torch.float32, DEV, fixed_sites={0: (taps - 1, width)}, slots=slots)
+        state = ctx.fixed_state(0)
+        state.copy_(state0)
+        out = torch.empty(3, width, device=DEV)
+        ops().short_conv(bcx, w, bias, state, ctx.row_of_token, ctx.seg_start, ctx.seg_len, ctx.slot, out,
+                         single_tokens=single)
+        results.append((out.cpu(), state.cpu().clone()))
+    assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
+    y, s = P.short_conv(bcx[1:2].cpu(), w.cpu().reshape(width, 1, taps), bias.cpu(), state=state0[1])
+    torch.testing.assert_close(results[1][0][1:2], y, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(results[1][1][1], s, rtol=1e-6, atol=1e-6)
 
 
 def test_short_conv_exact_vectors_from_the_reference():
