@@ -76,6 +76,44 @@ __global__ void k_rms_norm(float* __restrict__ x, const float* __restrict__ delt
     }
 }
 
+// The same for rows whose width is a multiple of 4 and at most 4 * blockDim:
+// one float4 per thread, every load of the row issued before anything waits.
+template <typename TOut>
+__global__ void k_rms_norm_v4(float* __restrict__ x, const float* __restrict__ delta,
+                              const int32_t* __restrict__ rows, const float* __restrict__ weight,
+                              TOut* __restrict__ out, int width, float eps, int write_back) {
+    __shared__ float scratch[16];
+    const int i_out = blockIdx.x;
+    const size_t src = (size_t)(rows ? rows[i_out] : i_out) * width;
+    const size_t dst = (size_t)i_out * width;
+    const int i = threadIdx.x * 4;
+    const bool in = i < width;
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f), w = a;
+    if (in) {
+        a = *reinterpret_cast<const float4*>(x + src + i);
+        w = *reinterpret_cast<const float4*>(weight + i);
+        if (delta) {
+            const float4 d = *reinterpret_cast<const float4*>(delta + src + i);
+            a.x += d.x;
+            a.y += d.y;
+            a.z += d.z;
+            a.w += d.w;
+        }
+        if (write_back) *reinterpret_cast<float4*>(x + src + i) = a;
+    }
+    // the same order of squares as the scalar kernel would not matter: each kernel is
+    // used for a given width whatever the batch, so a row always sums the same way
+    const float ss = a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
+    const float total = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(total / (float)width + eps);
+    if (in) {
+        store_f32<TOut>(out, dst + i, a.x * scale * w.x);
+        store_f32<TOut>(out, dst + i + 1, a.y * scale * w.y);
+        store_f32<TOut>(out, dst + i + 2, a.z * scale * w.z);
+        store_f32<TOut>(out, dst + i + 3, a.w * scale * w.w);
+    }
+}
+
 extern "C" int imparo_rms_norm(float* x, const float* delta, const int32_t* rows, const float* weight,
                                void* out, int out_dtype, int n_rows, int width, float eps, int write_back,
                                imparo_stream stream) {
@@ -83,6 +121,17 @@ extern "C" int imparo_rms_norm(float* x, const float* delta, const int32_t* rows
     if (write_back && rows) return IMPARO_BAD_ARGUMENT;
     if (n_rows == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;
+    const bool aligned = !(((uintptr_t)x | (uintptr_t)delta | (uintptr_t)weight) & 15);
+    if (width % 4 == 0 && width >= 512 && width <= 4096 && aligned) {
+        const int threads = ((width / 4) + 63) / 64 * 64;
+        if (out_dtype == IMPARO_F32)
+            k_rms_norm_v4<float><<<n_rows, threads, 0, s>>>(x, delta, rows, weight, (float*)out, width, eps, write_back);
+        else if (out_dtype == IMPARO_BF16)
+            k_rms_norm_v4<bf16_t><<<n_rows, threads, 0, s>>>(x, delta, rows, weight, (bf16_t*)out, width, eps, write_back);
+        else
+            return IMPARO_BAD_ARGUMENT;
+        return launch_status();
+    }
     const int threads = width <= 256 ? 64 : 256;
     if (out_dtype == IMPARO_F32)
         k_rms_norm<float, 8><<<n_rows, threads, 0, s>>>(x, delta, rows, weight, (float*)out, width, eps, write_back);

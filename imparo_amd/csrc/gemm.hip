@@ -246,19 +246,28 @@ __global__ __launch_bounds__(256, 2) void k_gemm_bf16_tile(const bf16_t* __restr
 }
 
 // ------------------------------------------------------------------ bfloat16, few rows
-// One block per 16 weight rows. Its waves split K in chunks of 128: wave w
-// takes chunks w, w + n_waves, ... so the block reads each weight row as one
+// One block per 16 weight rows. Its NW waves split K in chunks of 128: wave w
+// takes chunks w, w + NW, ... so the block reads each weight row as one
 // contiguous stream. The 16 weight rows are the MFMA's M side, up to 16*MT
-// activation rows its N side. Partial sums meet in LDS and are added in wave
-// order, so the result is the same from run to run.
-#define SK_WAVES 4
-template <typename TOut, int MT>
-__global__ __launch_bounds__(SK_WAVES * 64) void k_gemm_bf16_skinny(const bf16_t* __restrict__ X,
-                                                                    const bf16_t* __restrict__ W,
-                                                                    const float* __restrict__ bias,
-                                                                    TOut* __restrict__ Y, int M, int N, int K,
-                                                                    int epilogue) {
-    __shared__ float red[SK_WAVES][MT][64][4];
+// activation rows its N side. A decode step is a chain of such products, each
+// a few megabytes: what counts is how few memory round trips one of them
+// takes, so a wave has the loads of its next chunk in flight while it
+// multiplies the current one, and NW is chosen so that a wave has few chunks.
+// Partial sums meet in LDS and are added in wave order, so the result is the
+// same from run to run.
+template <int MT>
+struct SkinnyFrags {
+    Frag8 w[4];
+    Frag8 x[MT][4];
+};
+
+template <typename TOut, int MT, int NW>
+__global__ __launch_bounds__(NW * 64) void k_gemm_bf16_skinny(const bf16_t* __restrict__ X,
+                                                              const bf16_t* __restrict__ W,
+                                                              const float* __restrict__ bias,
+                                                              TOut* __restrict__ Y, int M, int N, int K,
+                                                              int epilogue) {
+    __shared__ float red[NW][MT][64][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0 = blockIdx.x * 16;
     const int r16 = lane & 15, g = lane >> 4;
@@ -269,25 +278,35 @@ __global__ __launch_bounds__(SK_WAVES * 64) void k_gemm_bf16_skinny(const bf16_t
     f32x4 acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const uint4 zero = make_uint4(0, 0, 0, 0);
 
-    for (int k0 = wave * 128; k0 < K; k0 += SK_WAVES * 128) {
-        Frag8 wf[4];
+    auto load = [&](int k0, SkinnyFrags<MT>& f) {
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             const int k = k0 + s * 32;
-            wf[s].u = (k + g * 8 < K) ? *reinterpret_cast<const uint4*>(wrow + k) : zero;
-        }
+            const bool in = k + g * 8 < K;
+            f.w[s].u = in ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const int k = k0 + s * 32;
-                Frag8 xf;
-                xf.u = (k + g * 8 < K) ? *reinterpret_cast<const uint4*>(xrow[mt] + k) : zero;
-                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s].v, xf.v, acc[mt], 0, 0, 0);
-            }
+            for (int mt = 0; mt < MT; ++mt)
+                f.x[mt][s].u = in ? *reinterpret_cast<const uint4*>(xrow[mt] + k) : make_uint4(0, 0, 0, 0);
         }
+    };
+    auto multiply = [&](const SkinnyFrags<MT>& f) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.w[s].v, f.x[mt][s].v, acc[mt], 0, 0, 0);
+    };
+
+    SkinnyFrags<MT> cur, nxt;
+    int k0 = wave * 128;
+    if (k0 < K) load(k0, cur);
+    while (k0 < K) {
+        const int k1 = k0 + NW * 128;
+        if (k1 < K) load(k1, nxt);
+        multiply(cur);
+        cur = nxt;
+        k0 = k1;
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -305,7 +324,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void k_gemm_bf16_skinny(const bf16_t
         for (int i = 0; i < 4; ++i) {
             v[i] = red[0][mt][lane][i];
 #pragma unroll
-            for (int w = 1; w < SK_WAVES; ++w) v[i] += red[w][mt][lane][i];
+            for (int w = 1; w < NW; ++w) v[i] += red[w][mt][lane][i];
             const int n = n0 + g * 4 + i;
             if (bias && n < N) v[i] += bias[n];
         }
@@ -326,17 +345,31 @@ __global__ __launch_bounds__(SK_WAVES * 64) void k_gemm_bf16_skinny(const bf16_t
     }
 }
 
+template <typename TOut, int MT>
+static void launch_skinny(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k,
+                          int epilogue, hipStream_t s) {
+    const unsigned blocks = (unsigned)((n + 15) / 16);
+    // few chunks of 128 per wave: 4 waves up to K = 512, 8 up to 2048, 16 beyond
+    if (k <= 512)
+        k_gemm_bf16_skinny<TOut, MT, 4><<<blocks, 4 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+    else if (k <= 2048)
+        k_gemm_bf16_skinny<TOut, MT, 8><<<blocks, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+    else if (MT <= 2)
+        k_gemm_bf16_skinny<TOut, MT, 16><<<blocks, 16 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+    else   // 64 activation rows keep too many fragments in registers for 1024 threads
+        k_gemm_bf16_skinny<TOut, MT, 8><<<blocks, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+}
+
 template <typename TOut>
 static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
                        hipStream_t s) {
     if (m <= 64) {
-        const unsigned blocks = (unsigned)((n + 15) / 16);
         if (m <= 16)
-            k_gemm_bf16_skinny<TOut, 1><<<blocks, SK_WAVES * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+            launch_skinny<TOut, 1>(x, w, bias, y, m, n, k, epilogue, s);
         else if (m <= 32)
-            k_gemm_bf16_skinny<TOut, 2><<<blocks, SK_WAVES * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+            launch_skinny<TOut, 2>(x, w, bias, y, m, n, k, epilogue, s);
         else
-            k_gemm_bf16_skinny<TOut, 4><<<blocks, SK_WAVES * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+            launch_skinny<TOut, 4>(x, w, bias, y, m, n, k, epilogue, s);
     } else {
         const int tiles_m = (m + BG_BM - 1) / BG_BM, tiles_n = (n + BG_BN - 1) / BG_BN;
         const long long total = (long long)tiles_m * tiles_n;

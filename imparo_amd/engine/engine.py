@@ -52,7 +52,9 @@ class _Upload:
         self.events: List[Optional[torch.cuda.Event]] = [None] * depth
         self.turn = 0
 
-    def send(self, packed: np.ndarray) -> torch.Tensor:
+    def send(self, packed: np.ndarray, into: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Copies `packed` to the device: into this ring entry's own device
+        buffer, or into `into` (a buffer whose address a captured graph reads)."""
         i = self.turn
         self.turn = (self.turn + 1) % self.depth
         n = packed.shape[0]
@@ -63,16 +65,34 @@ class _Upload:
         if self.events[i] is not None:
             self.events[i].synchronize()     # the copy that last read this host buffer has run
         self.host[i][:n].numpy()[:] = packed
-        self.dev[i][:n].copy_(self.host[i][:n], non_blocking=True)
+        target = self.dev[i] if into is None else into
+        target[:n].copy_(self.host[i][:n], non_blocking=True)
         ev = torch.cuda.Event()
         ev.record()
         self.events[i] = ev
-        return self.dev[i]
+        return target
+
+
+class _DecodeGraph:
+    """A captured decode step for one batch shape: `rows` single-token requests
+    whose block tables are `table_width` pages wide. Its index arrays, its
+    scratch and its logits live at fixed addresses; a replay reads new indices
+    from the same place."""
+
+    def __init__(self):
+        self.graph = None
+        self.meta: Optional[torch.Tensor] = None
+        self.workspace: Optional[Workspace] = None
+        self.logits: Optional[torch.Tensor] = None
+        self.seen = 0
+
+
+TABLE_BUCKET = 8     # captured steps round their block-table width up to this many pages
 
 
 class Engine:
     def __init__(self, model_dir: str, dtype: str = "bfloat16", max_tokens: int = 8192, page_size: int = 64,
-                 max_requests: int = 64, device: str = "cuda:0"):
+                 max_requests: int = 64, device: str = "cuda:0", use_graphs: bool = True):
         if dtype not in DTYPES:
             raise ValueError(f"dtype must be one of {sorted(DTYPES)}, got {dtype!r}")
         library()                       # fail now, and loudly, if the kernels are missing
@@ -97,6 +117,11 @@ class Engine:
         self.storage = CacheStorage(self.cache, self.dtype, self.device)
         self.workspace = Workspace(self.device)
         self._upload = _Upload(self.device)
+        # decode steps (every request brings one token and wants its logits) replay a captured
+        # HIP graph: the launches of a step cost more host time than the step's kernels take
+        self.use_graphs = use_graphs
+        self._graphs: Dict[Tuple[int, int], _DecodeGraph] = {}
+        self._graph_pool = None
         self.vocab_size = self.plan.vocab_size
         self.max_position = self.plan.max_position
         self.steps_run = 0
@@ -160,19 +185,57 @@ class Engine:
                 self.cache.release(req)
             raise
 
-        ctx, token_ids, want_rows = self._pack(entries)
-        logits = self.model.forward(ctx, token_ids, want_rows)
+        if (self.use_graphs and self.model.graph_safe
+                and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)):
+            logits = self._decode_step(entries)
+        else:
+            ctx, token_ids, want_rows = self._pack(entries)
+            logits = self.model.forward(ctx, token_ids, want_rows)
         for e in entries:
             self.cache.commit(e.request, self.cache.length[e.request] + len(e.tokens))
         self.steps_run += 1
         return logits
 
-    def _pack(self, entries: Sequence[StepEntry]):
+    def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """A step of single tokens. The first step of a batch shape runs
+        launch by launch (so that every kernel it needs has been loaded), the
+        second is captured, later ones replay the capture."""
+        G = len(self.cache.groups)
+        widest = max([len(self.cache.table(g, e.request)) for e in entries for g in range(G)] or [1])
+        width = -(-widest // TABLE_BUCKET) * TABLE_BUCKET
+        key = (len(entries), width)
+        g = self._graphs.setdefault(key, _DecodeGraph())
+        g.seen += 1
+        if g.seen == 1:
+            ctx, token_ids, want_rows = self._pack(entries)
+            return self.model.forward(ctx, token_ids, want_rows)
+        if g.graph is None:
+            g.workspace = Workspace(self.device)
+            # the capture fixes grid sizes: they are sized for the widest context the tables can hold
+            ctx, token_ids, want_rows = self._pack(entries, table_width=width, workspace=g.workspace, graph=g)
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                g.logits = self.model.forward(ctx, token_ids, want_rows)
+            g.graph = graph
+        else:
+            self._pack(entries, table_width=width, workspace=g.workspace, graph=g)
+        g.graph.replay()
+        return g.logits
+
+    def _pack(self, entries: Sequence[StepEntry], table_width: Optional[int] = None,
+              workspace: Optional[Workspace] = None, graph: Optional[_DecodeGraph] = None):
+        """Builds the step's index arrays, sends them to the device in one
+        copy and wraps them in a StepContext. For a captured step the arrays go
+        to the capture's own fixed buffer and sizes are the capture's bounds."""
         R = len(entries)
         T = sum(len(e.tokens) for e in entries)
         G = len(self.cache.groups)
         lengths = [self.cache.length[e.request] for e in entries]
         P = max(1, max(len(self.cache.table(g, e.request)) for e in entries for g in range(G)) if G else 1)
+        if table_width is not None:
+            P = table_width
         W = sum(len(e.want) for e in entries)
         # layout: tokens | positions | row_of_token | seg_start | seg_len | slot | row lists | want | tables[G][R][P]
         total = 3 * T + 4 * R + W + G * R * P
@@ -207,16 +270,22 @@ class Engine:
                 for r, e in enumerate(entries):
                     tab = self.cache.table(g, e.request)
                     tables[g, r, :len(tab)] = tab
-        dev = self._upload.send(a)
+        if graph is not None:
+            if graph.meta is None:
+                graph.meta = torch.empty(total, dtype=torch.int32, device=self.device)
+            dev = self._upload.send(a, into=graph.meta)
+        else:
+            dev = self._upload.send(a)
         block_tables = {g: dev[o_tab + g * R * P:o_tab + (g + 1) * R * P].view(R, P) for g in range(G)}
         ctx = StepContext(
             n_tokens=T, n_rows=R,
             positions=dev[o_pos:o_pos + T], row_of_token=dev[o_row:o_row + T],
             seg_start=dev[o_start:o_start + R], seg_len=dev[o_len:o_len + R], slot=dev[o_slot:o_slot + R],
             block_tables=block_tables, page_size=self.page_size, dtype=self.dtype,
-            workspace=self.workspace, storage=self.storage, group_of_site=self.cache.group_of_site,
+            workspace=workspace or self.workspace, storage=self.storage, group_of_site=self.cache.group_of_site,
             max_seg_len=max(len(e.tokens) for e in entries),
-            max_context=max(lengths[r] + len(e.tokens) for r, e in enumerate(entries)),
+            max_context=(max(lengths[r] + len(e.tokens) for r, e in enumerate(entries)) if table_width is None
+                         else table_width * self.page_size),
             decode_rows=dev[o_lists:o_lists + len(dec)], n_decode_rows=len(dec),
             prefill_rows=dev[o_lists + len(dec):o_lists + R], n_prefill_rows=len(pre),
             n_prefill_tiles=sum((len(entries[r].tokens) + 63) // 64 for r in pre),

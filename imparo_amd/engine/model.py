@@ -62,6 +62,11 @@ class Model:
                                          mk("norm", layer.ffn_norm), mk("feed_forward", layer.ffn)))
         self.final_norm = part_class("norm", plan.final_norm.kind)(plan.final_norm, tensors, device, dtype)
         self.head = part_class("head", plan.head.kind)(plan.head, tensors, device, dtype, placed)
+        # a step can be captured into a graph only if every part says it launches kernels and nothing else
+        parts = [self.embedding, self.final_norm, self.head] + self.blocks
+        for b in self.blocks:
+            parts += [b.mixer_norm, b.mixer, b.ffn_norm, b.ffn] if hasattr(b, "mixer_norm") else []
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in parts)
         # cache sites: one per entry of the run order; None where the call borrows
         self.site_of_call: List[int] = []
         self.site_specs: List[StateSpec] = []

@@ -25,6 +25,7 @@ _DEFAULT_NAMES = dict(q="q_proj", k="k_proj", v="v_proj", o="o_proj", q_norm="q_
 
 class Attention:
     role = "mixer"
+    graph_safe = True     # launches kernels only: a step made of such parts can be captured
 
     @staticmethod
     def _names(spec: PartSpec) -> Dict[str, str]:

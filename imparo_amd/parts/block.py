@@ -14,6 +14,7 @@ from .registry import register_part
 
 class PreNormBlock:
     role = "block"
+    graph_safe = True     # launches kernels only: a step made of such parts can be captured
 
     def __init__(self, mixer_norm, mixer, ffn_norm, ffn):
         self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn

@@ -18,6 +18,7 @@ from .registry import register_part
 
 class Embedding:
     role = "embedding"
+    graph_safe = True     # launches kernels only: a step made of such parts can be captured
 
     @staticmethod
     def declare(spec: PartSpec) -> Declared:
@@ -38,6 +39,7 @@ class Embedding:
 
 class LinearHead:
     role = "head"
+    graph_safe = True     # launches kernels only: a step made of such parts can be captured
 
     @staticmethod
     def declare(spec: PartSpec) -> Declared:

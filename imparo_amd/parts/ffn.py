@@ -18,6 +18,7 @@ _DEFAULT_NAMES = dict(gate="gate_proj", up="up_proj", down="down_proj")
 
 class SwiGlu:
     role = "feed_forward"
+    graph_safe = True     # launches kernels only: a step made of such parts can be captured
 
     @staticmethod
     def _names(spec: PartSpec) -> Dict[str, str]:

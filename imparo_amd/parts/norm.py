@@ -18,6 +18,7 @@ from .registry import register_part
 
 class RmsNorm:
     role = "norm"
+    graph_safe = True     # launches kernels only: a step made of such parts can be captured
 
     @staticmethod
     def declare(spec: PartSpec) -> Declared:

@@ -24,6 +24,7 @@ from .registry import register_part
 
 class ShortConv:
     role = "mixer"
+    graph_safe = True     # launches kernels only: a step made of such parts can be captured
 
     @staticmethod
     def declare(spec: PartSpec) -> Declared:

@@ -211,6 +211,45 @@ def test_cutting_and_batching_leave_float32_bits_alone(zoo, engines):
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_captured_decode_steps_equal_launched_ones(zoo, dtype):
+    """Decode steps replay a captured graph. Replays are interleaved with
+    launched work (a prompt portion of another request, a request that joins,
+    one that leaves, contexts that grow past a table bucket) and every replay
+    is compared, bit for bit, with the engine that launches each kernel."""
+    from imparo_amd.engine import StepEntry
+    V = vocab_of(zoo, "C_keen")
+    prompts = [prompt_tokens(V, n, 300 + i) for i, n in enumerate((40, 37, 90, 260))]
+    runs = []
+    for use_graphs in (True, False):
+        eng = make_engine(zoo[0]["C_keen"], dtype, page_size=16, max_tokens=4096, use_graphs=use_graphs)
+        out = []
+        for i in range(3):
+            eng.step([StepEntry(f"r{i}", prompts[i][:-30], [])])
+        for s in range(30):                          # three rows decode, teacher-forced
+            batch = [StepEntry(f"r{i}", [prompts[i][len(prompts[i]) - 30 + s]], [0]) for i in range(3)]
+            if s == 20:
+                batch = batch[:2]                    # r2 sits this step out...
+            out.append(eng.step(batch).cpu().clone())
+            if s == 20:
+                out.append(eng.step([batch_r2(prompts, s)]).cpu().clone())   # ...and goes on alone
+            if s % 7 == 3:                           # launched work between replays
+                lo = (s // 7) * 60
+                out.append(eng.step([StepEntry("late", prompts[3][lo:lo + 60], [59])]).cpu().clone())
+        if use_graphs:
+            assert any(g.graph is not None for g in eng._graphs.values())
+            assert len(eng._graphs) >= 2
+        runs.append(torch.cat(out))
+    assert torch.equal(runs[0], runs[1])
+    ref = zoo[1]["C_keen"](prompts[0])
+    check_logits(runs[0][0:1], ref[len(prompts[0]) - 30:len(prompts[0]) - 29], dtype, "first decoded row")
+
+
+def batch_r2(prompts, s):
+    from imparo_amd.engine import StepEntry
+    return StepEntry("r2", [prompts[2][len(prompts[2]) - 30 + s]], [0])
+
+
 def test_a_step_that_does_not_fit_changes_nothing(zoo):
     from imparo_amd.engine import StepEntry
     from imparo_amd.cache import OutOfPages
