@@ -112,6 +112,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the prefill")
+    ap.add_argument("--prefill-only", action="store_true", help="run only the 2,048-token prefill (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -133,7 +134,7 @@ def main() -> int:
     print(f"[bench] writing random weights ({(nums['layer_params'] + nums['head_params']) / 1e9:.2f} B parameters) ...",
           file=sys.stderr, flush=True)
     write_random_model(cfg, 2, tmp)
-    biggest = max(args.batch, 1 if args.no_points else 64)
+    biggest = max(args.batch, 1 if (args.no_points or args.prefill_only) else 64)
     engine = Engine(tmp, dtype=args.dtype, max_tokens=biggest * (args.context + 64), page_size=64,
                     max_requests=biggest)
     for f in os.listdir(tmp):
@@ -141,6 +142,10 @@ def main() -> int:
     os.rmdir(tmp)
     sampler = Sampler(engine.device)
     elem = 2 if args.dtype == "bfloat16" else 4
+    if args.prefill_only:
+        pt = prefill_run(engine, 2048, c.vocab_size, 5, 3)
+        print(json.dumps({"prefill_ms": round(pt * 1e3, 3), "tokens": 2048}), flush=True)
+        return 0
     print("[bench] decode ...", file=sys.stderr, flush=True)
     dt = decode_run(engine, sampler, args.batch, args.context, args.steps, args.warmup, c.vocab_size, 2)
     ms = dt / args.steps * 1e3
