@@ -181,32 +181,58 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_decode(
     }
 }
 
-// One wave per (decode row, head): merges the splits in order.
+// One wave per (decode row, head): merges the splits in split order. Lane s
+// first fetches split s's (max, sum), so the weights of up to 64 splits are
+// known after one round trip; the sums over splits then run with the loads of
+// several splits in flight.
 __global__ void k_attn_decode_merge(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                     bf16_t* __restrict__ out, const int32_t* __restrict__ rows,
                                     const int32_t* __restrict__ seg_start, const int32_t* __restrict__ positions,
                                     int heads, int head_dim, int n_splits, int window) {
     const int ri = blockIdx.x / heads, head = blockIdx.x % heads;
+    const int lane = threadIdx.x;
     const int t = seg_start[rows[ri]];
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
     const int s_lo = (lo & ~15) / DEC_SPLIT, s_hi = pos / DEC_SPLIT;
     const size_t base = ((size_t)ri * heads + head) * n_splits;
     float ms = -INFINITY;
-    for (int s = s_lo; s <= s_hi; ++s) ms = fmaxf(ms, part_ml[(base + s) * 2]);
+    for (int s0 = s_lo; s0 <= s_hi; s0 += WAVE) {
+        const int s = s0 + lane;
+        ms = fmaxf(ms, s <= s_hi ? part_ml[(base + s) * 2] : -INFINITY);
+    }
+    ms = wave_max(ms);
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
     float ls = 0.f;
-    for (int s = s_lo; s <= s_hi; ++s) {
-        const float m = part_ml[(base + s) * 2];
-        ls += (m == -INFINITY) ? 0.f : part_ml[(base + s) * 2 + 1] * __expf(m - ms);
+    for (int s0 = s_lo; s0 <= s_hi; s0 += WAVE) {
+        const int s = s0 + lane;
+        float wgt = 0.f, l = 0.f;
+        if (s <= s_hi) {
+            const float m = part_ml[(base + s) * 2];
+            wgt = (m == -INFINITY) ? 0.f : __expf(m - ms);
+            l = part_ml[(base + s) * 2 + 1] * wgt;
+        }
+        // sum in split order: lane by lane
+        const int n_here = min(WAVE, s_hi - s0 + 1);
+        for (int k = 0; k < n_here; ++k) ls += __shfl(l, k, WAVE);
+#pragma unroll 4
+        for (int k = 0; k < n_here; ++k) {
+            const float wk = __shfl(wgt, k, WAVE);
+            const float* po = part_o + (base + s0 + k) * head_dim;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int d = lane + j * WAVE;
+                if (d < head_dim) acc[j] += po[d] * wk;
+            }
+        }
     }
     const float inv = ls > 0.f ? 1.0f / ls : 0.f;
-    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-        float acc = 0.f;
-        for (int s = s_lo; s <= s_hi; ++s) {
-            const float m = part_ml[(base + s) * 2];
-            if (m != -INFINITY) acc += part_o[(base + s) * head_dim + d] * __expf(m - ms);
-        }
-        out[((size_t)t * heads + head) * head_dim + d] = f32_to_bf16(acc * inv);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int d = lane + j * WAVE;
+        if (d < head_dim) out[((size_t)t * heads + head) * head_dim + d] = f32_to_bf16(acc[j] * inv);
     }
 }
 

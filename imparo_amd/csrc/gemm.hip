@@ -360,9 +360,132 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, const float* bias, T
         k_gemm_bf16_skinny<TOut, MT, 8><<<blocks, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
 }
 
+// ------------------------------------------------------------------ bfloat16, few rows, many weight rows
+// For weights with so many rows that one block per 128 of them fills the chip
+// (the output head): a block of 8 waves takes 128 weight rows (16 per wave) and
+// walks all of K. The activation chunk [rows x 128] is staged in LDS once per
+// block and shared by the 8 waves, so activations cost an eighth of the L2
+// traffic they cost when every wave fetches its own; every output element is
+// summed by one wave in k order.
+#define ST_WAVES 8
+#define ST_BN (ST_WAVES * 16)
+#define ST_BK 128
+#define ST_LD (ST_BK + 8)   // LDS row stride in elements: 272 bytes, 16 rows of 16-byte reads on distinct banks
+#define ST_MIN_TILES 192    // below this many blocks the K-split kernel keeps more of the chip busy
+
+template <typename TOut, int MT>
+__global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, const float* __restrict__ bias,
+    TOut* __restrict__ Y, int M, int N, int K, int epilogue) {
+    __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16 * ST_LD];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * ST_BN + wave * 16;
+    const bf16_t* wrow = W + (size_t)min(n0 + r16, N - 1) * K + g * 8;
+
+    // staging of the activation chunk: MT*16 rows x 16 pieces of 16 bytes, 512 threads
+    constexpr int PIECES = MT * 16 * (ST_BK / 8);
+    constexpr int PER_THREAD = (PIECES + ST_WAVES * 64 - 1) / (ST_WAVES * 64);
+    auto stage_load = [&](int k0, uint4 (&r)[PER_THREAD]) {
+#pragma unroll
+        for (int j = 0; j < PER_THREAD; ++j) {
+            const int p = tid + j * ST_WAVES * 64;
+            const int row = p / (ST_BK / 8), kc = (p % (ST_BK / 8)) * 8;
+            const bool in = p < PIECES && k0 + kc < K;
+            r[j] = in ? *reinterpret_cast<const uint4*>(X + (size_t)min(row, M - 1) * K + k0 + kc)
+                      : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto stage_store = [&](int buf, const uint4 (&r)[PER_THREAD]) {
+#pragma unroll
+        for (int j = 0; j < PER_THREAD; ++j) {
+            const int p = tid + j * ST_WAVES * 64;
+            if (p < PIECES) {
+                const int row = p / (ST_BK / 8), kc = (p % (ST_BK / 8)) * 8;
+                *reinterpret_cast<uint4*>(&xs[buf][row * ST_LD + kc]) = r[j];
+            }
+        }
+    };
+    auto load_w = [&](int k0, Frag8 (&f)[4]) {
+#pragma unroll
+        for (int s2 = 0; s2 < 4; ++s2) {
+            const int k = k0 + s2 * 32;
+            f[s2].u = (k + g * 8 < K) ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
+        }
+    };
+
+    f32x4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    uint4 xr[PER_THREAD];
+    Frag8 wcur[4], wnxt[4];
+    stage_load(0, xr);
+    load_w(0, wcur);
+    stage_store(0, xr);
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = 0; k0 < K; k0 += ST_BK) {
+        const int k1 = k0 + ST_BK;
+        if (k1 < K) {
+            stage_load(k1, xr);
+            load_w(k1, wnxt);
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int s2 = 0; s2 < 4; ++s2) {
+                Frag8 xf;
+                xf.u = *reinterpret_cast<const uint4*>(&xs[buf][(mt * 16 + r16) * ST_LD + s2 * 32 + g * 8]);
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wcur[s2].v, xf.v, acc[mt], 0, 0, 0);
+            }
+        if (k1 < K) {
+            stage_store(buf ^ 1, xr);
+#pragma unroll
+            for (int s2 = 0; s2 < 4; ++s2) wcur[s2] = wnxt[s2];
+        }
+        __syncthreads();
+        buf ^= 1;
+    }
+    // D layout of the 16x16 tile: lane holds column lane%16 (an activation row), rows 4*(lane/16)+i (weight rows)
+    const int nq = n0 + g * 4;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + r16;
+        if (m >= M) continue;
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = acc[mt][i] + ((bias && nq + i < N) ? bias[nq + i] : 0.f);
+        if (epilogue == EPI_SWIGLU) {
+#pragma unroll
+            for (int i = 0; i < 4; i += 2)
+                if (nq + i + 1 < N) store_f32<TOut>(Y, (size_t)m * (N / 2) + (nq + i) / 2, silu_mul_f(v[i], v[i + 1]));
+            continue;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (nq + i < N) store_f32<TOut>(Y, (size_t)m * N + nq + i, v[i]);
+    }
+}
+
+template <typename TOut, int MT>
+static void launch_stream(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k,
+                          int epilogue, hipStream_t s) {
+    k_gemm_bf16_stream<TOut, MT><<<(n + ST_BN - 1) / ST_BN, ST_WAVES * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+}
+
 template <typename TOut>
 static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
                        hipStream_t s) {
+    if (m <= 64 && (n + ST_BN - 1) / ST_BN >= ST_MIN_TILES) {
+        if (m <= 16)
+            launch_stream<TOut, 1>(x, w, bias, y, m, n, k, epilogue, s);
+        else if (m <= 32)
+            launch_stream<TOut, 2>(x, w, bias, y, m, n, k, epilogue, s);
+        else
+            launch_stream<TOut, 4>(x, w, bias, y, m, n, k, epilogue, s);
+        return launch_status();
+    }
     if (m <= 64) {
         if (m <= 16)
             launch_skinny<TOut, 1>(x, w, bias, y, m, n, k, epilogue, s);

@@ -35,11 +35,29 @@ __device__ __forceinline__ Best row_best(const float* __restrict__ row, int voca
     Best b;
     b.v = -INFINITY;
     b.i = INT_MAX;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-        const float v = row[i];
-        if (v > b.v || (v == b.v && i < b.i)) {
-            b.v = v;
-            b.i = i;
+    if ((vocab & 3) == 0 && (((uintptr_t)row) & 15) == 0) {
+        // four values a load, four loads in flight; a thread meets its indices in ascending
+        // order, so "greater than" alone keeps the smallest index at the maximum
+        const float4* row4 = reinterpret_cast<const float4*>(row);
+        const int n4 = vocab >> 2;
+#pragma unroll 4
+        for (int i = threadIdx.x; i < n4; i += blockDim.x) {
+            const float4 v = row4[i];
+            const float vs[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (vs[j] > b.v || (vs[j] == b.v && 4 * i + j < b.i)) {
+                    b.v = vs[j];
+                    b.i = 4 * i + j;
+                }
+        }
+    } else {
+        for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+            const float v = row[i];
+            if (v > b.v || (v == b.v && i < b.i)) {
+                b.v = v;
+                b.i = i;
+            }
         }
     }
     b = block_best(b, scratch);
