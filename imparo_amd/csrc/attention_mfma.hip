@@ -238,8 +238,16 @@ __global__ void k_attn_decode_merge(const float* __restrict__ part_o, const floa
 
 // ---------------------------------------------------------------- prompt portions
 // grid (tile of 64 queries, head). A block's four waves take 16 consecutive
-// queries each and walk the keys from the lowest any of them may read up to
-// the last query's own position.
+// queries each. Keys go by in tiles of 64: the block stages the K rows and the
+// V^T rows of a tile in LDS once (next tile's loads in flight meanwhile), each
+// wave multiplies its queries against the four 16-key sub-tiles, runs one
+// softmax update over the 64 scores and adds the weighted values. Rows are
+// padded to 144 bytes in LDS so that the 8-byte operand reads of 16 rows fall
+// on distinct banks.
+#define PF_KEYS 64
+#define PF_LD_K(D) ((D) + 8)
+#define PF_LD_V (PF_KEYS + 8)
+
 template <int ND>
 __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
@@ -248,6 +256,9 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
     const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int n_pages,
     float scale, int window) {
     constexpr int D = ND * 16;
+    constexpr int LDK = PF_LD_K(D);
+    __shared__ __attribute__((aligned(16))) bf16_t ks[2][PF_KEYS * LDK];
+    __shared__ __attribute__((aligned(16))) bf16_t vs[2][D * PF_LD_V];
     int tile = blockIdx.x, row = -1;
     for (int i = 0; i < n_rows; ++i) {
         const int r = rows[i];
@@ -259,15 +270,24 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
         tile -= nt;
     }
     if (row < 0) return;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int len = seg_len[row];
-    const int q_first = tile * 64 + wave * 16;
-    if (q_first >= len) return;
     const int head = blockIdx.y;
     const int kvh = head / (heads / kv_heads);
     const int t0 = seg_start[row];
     const int pos0 = positions[t0];
+    const int32_t* table = block_table + (size_t)row * table_stride;
+
+    // the block's key range: from the lowest key its first query may read to its last query's position
+    const int blk_first = pos0 + tile * 64;
+    const int blk_last = pos0 + min(len, tile * 64 + 64) - 1;
+    const int blk_lo = window > 0 ? max(0, blk_first + 1 - window) : 0;
+
+    // this wave's queries
+    const int q_first = tile * 64 + wave * 16;
+    const bool wave_on = q_first < len;
     const int qi = q_first + c;
     const bool qvalid = qi < len;
     const int pos_q = pos0 + qi;
@@ -278,13 +298,128 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
     const int lo_all = window > 0 ? max(0, pos_first + 1 - window) : 0;
     const int lo_max = window > 0 ? max(0, pos_last + 1 - window) : 0;
     WaveState<ND> st;
-    load_q<ND>(st, q + ((size_t)(t0 + min(qi, len - 1)) * heads + head) * D, qvalid, lane);
-    Paged kv{k_cache, v_cache, block_table + (size_t)row * table_stride, page_size, kv_heads, kvh, n_pages};
-    for (int kb = lo_all & ~15; kb <= pos_last; kb += 16) {
-        const bool full = kb >= lo_max && kb + 15 <= pos_first;
-        attn_tile<ND>(st, kv, kb, lo_q, hi_q, lo_all, pos_last, full, scale, lane);
+    load_q<ND>(st, q + ((size_t)(t0 + min(qi, len - 1)) * heads + head) * D, qvalid && wave_on, lane);
+
+    // staging: K tile = 64 keys x D/8 pieces of 16 bytes; V^T tile = D rows x 8 pieces of 8 keys
+    constexpr int K_PIECES = PF_KEYS * (D / 8), V_PIECES = D * (PF_KEYS / 8);
+    constexpr int K_PER = (K_PIECES + 255) / 256, V_PER = (V_PIECES + 255) / 256;
+    uint4 kr[K_PER], vr[V_PER];
+    auto stage_load = [&](int kb) {
+#pragma unroll
+        for (int j = 0; j < K_PER; ++j) {
+            const int p = tid + j * 256;
+            const int key = min(max(kb + p / (D / 8), blk_lo), blk_last);      // a live key: address always valid
+            int page = table[key / page_size];
+            page = min(max(page, 0), n_pages - 1);
+            kr[j] = (p < K_PIECES)
+                        ? *reinterpret_cast<const uint4*>(k_cache + (((size_t)page * kv_heads + kvh) * page_size +
+                                                                     (key % page_size)) * D + (p % (D / 8)) * 8)
+                        : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < V_PER; ++j) {
+            const int p = tid + j * 256;
+            const int d = p / (PF_KEYS / 8), kg = kb + (p % (PF_KEYS / 8)) * 8;   // 8 keys kg .. kg+7, one page
+            const int kgc = min(max(kg, blk_lo & ~7), blk_last & ~7);
+            int page = table[kgc / page_size];
+            page = min(max(page, 0), n_pages - 1);
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (p < V_PIECES)
+                v = *reinterpret_cast<const uint4*>(v_cache + (((size_t)page * kv_heads + kvh) * D + d) * page_size +
+                                                    (kgc % page_size));
+            // values of keys outside the live range are zero, never stale memory
+            if (kg < blk_lo || kg + 7 > blk_last) {
+                uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (kg + e < blk_lo || kg + e > blk_last) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+                v = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+            vr[j] = v;
+        }
+    };
+    auto stage_store = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < K_PER; ++j) {
+            const int p = tid + j * 256;
+            if (p < K_PIECES) *reinterpret_cast<uint4*>(&ks[buf][(p / (D / 8)) * LDK + (p % (D / 8)) * 8]) = kr[j];
+        }
+#pragma unroll
+        for (int j = 0; j < V_PER; ++j) {
+            const int p = tid + j * 256;
+            if (p < V_PIECES)
+                *reinterpret_cast<uint4*>(&vs[buf][(p / (PF_KEYS / 8)) * PF_LD_V + (p % (PF_KEYS / 8)) * 8]) = vr[j];
+        }
+    };
+
+    const int kb_first = blk_lo & ~(PF_KEYS - 1);
+    stage_load(kb_first);
+    stage_store(0);
+    __syncthreads();
+    int buf = 0;
+    for (int kb = kb_first; kb <= blk_last; kb += PF_KEYS) {
+        const int kn = kb + PF_KEYS;
+        if (kn <= blk_last) stage_load(kn);
+        // this wave's part of the tile: keys lo_all .. pos_last
+        if (wave_on && kb <= pos_last && kb + PF_KEYS - 1 >= lo_all) {
+            const bool full = kb >= lo_max && kb + PF_KEYS - 1 <= pos_first;
+            f32x4 sc[4];
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt) {
+                sc[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                const bf16_t* krow = &ks[buf][(kt * 16 + c) * LDK + 4 * g];
+#pragma unroll
+                for (int dk = 0; dk < ND; ++dk) {
+                    const s16x4 a = *reinterpret_cast<const s16x4*>(krow + dk * 16);
+                    sc[kt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, st.q[dk], sc[kt], 0, 0, 0);
+                }
+            }
+            // sc[kt][i] = score of key kb + 16 kt + 4 g + i for query lane%16
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int kp = kb + kt * 16 + 4 * g + i;
+                    const bool ok = full || (kp >= lo_q && kp <= hi_q);
+                    sc[kt][i] = ok ? sc[kt][i] * scale : -INFINITY;
+                    mx = fmaxf(mx, sc[kt][i]);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+            const float m_new = fmaxf(st.m, mx);
+            const float corr = (st.m == -INFINITY) ? 0.f : __expf(st.m - m_new);
+            s16x4 pb[4];
+            float psum = 0.f;
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float p = (sc[kt][i] == -INFINITY) ? 0.f : __expf(sc[kt][i] - m_new);
+                    const bf16_t r = f32_to_bf16(p);
+                    pb[kt][i] = (short)r;
+                    psum += bf16_to_f32(r);
+                }
+            psum += __shfl_xor(psum, 16, WAVE);
+            psum += __shfl_xor(psum, 32, WAVE);
+            st.l = st.l * corr + psum;
+            st.m = m_new;
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) {
+                st.o[dt] = st.o[dt] * corr;
+                const bf16_t* vrow = &vs[buf][(dt * 16 + c) * PF_LD_V + 4 * g];
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt) {
+                    const s16x4 a = *reinterpret_cast<const s16x4*>(vrow + kt * 16);
+                    st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb[kt], st.o[dt], 0, 0, 0);
+                }
+            }
+        }
+        if (kn <= blk_last) stage_store(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
     }
-    if (!qvalid) return;
+    if (!qvalid || !wave_on) return;
     const float inv = st.l > 0.f ? 1.0f / st.l : 0.f;
     bf16_t* dst = out + ((size_t)(t0 + qi) * heads + head) * D + 4 * g;
 #pragma unroll
