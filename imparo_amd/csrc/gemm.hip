@@ -367,13 +367,10 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, const float* bias, T
 // block and shared by the 8 waves, so activations cost an eighth of the L2
 // traffic they cost when every wave fetches its own; every output element is
 // summed by one wave in k order.
-#define ST_WAVES 8
-#define ST_BN (ST_WAVES * 16)
 #define ST_BK 128
 #define ST_LD (ST_BK + 8)   // LDS row stride in elements: 272 bytes, 16 rows of 16-byte reads on distinct banks
-#define ST_MIN_TILES 192    // below this many blocks the K-split kernel keeps more of the chip busy
 
-template <typename TOut, int MT>
+template <typename TOut, int MT, int ST_WAVES>
 __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, const float* __restrict__ bias,
     TOut* __restrict__ Y, int M, int N, int K, int epilogue) {
@@ -381,10 +378,10 @@ __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * ST_BN + wave * 16;
+    const int n0 = blockIdx.x * (ST_WAVES * 16) + wave * 16;
     const bf16_t* wrow = W + (size_t)min(n0 + r16, N - 1) * K + g * 8;
 
-    // staging of the activation chunk: MT*16 rows x 16 pieces of 16 bytes, 512 threads
+    // staging of the activation chunk: MT*16 rows x 16 pieces of 16 bytes
     constexpr int PIECES = MT * 16 * (ST_BK / 8);
     constexpr int PER_THREAD = (PIECES + ST_WAVES * 64 - 1) / (ST_WAVES * 64);
     auto stage_load = [&](int k0, uint4 (&r)[PER_THREAD]) {
@@ -468,22 +465,44 @@ __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
     }
 }
 
+// Waves per block for the wide kernel, or 0 for "use the K-split kernel". Measured with cold
+// weights (they never stay in cache between decode steps): the wide kernel wins from about
+// 12k weight rows on, with 2 waves a block, and with 4 from about 32k rows on; below that
+// its walk along K (one chunk of 128 per round trip) costs more than shared activations save.
+static int stream_waves(int n) {
+    if (n >= 32768) return 4;
+    if (n >= 12288) return 2;
+    return 0;
+}
+
 template <typename TOut, int MT>
 static void launch_stream(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k,
-                          int epilogue, hipStream_t s) {
-    k_gemm_bf16_stream<TOut, MT><<<(n + ST_BN - 1) / ST_BN, ST_WAVES * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+                          int epilogue, int nw, hipStream_t s) {
+    const unsigned blocks = (unsigned)((n + nw * 16 - 1) / (nw * 16));
+    if (nw == 8)
+        k_gemm_bf16_stream<TOut, MT, 8><<<blocks, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+    else if (nw == 4)
+        k_gemm_bf16_stream<TOut, MT, 4><<<blocks, 4 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+    else
+        k_gemm_bf16_stream<TOut, MT, 2><<<blocks, 2 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
 }
 
 template <typename TOut>
 static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
-                       hipStream_t s) {
-    if (m <= 64 && (n + ST_BN - 1) / ST_BN >= ST_MIN_TILES) {
+                       int force, hipStream_t s) {
+    // 17..64 rows: sharing the activations between the waves of a block matters more than anything
+    // else, if the weight has rows enough for enough blocks. (Up to 16 rows the K-split kernel keeps
+    // more loads in flight and wins.) `force` (for measurements): 1 = K-split kernel, 2/4/8 = wide with that many waves
+    int nw = (m > 16) ? stream_waves(n) : 0;
+    if (force == 1) nw = 0;
+    if (force == 2 || force == 4 || force == 8) nw = force;
+    if (m <= 64 && nw) {
         if (m <= 16)
-            launch_stream<TOut, 1>(x, w, bias, y, m, n, k, epilogue, s);
+            launch_stream<TOut, 1>(x, w, bias, y, m, n, k, epilogue, nw, s);
         else if (m <= 32)
-            launch_stream<TOut, 2>(x, w, bias, y, m, n, k, epilogue, s);
+            launch_stream<TOut, 2>(x, w, bias, y, m, n, k, epilogue, nw, s);
         else
-            launch_stream<TOut, 4>(x, w, bias, y, m, n, k, epilogue, s);
+            launch_stream<TOut, 4>(x, w, bias, y, m, n, k, epilogue, nw, s);
         return launch_status();
     }
     if (m <= 64) {
@@ -502,6 +521,12 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
     }
     return launch_status();
 }
+
+static int g_force_few_row_kernel = 0;
+
+// For measurements only: 0 lets the library choose the few-row kernel, 1 forces the K-split
+// kernel, 2, 4 or 8 the wide kernel with that many waves.
+extern "C" void imparo_gemm_force_kernel(int which) { g_force_few_row_kernel = which; }
 
 extern "C" int imparo_gemm(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
                            int m, int n, int k, int epilogue, imparo_stream stream) {
@@ -525,8 +550,10 @@ extern "C" int imparo_gemm(const void* x, const void* w, const float* bias, void
     // 16-byte loads along K: rows must start 16-byte aligned
     if (k % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return IMPARO_BAD_ARGUMENT;
     if (out_dtype == IMPARO_F32)
-        return launch_bf16<float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)y, m, n, k, epilogue, s);
+        return launch_bf16<float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)y, m, n, k, epilogue,
+                                  g_force_few_row_kernel, s);
     if (out_dtype == IMPARO_BF16)
-        return launch_bf16<bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)y, m, n, k, epilogue, s);
+        return launch_bf16<bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)y, m, n, k, epilogue,
+                                   g_force_few_row_kernel, s);
     return IMPARO_BAD_ARGUMENT;
 }
