@@ -1,0 +1,55 @@
+"""Loads the host runtime library (page pools, cache manager, step packing)
+and declares its C entry points. Built with the C++ compiler at first use if
+it is not there; no GPU is needed for it."""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from ctypes import POINTER, c_int, c_int32, c_int64, c_uint64, c_void_p
+
+from ..csrc import build as _build
+
+_lock = threading.Lock()
+_lib = None
+
+I, P = c_int, c_void_p
+PI32, PI64 = POINTER(c_int32), POINTER(c_int64)
+
+_SIGNATURES = {
+    "imparo_pool_new": ([I], P), "imparo_pool_delete": ([P], None), "imparo_pool_alloc": ([P], I),
+    "imparo_pool_free": ([P, I], I), "imparo_pool_n_free": ([P], I), "imparo_pool_n_pages": ([P], I),
+    "imparo_pool_high_water": ([P], I), "imparo_pool_is_free": ([P, I], I), "imparo_pool_scramble": ([P, c_uint64], I),
+    "imparo_cache_new": ([I, P, I, I, I], P), "imparo_cache_delete": ([P], None),
+    "imparo_cache_group_pool": ([P, I], P), "imparo_cache_slot_pool": ([P], P),
+    "imparo_cache_admit": ([P, c_int64], I), "imparo_cache_release": ([P, c_int64], I),
+    "imparo_cache_reserve": ([P, c_int64, I], I), "imparo_cache_rollback": ([P, c_int64], I),
+    "imparo_cache_commit": ([P, c_int64, I], I), "imparo_cache_is_live": ([P, c_int64], I),
+    "imparo_cache_length": ([P, c_int64], I), "imparo_cache_slot": ([P, c_int64], I),
+    "imparo_cache_table_len": ([P, I, c_int64], I), "imparo_cache_table_copy": ([P, I, c_int64, P, I], I),
+    "imparo_cache_pages_needed": ([P, c_int64, I, P], I), "imparo_cache_first_needed_page": ([P, I, I], I),
+    "imparo_cache_n_live": ([P], I), "imparo_cache_live_requests": ([P, P, I], I), "imparo_cache_check": ([P], I),
+    "imparo_cache_pack": ([P, I, P, P, P, P, P, I, P, c_int64, P], c_int64),
+}
+
+E_OUT_OF_PAGES, E_NOT_LIVE, E_ALREADY_LIVE, E_SHRINK, E_DOUBLE_FREE, E_RANGE, E_BUSY, E_CAPACITY = range(-1, -9, -1)
+E_LOST_PAGE, E_SHARED_PAGE, E_SLOTS = -9, -10, -11
+
+
+def host_library() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        path = _build.host_library_path()
+        if not os.path.isfile(path):
+            path = _build.build_host(verbose=True)
+        lib = ctypes.CDLL(path)
+        for name, (argtypes, restype) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = restype
+        _lib = lib
+        return _lib

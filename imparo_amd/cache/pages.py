@@ -1,6 +1,8 @@
 """Host-side bookkeeping of the cache: pages, block tables, state slots.
 
-Nothing here touches the GPU; the tensors the pages index live in
+The bookkeeping itself is native (csrc/host/cache_manager.cpp, reached through
+a C ABI); the classes here give it Python names and errors. Nothing here
+touches the GPU; the tensors the pages index live in
 `imparo_amd.cache.storage`.
 
 Allocation always takes the lowest free page, so which pages a request gets
@@ -10,9 +12,13 @@ twice is an error. The reference's block allocator keeps the same two rules
 """
 from __future__ import annotations
 
-import heapq
+import ctypes
 from dataclasses import dataclass
-from typing import Dict, Hashable, List, Optional, Sequence, Tuple, Union
+from typing import Dict, Hashable, Iterator, List, Optional, Sequence, Tuple, Union
+
+import numpy as np
+
+from . import native as N
 
 
 class OutOfPages(RuntimeError):
@@ -24,54 +30,58 @@ class CacheError(RuntimeError):
 
 
 class PagePool:
-    def __init__(self, n_pages: int):
-        if n_pages < 0:
-            raise ValueError("a pool cannot have a negative number of pages")
-        self.n_pages = n_pages
-        self._place: Optional[List[int]] = None   # rank -> page, when placement is scrambled
-        self._rank: Optional[List[int]] = None
-        self._heap = list(range(n_pages))
-        self._free = [True] * n_pages
-        self.n_free = n_pages
-        self.high_water = 0      # one past the highest page ever handed out
+    """A pool of pages: the lowest free page first, always."""
+
+    def __init__(self, n_pages: int, _borrowed=None):
+        self._lib = N.host_library()
+        if _borrowed is not None:
+            self._p, self._owned = _borrowed, False
+        else:
+            if n_pages < 0:
+                raise ValueError("a pool cannot have a negative number of pages")
+            self._p, self._owned = self._lib.imparo_pool_new(n_pages), True
+
+    def __del__(self):
+        if getattr(self, "_owned", False) and self._p:
+            self._lib.imparo_pool_delete(self._p)
+            self._p = None
+
+    @property
+    def n_pages(self) -> int:
+        return self._lib.imparo_pool_n_pages(self._p)
+
+    @property
+    def n_free(self) -> int:
+        return self._lib.imparo_pool_n_free(self._p)
+
+    @property
+    def high_water(self) -> int:
+        """One past the highest page ever handed out."""
+        return self._lib.imparo_pool_high_water(self._p)
 
     def alloc(self) -> int:
-        if self.n_free == 0:
+        page = self._lib.imparo_pool_alloc(self._p)
+        if page < 0:
             raise OutOfPages("no free page")
-        page = heapq.heappop(self._heap)
-        if self._place is not None:
-            page = self._place[page]
-        self._free[page] = False
-        self.n_free -= 1
-        self.high_water = max(self.high_water, page + 1)
         return page
 
     def free(self, page: int) -> None:
-        if not 0 <= page < self.n_pages:
+        rc = self._lib.imparo_pool_free(self._p, page)
+        if rc == N.E_RANGE:
             raise CacheError(f"page {page} is outside the pool of {self.n_pages}")
-        if self._free[page]:
+        if rc == N.E_DOUBLE_FREE:
             raise CacheError(f"page {page} freed twice")
-        self._free[page] = True
-        self.n_free += 1
-        heapq.heappush(self._heap, page if self._rank is None else self._rank[page])
+
+    def is_free(self, page: int) -> bool:
+        return self._lib.imparo_pool_is_free(self._p, page) == 1
 
     def scramble(self, seed: int) -> None:
         """Permutes which physical page each allocation rank maps to, so that
         block tables are not the identity. Only on an untouched pool. Output
         must not depend on it: placement is invisible
         (/root/reference/crates/imparo-kv/src/resident.rs:56-99)."""
-        if self.n_free != self.n_pages:
+        if self._lib.imparo_pool_scramble(self._p, seed) != 0:
             raise CacheError("placement can only be scrambled while every page is free")
-        import random
-        place = list(range(self.n_pages))
-        random.Random(seed).shuffle(place)
-        self._place = place
-        self._rank = [0] * self.n_pages
-        for rank, page in enumerate(place):
-            self._rank[page] = rank
-
-    def is_free(self, page: int) -> bool:
-        return self._free[page]
 
 
 @dataclass(frozen=True)
@@ -92,22 +102,76 @@ class FixedSpec:
 StateSpec = Union[PagedSpec, FixedSpec, None]
 
 
+class _Tables:
+    """The block tables of one group, by request: a read-only mapping."""
+
+    def __init__(self, manager: "CacheManager", group: int):
+        self._m, self._g = manager, group
+
+    def __getitem__(self, req: Hashable) -> List[int]:
+        return self._m.table(self._g, req)
+
+    def __iter__(self) -> Iterator[Hashable]:
+        return iter(list(self._m._handles))
+
+    def __len__(self) -> int:
+        return len(self._m._handles)
+
+    def __contains__(self, req: Hashable) -> bool:
+        return req in self._m._handles
+
+    def keys(self):
+        return list(self._m._handles)
+
+    def values(self):
+        return [self[r] for r in self.keys()]
+
+    def items(self):
+        return [(r, self[r]) for r in self.keys()]
+
+
 class CacheGroup:
     """The cache sites that share one paged spec: one pool of pages, one block
     table per request, the same page ids on every site of the group."""
 
-    def __init__(self, spec: PagedSpec, sites: Sequence[int], n_pages: int, page_size: int):
+    def __init__(self, manager: "CacheManager", index: int, spec: PagedSpec, pool: PagePool, page_size: int):
+        self._m, self.index = manager, index
         self.spec = spec
-        self.sites = list(sites)
+        self.sites: List[int] = []
         self.page_size = page_size
-        self.pool = PagePool(n_pages)
-        self.tables: Dict[Hashable, List[int]] = {}
+        self.pool = pool
+        self.tables = _Tables(manager, index)
 
     def first_needed_page(self, next_position: int) -> int:
         """The lowest logical page a query at `next_position` or later reads."""
-        if self.spec.window is None:
-            return 0
-        return max(0, next_position + 1 - self.spec.window) // self.page_size
+        return self._m._lib.imparo_cache_first_needed_page(self._m._c, self.index, next_position)
+
+
+class _PerRequest:
+    """cache.length / cache.slot_of: read-only mappings over the live requests."""
+
+    def __init__(self, manager: "CacheManager", fn):
+        self._m, self._fn = manager, fn
+
+    def __getitem__(self, req: Hashable) -> int:
+        if req not in self._m._handles:
+            raise KeyError(req)
+        return self._fn(self._m._c, self._m._handles[req])
+
+    def get(self, req: Hashable, default=None):
+        return self[req] if req in self._m._handles else default
+
+    def __contains__(self, req: Hashable) -> bool:
+        return req in self._m._handles
+
+    def __iter__(self):
+        return iter(list(self._m._handles))
+
+    def values(self):
+        return [self[r] for r in list(self._m._handles)]
+
+    def items(self):
+        return [(r, self[r]) for r in list(self._m._handles)]
 
 
 class CacheManager:
@@ -122,115 +186,98 @@ class CacheManager:
     def __init__(self, site_specs: Sequence[StateSpec], page_size: int, n_pages: int, n_slots: int):
         if page_size <= 0 or page_size & (page_size - 1):
             raise ValueError(f"page size must be a power of two, got {page_size}")
+        self._lib = N.host_library()
         self.page_size = page_size
         self.site_specs = list(site_specs)
-        self.groups: List[CacheGroup] = []
+        specs: List[PagedSpec] = []
         self.group_of_site: Dict[int, int] = {}
-        by_spec: Dict[PagedSpec, int] = {}
+        sites_of: List[List[int]] = []
         for site, spec in enumerate(self.site_specs):
             if isinstance(spec, PagedSpec):
-                if spec not in by_spec:
-                    by_spec[spec] = len(self.groups)
-                    self.groups.append(CacheGroup(spec, [], n_pages, page_size))
-                g = by_spec[spec]
-                self.groups[g].sites.append(site)
+                if spec not in specs:
+                    specs.append(spec)
+                    sites_of.append([])
+                g = specs.index(spec)
+                sites_of[g].append(site)
                 self.group_of_site[site] = g
+        windows = (ctypes.c_int32 * max(1, len(specs)))(*[s.window or 0 for s in specs])
+        self._c = self._lib.imparo_cache_new(len(specs), windows, page_size, n_pages, n_slots)
+        if not self._c:
+            raise ValueError("the cache manager refused its sizes")
+        self.groups: List[CacheGroup] = []
+        for g, spec in enumerate(specs):
+            pool = PagePool(0, _borrowed=self._lib.imparo_cache_group_pool(self._c, g))
+            grp = CacheGroup(self, g, spec, pool, page_size)
+            grp.sites = sites_of[g]
+            self.groups.append(grp)
         self.fixed_sites = [s for s, spec in enumerate(self.site_specs) if isinstance(spec, FixedSpec)]
         self.n_slots = n_slots
-        self.slots = PagePool(n_slots)
-        self.slot_of: Dict[Hashable, int] = {}
-        self.length: Dict[Hashable, int] = {}
+        self.slots = PagePool(0, _borrowed=self._lib.imparo_cache_slot_pool(self._c))
+        self._handles: Dict[Hashable, int] = {}
+        self._next_handle = 1
+        self.length = _PerRequest(self, self._lib.imparo_cache_length)
+        self.slot_of = _PerRequest(self, self._lib.imparo_cache_slot)
+        self._scratch = np.empty(1024, dtype=np.int32)
+
+    def __del__(self):
+        if getattr(self, "_c", None):
+            self._lib.imparo_cache_delete(self._c)
+            self._c = None
+
+    def _h(self, req: Hashable) -> int:
+        try:
+            return self._handles[req]
+        except KeyError:
+            raise CacheError(f"request {req!r} is not live") from None
 
     # ------------------------------------------------------------ requests
     def is_live(self, req: Hashable) -> bool:
-        return req in self.slot_of
+        return req in self._handles
 
     def admit(self, req: Hashable) -> int:
         """Takes a state slot for a new request; its tables start empty. The
         caller zeroes the slot's device state."""
-        if req in self.slot_of:
+        if req in self._handles:
             raise CacheError(f"request {req!r} is already live")
-        try:
-            slot = self.slots.alloc()
-        except OutOfPages:
-            raise OutOfPages(f"all {self.n_slots} request slots are in use") from None
-        self.slot_of[req] = slot
-        self.length[req] = 0
-        for g in self.groups:
-            g.tables[req] = []
+        h = self._next_handle
+        slot = self._lib.imparo_cache_admit(self._c, h)
+        if slot == N.E_OUT_OF_PAGES:
+            raise OutOfPages(f"all {self.n_slots} request slots are in use")
+        self._next_handle += 1
+        self._handles[req] = h
         return slot
 
     def release(self, req: Hashable) -> None:
-        if req not in self.slot_of:
-            raise CacheError(f"request {req!r} is not live")
-        for g in self.groups:
-            for page in g.tables.pop(req):
-                if page >= 0:
-                    g.pool.free(page)
-        self.slots.free(self.slot_of.pop(req))
-        del self.length[req]
+        self._lib.imparo_cache_release(self._c, self._h(req))
+        del self._handles[req]
 
     # ------------------------------------------------------------ growth
     def pages_needed(self, req: Hashable, new_length: int) -> List[int]:
         """How many pages each group must add for the request to hold
         positions below `new_length`."""
-        out = []
-        for g in self.groups:
-            table = g.tables[req]
-            total = (new_length + self.page_size - 1) // self.page_size
-            out.append(max(0, total - len(table)))
-        return out
+        out = (ctypes.c_int32 * max(1, len(self.groups)))()
+        self._lib.imparo_cache_pages_needed(self._c, self._h(req), new_length, out)
+        return list(out[:len(self.groups)])
 
-    def reserve(self, req: Hashable, new_length: int) -> List[Tuple[int, int]]:
+    def reserve(self, req: Hashable, new_length: int):
         """Allocates the pages for positions [length, new_length) in every
-        group, all or nothing. Returns what it took, for `rollback`."""
-        if req not in self.slot_of:
-            raise CacheError(f"request {req!r} is not live")
-        if new_length < self.length[req]:
-            raise CacheError(f"request {req!r} cannot shrink from {self.length[req]} to {new_length}")
-        taken: List[Tuple[int, int]] = []
-        try:
-            for gi, g in enumerate(self.groups):
-                table = g.tables[req]
-                total = (new_length + self.page_size - 1) // self.page_size
-                first = g.first_needed_page(self.length[req])
-                while len(table) < total:
-                    if len(table) < first:
-                        table.append(-1)          # wholly behind the window: never needed
-                        taken.append((gi, -1))
-                        continue
-                    page = g.pool.alloc()
-                    table.append(page)
-                    taken.append((gi, page))
-        except OutOfPages:
-            self._undo(req, taken)
+        group, all or nothing. What it took can be given back with `rollback`
+        until the request's next `commit`."""
+        rc = self._lib.imparo_cache_reserve(self._c, self._h(req), new_length)
+        if rc == N.E_OUT_OF_PAGES:
             raise OutOfPages(f"request {req!r} needs pages for {new_length} positions and the pool "
-                             f"has none left") from None
-        return taken
+                             f"has none left")
+        if rc == N.E_SHRINK:
+            raise CacheError(f"request {req!r} cannot shrink from {self.length[req]} to {new_length}")
+        return req
 
-    def _undo(self, req: Hashable, taken: List[Tuple[int, int]]) -> None:
-        for gi, page in reversed(taken):
-            table = self.groups[gi].tables[req]
-            got = table.pop()
-            assert got == page
-            if page >= 0:
-                self.groups[gi].pool.free(page)
-
-    def rollback(self, req: Hashable, taken: List[Tuple[int, int]]) -> None:
-        self._undo(req, taken)
+    def rollback(self, req: Hashable, taken=None) -> None:
+        self._lib.imparo_cache_rollback(self._c, self._h(req))
 
     def commit(self, req: Hashable, new_length: int) -> None:
         """The step ran: the request now holds `new_length` positions. Pages a
         window has passed are given back."""
-        self.length[req] = new_length
-        for g in self.groups:
-            if g.spec.window is None:
-                continue
-            table = g.tables[req]
-            for idx in range(min(g.first_needed_page(new_length), len(table))):
-                if table[idx] >= 0:
-                    g.pool.free(table[idx])
-                    table[idx] = -1
+        self._lib.imparo_cache_commit(self._c, self._h(req), new_length)
 
     def scramble(self, seed: int) -> None:
         for i, g in enumerate(self.groups):
@@ -238,29 +285,56 @@ class CacheManager:
 
     # ------------------------------------------------------------ views
     def table(self, group: int, req: Hashable) -> List[int]:
-        return self.groups[group].tables[req]
+        h = self._h(req)
+        n = self._lib.imparo_cache_table_len(self._c, group, h)
+        if n > self._scratch.shape[0]:
+            self._scratch = np.empty(2 * n, dtype=np.int32)
+        self._lib.imparo_cache_table_copy(self._c, group, h, self._scratch.ctypes.data, self._scratch.shape[0])
+        return self._scratch[:n].tolist()
+
+    def table_len(self, group: int, req: Hashable) -> int:
+        return self._lib.imparo_cache_table_len(self._c, group, self._h(req))
 
     def free_pages(self) -> List[int]:
         return [g.pool.n_free for g in self.groups]
 
     def held_pages(self, req: Hashable) -> List[int]:
-        return [sum(1 for p in g.tables[req] if p >= 0) for g in self.groups]
+        return [sum(1 for p in self.table(g, req) if p >= 0) for g in range(len(self.groups))]
 
     def check(self) -> None:
         """Every page is free or held by exactly one request; raises otherwise."""
-        for gi, g in enumerate(self.groups):
-            seen: Dict[int, Hashable] = {}
-            for req, table in g.tables.items():
-                for page in table:
-                    if page < 0:
-                        continue
-                    if page in seen:
-                        raise CacheError(f"group {gi}: page {page} is held by {seen[page]!r} and {req!r}")
-                    if g.pool.is_free(page):
-                        raise CacheError(f"group {gi}: page {page} is held by {req!r} and free")
-                    seen[page] = req
-            if len(seen) + g.pool.n_free != g.pool.n_pages:
-                raise CacheError(f"group {gi}: {g.pool.n_pages - len(seen) - g.pool.n_free} pages are lost")
-        slots = list(self.slot_of.values())
-        if len(set(slots)) != len(slots) or len(slots) + self.slots.n_free != self.n_slots:
+        rc = self._lib.imparo_cache_check(self._c)
+        if rc == N.E_SHARED_PAGE:
+            raise CacheError("a page is held by two requests, or held and free")
+        if rc == N.E_LOST_PAGE:
+            raise CacheError("pages are lost: neither free nor held")
+        if rc == N.E_SLOTS:
             raise CacheError("state slots are lost or held twice")
+
+    # ------------------------------------------------------------ a step's index arrays
+    LAYOUT = ("T", "R", "W", "G", "P", "n_single", "n_multi", "n_prefill_tiles", "max_seg_len", "max_context", "total")
+
+    def pack(self, requests: Sequence[Hashable], token_lists: Sequence[Sequence[int]],
+             want_lists: Sequence[Sequence[int]], table_width: int = 0) -> Tuple[np.ndarray, Dict[str, int]]:
+        """One int32 array holding everything the kernels index by, laid out
+        tokens | positions | row_of_token | seg_start | seg_len | slot | row
+        lists | want | tables[group][row][page], and the sizes of its parts.
+        Lengths are those before the step."""
+        R = len(requests)
+        reqs = np.fromiter((self._h(r) for r in requests), dtype=np.int64, count=R)
+        n_tok = np.fromiter((len(t) for t in token_lists), dtype=np.int32, count=R)
+        n_want = np.fromiter((len(w) for w in want_lists), dtype=np.int32, count=R)
+        T, W = int(n_tok.sum()), int(n_want.sum())
+        tokens = np.fromiter((t for ts in token_lists for t in ts), dtype=np.int32, count=T)
+        want = np.fromiter((w for ws in want_lists for w in ws), dtype=np.int32, count=W)
+        layout = np.zeros(len(self.LAYOUT), dtype=np.int32)
+        P = table_width if table_width > 0 else max(
+            [1] + [self._lib.imparo_cache_table_len(self._c, g, int(h)) for h in reqs for g in range(len(self.groups))])
+        capacity = 3 * T + 4 * R + W + len(self.groups) * R * P
+        out = np.empty(capacity, dtype=np.int32)
+        n = self._lib.imparo_cache_pack(self._c, R, reqs.ctypes.data, n_tok.ctypes.data, tokens.ctypes.data,
+                                        n_want.ctypes.data, want.ctypes.data, table_width, out.ctypes.data,
+                                        capacity, layout.ctypes.data)
+        if n < 0:
+            raise CacheError(f"packing the step failed with code {n}")
+        return out[:n], dict(zip(self.LAYOUT, layout.tolist()))

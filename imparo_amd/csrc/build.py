@@ -17,6 +17,7 @@ from typing import List
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libimparo_hip.so"
+HOST_LIB_NAME = "libimparo_host.so"     # the host runtime (no GPU code): csrc/host/*.cpp
 ARCH = "gfx950"
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -51,12 +52,41 @@ def _fallback_dir() -> str:
     return os.path.join(tempfile.gettempdir(), f"imparo_amd_build_{os.getuid()}_{tag}")
 
 
-def library_path() -> str:
+def library_path(name: str = LIB_NAME) -> str:
     """The built library: in-tree if it is there, else the fallback location."""
-    in_tree = os.path.join(HERE, LIB_NAME)
+    in_tree = os.path.join(HERE, name)
     if os.path.isfile(in_tree):
         return in_tree
-    return os.path.join(_fallback_dir(), LIB_NAME)
+    return os.path.join(_fallback_dir(), name)
+
+
+def host_library_path() -> str:
+    return library_path(HOST_LIB_NAME)
+
+
+def build_host(verbose: bool = True) -> str:
+    """Compiles the host runtime library with the C++ compiler."""
+    cxx = shutil.which("g++") or shutil.which("c++") or shutil.which("clang++")
+    if cxx is None:
+        for cand in ("/opt/rocm/lib/llvm/bin/clang++", "/opt/rocm/llvm/bin/clang++"):
+            if os.path.isfile(cand):
+                cxx = cand
+    if cxx is None:
+        raise RuntimeError("no C++ compiler was found (g++, c++, clang++); the host runtime cannot be built")
+    out_dir = HERE if _writable(os.path.join(HERE, "_build")) else _fallback_dir()
+    os.makedirs(out_dir, exist_ok=True)
+    src_dir = os.path.join(HERE, "host")
+    srcs = sorted(os.path.join(src_dir, f) for f in os.listdir(src_dir) if f.endswith(".cpp"))
+    lib = os.path.join(out_dir, HOST_LIB_NAME)
+    tmp = lib + f".tmp{os.getpid()}"
+    proc = subprocess.run([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-I", src_dir] + srcs + ["-o", tmp],
+                          stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"building {HOST_LIB_NAME} failed:\n{proc.stderr}")
+    os.replace(tmp, lib)
+    if verbose:
+        _say(f"built {lib}")
+    return lib
 
 
 def _say(msg: str) -> None:
@@ -98,4 +128,5 @@ def build(verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
+    build_host()
     build()

@@ -1,0 +1,74 @@
+// C entry points of the host runtime library: the page allocator, the cache
+// manager (pages, block tables, state slots of every live request) and the
+// packing of a step's index arrays. Nothing here touches the GPU. Requests are
+// named by 64-bit handles the caller chooses. Functions return 0 or a
+// non-negative result on success and a negative IMPARO_E_* code otherwise.
+#pragma once
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define IMPARO_E_OUT_OF_PAGES (-1)   // nothing was changed
+#define IMPARO_E_NOT_LIVE (-2)
+#define IMPARO_E_ALREADY_LIVE (-3)
+#define IMPARO_E_SHRINK (-4)
+#define IMPARO_E_DOUBLE_FREE (-5)
+#define IMPARO_E_RANGE (-6)
+#define IMPARO_E_BUSY (-7)           // the pool is not untouched
+#define IMPARO_E_CAPACITY (-8)       // the output buffer is too small
+#define IMPARO_E_LOST_PAGE (-9)      // check: a page is neither free nor held
+#define IMPARO_E_SHARED_PAGE (-10)   // check: a page is held twice, or held and free
+#define IMPARO_E_SLOTS (-11)         // check: slots lost or held twice
+
+typedef struct ImparoPool ImparoPool;
+typedef struct ImparoCache ImparoCache;
+
+// ---- a pool of pages: the lowest free page first, always
+ImparoPool* imparo_pool_new(int n_pages);
+void imparo_pool_delete(ImparoPool* p);
+int imparo_pool_alloc(ImparoPool* p);                 // page | IMPARO_E_OUT_OF_PAGES
+int imparo_pool_free(ImparoPool* p, int page);        // 0 | IMPARO_E_DOUBLE_FREE | IMPARO_E_RANGE
+int imparo_pool_n_free(const ImparoPool* p);
+int imparo_pool_n_pages(const ImparoPool* p);
+int imparo_pool_high_water(const ImparoPool* p);
+int imparo_pool_is_free(const ImparoPool* p, int page);
+int imparo_pool_scramble(ImparoPool* p, uint64_t seed);   // only while every page is free
+
+// ---- the cache manager: n_groups paged groups (window 0 = keep every position), n_slots state slots
+ImparoCache* imparo_cache_new(int n_groups, const int32_t* windows, int page_size, int n_pages, int n_slots);
+void imparo_cache_delete(ImparoCache* c);
+ImparoPool* imparo_cache_group_pool(ImparoCache* c, int group);
+ImparoPool* imparo_cache_slot_pool(ImparoCache* c);
+int imparo_cache_admit(ImparoCache* c, int64_t req);                     // slot | E_ALREADY_LIVE | E_OUT_OF_PAGES (no slot)
+int imparo_cache_release(ImparoCache* c, int64_t req);
+// pages for positions below new_length in every group, all or nothing; what it took stays
+// revocable (imparo_cache_rollback) until the next commit of the request
+int imparo_cache_reserve(ImparoCache* c, int64_t req, int new_length);
+int imparo_cache_rollback(ImparoCache* c, int64_t req);
+int imparo_cache_commit(ImparoCache* c, int64_t req, int new_length);    // pages a window has passed are given back
+int imparo_cache_is_live(const ImparoCache* c, int64_t req);
+int imparo_cache_length(const ImparoCache* c, int64_t req);
+int imparo_cache_slot(const ImparoCache* c, int64_t req);
+int imparo_cache_table_len(const ImparoCache* c, int group, int64_t req);
+int imparo_cache_table_copy(const ImparoCache* c, int group, int64_t req, int32_t* out, int capacity);
+int imparo_cache_pages_needed(const ImparoCache* c, int64_t req, int new_length, int32_t* per_group);
+int imparo_cache_first_needed_page(const ImparoCache* c, int group, int next_position);
+int imparo_cache_n_live(const ImparoCache* c);
+int imparo_cache_live_requests(const ImparoCache* c, int64_t* out, int capacity);
+int imparo_cache_check(const ImparoCache* c);
+
+// ---- a step's index arrays, packed for one host-to-device copy.
+// Layout (int32): tokens[T] | positions[T] | row_of_token[T] | seg_start[R] | seg_len[R] | slot[R] |
+// row lists[R] (rows with one token first, then the others) | want[W] | tables[G][R][P].
+// P = table_width, or the widest table of the batch if table_width is 0. `layout` receives
+// {T, R, W, G, P, n_single, n_multi, n_prefill_tiles, max_seg_len, max_context, total}.
+// Returns the number of int32 written, or a negative code; lengths are those before the step.
+int64_t imparo_cache_pack(const ImparoCache* c, int n_rows, const int64_t* reqs, const int32_t* n_tokens,
+                          const int32_t* tokens, const int32_t* n_want, const int32_t* want, int table_width,
+                          int32_t* out, int64_t capacity, int32_t* layout);
+
+#ifdef __cplusplus
+}
+#endif

@@ -201,7 +201,7 @@ class Engine:
         launch by launch (so that every kernel it needs has been loaded), the
         second is captured, later ones replay the capture."""
         G = len(self.cache.groups)
-        widest = max([len(self.cache.table(g, e.request)) for e in entries for g in range(G)] or [1])
+        widest = max([self.cache.table_len(g, e.request) for e in entries for g in range(G)] or [1])
         width = -(-widest // TABLE_BUCKET) * TABLE_BUCKET
         key = (len(entries), width)
         g = self._graphs.setdefault(key, _DecodeGraph())
@@ -229,47 +229,16 @@ class Engine:
         """Builds the step's index arrays, sends them to the device in one
         copy and wraps them in a StepContext. For a captured step the arrays go
         to the capture's own fixed buffer and sizes are the capture's bounds."""
-        R = len(entries)
-        T = sum(len(e.tokens) for e in entries)
-        G = len(self.cache.groups)
-        lengths = [self.cache.length[e.request] for e in entries]
-        P = max(1, max(len(self.cache.table(g, e.request)) for e in entries for g in range(G)) if G else 1)
-        if table_width is not None:
-            P = table_width
-        W = sum(len(e.want) for e in entries)
-        # layout: tokens | positions | row_of_token | seg_start | seg_len | slot | row lists | want | tables[G][R][P]
-        total = 3 * T + 4 * R + W + G * R * P
-        a = np.empty(total, dtype=np.int32)
-        o_tok, o_pos, o_row = 0, T, 2 * T
+        a, lay = self.cache.pack([e.request for e in entries], [e.tokens for e in entries],
+                                 [e.want for e in entries], table_width or 0)
+        T, R, W, G, P, total = lay["T"], lay["R"], lay["W"], lay["G"], lay["P"], lay["total"]
+        o_pos, o_row = T, 2 * T
         o_start, o_len, o_slot = 3 * T, 3 * T + R, 3 * T + 2 * R
         o_lists = 3 * T + 3 * R
         o_want = 3 * T + 4 * R
         o_tab = o_want + W
-        t = 0
-        w = 0
-        for r, e in enumerate(entries):
-            n = len(e.tokens)
-            a[o_tok + t:o_tok + t + n] = np.asarray(e.tokens, dtype=np.int32)
-            a[o_pos + t:o_pos + t + n] = np.arange(lengths[r], lengths[r] + n, dtype=np.int32)
-            a[o_row + t:o_row + t + n] = r
-            a[o_start + r] = t
-            a[o_len + r] = n
-            a[o_slot + r] = self.cache.slot_of[e.request]
-            for wi in e.want:
-                a[o_want + w] = t + int(wi)
-                w += 1
-            t += n
-        # rows with one token first, rows with a portion after them
-        dec = [r for r, e in enumerate(entries) if len(e.tokens) == 1]
-        pre = [r for r, e in enumerate(entries) if len(e.tokens) > 1]
-        a[o_lists:o_lists + R] = np.asarray(dec + pre, dtype=np.int32)
-        tables = a[o_tab:].reshape(G, R, P) if G else None
-        if G:
-            tables.fill(-1)
-            for g in range(G):
-                for r, e in enumerate(entries):
-                    tab = self.cache.table(g, e.request)
-                    tables[g, r, :len(tab)] = tab
+        o_tok = 0
+        n_dec = lay["n_single"]
         if graph is not None:
             if graph.meta is None:
                 graph.meta = torch.empty(total, dtype=torch.int32, device=self.device)
@@ -283,12 +252,11 @@ class Engine:
             seg_start=dev[o_start:o_start + R], seg_len=dev[o_len:o_len + R], slot=dev[o_slot:o_slot + R],
             block_tables=block_tables, page_size=self.page_size, dtype=self.dtype,
             workspace=workspace or self.workspace, storage=self.storage, group_of_site=self.cache.group_of_site,
-            max_seg_len=max(len(e.tokens) for e in entries),
-            max_context=(max(lengths[r] + len(e.tokens) for r, e in enumerate(entries)) if table_width is None
-                         else table_width * self.page_size),
-            decode_rows=dev[o_lists:o_lists + len(dec)], n_decode_rows=len(dec),
-            prefill_rows=dev[o_lists + len(dec):o_lists + R], n_prefill_rows=len(pre),
-            n_prefill_tiles=sum((len(entries[r].tokens) + 63) // 64 for r in pre),
+            max_seg_len=lay["max_seg_len"],
+            max_context=lay["max_context"] if table_width is None else table_width * self.page_size,
+            decode_rows=dev[o_lists:o_lists + n_dec], n_decode_rows=n_dec,
+            prefill_rows=dev[o_lists + n_dec:o_lists + R], n_prefill_rows=lay["n_multi"],
+            n_prefill_tiles=lay["n_prefill_tiles"],
         )
         want_rows = dev[o_want:o_want + W] if W else None
         return ctx, dev[o_tok:o_tok + T], want_rows
