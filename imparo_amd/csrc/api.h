@@ -16,9 +16,10 @@ int imparo_embed_gather(const void* table, int table_dtype, const int32_t* ids, 
                         int n_tokens, int width, int vocab, imparo_stream stream);
 
 // Row-wise RMS norm. For output row i the source row is rows ? rows[i] : i.
-// If delta is given the row is x + delta first; with write_back (rows must be
-// null) the sum is stored to x. out[i, :] = v * rsqrt(mean(v^2) + eps) * weight.
-int imparo_rms_norm(float* x, const float* delta, const int32_t* rows, const float* weight,
+// If delta is given the row is x + delta[0] + delta[1] + ... first (n_delta
+// slices, each [n_x_rows, width], added in order); with write_back (rows must
+// be null) the sum is stored to x. out[i, :] = v * rsqrt(mean(v^2) + eps) * weight.
+int imparo_rms_norm(float* x, const float* delta, int n_delta, int n_x_rows, const int32_t* rows, const float* weight,
                     void* out, int out_dtype, int n_rows, int width, float eps, int write_back,
                     imparo_stream stream);
 
@@ -33,8 +34,12 @@ int imparo_add_bias(float* y, const float* bias, int m, int n, imparo_stream str
 // accumulate. X and W share `dtype`. epilogue 0: Y is [m, n]. epilogue 1
 // (SwiGLU): W's rows alternate gate, up; Y is [m, n/2] with
 // Y[m, j] = silu(y[m, 2j]) * y[m, 2j+1].
+// `slices` > 1 (only the number imparo_gemm_slices gives, float32 out, epilogue 0): K is cut into
+// that many slices and Y is [slices, m, n], slice s holding the sum over its part of K (the bias
+// in slice 0); the consumer adds the slices in order.
 int imparo_gemm(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
-                int m, int n, int k, int epilogue, imparo_stream stream);
+                int m, int n, int k, int epilogue, int slices, imparo_stream stream);
+int imparo_gemm_slices(int m, int n, int k, int dtype);
 
 // Per (token, head): RMS norm over the head (weight null: none), NeoX rotation
 // with angles pos * inv_freq[i] over the first 2*n_freq dims (n_freq 0: none).

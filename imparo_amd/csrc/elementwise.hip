@@ -34,7 +34,7 @@ extern "C" int imparo_embed_gather(const void* table, int table_dtype, const int
 // fixed by the block size. Two passes over the row; the second re-reads what
 // the first left in registers when the row fits (width <= 8 * blockDim).
 template <typename TOut, int PER_THREAD>
-__global__ void k_rms_norm(float* __restrict__ x, const float* __restrict__ delta,
+__global__ void k_rms_norm(float* __restrict__ x, const float* __restrict__ delta, int n_delta, size_t delta_stride,
                            const int32_t* __restrict__ rows, const float* __restrict__ weight,
                            TOut* __restrict__ out, int width, float eps, int write_back) {
     __shared__ float scratch[16];
@@ -49,7 +49,9 @@ __global__ void k_rms_norm(float* __restrict__ x, const float* __restrict__ delt
         float a = 0.f;
         if (i < width) {
             a = x[src + i];
-            if (delta) a += delta[src + i];
+            float d = 0.f;                   // the slices make up the delta first, then the delta joins x
+            for (int s = 0; s < n_delta; ++s) d += delta[s * delta_stride + src + i];
+            a += d;
             if (write_back) x[src + i] = a;
         }
         v[j] = a;
@@ -57,8 +59,9 @@ __global__ void k_rms_norm(float* __restrict__ x, const float* __restrict__ delt
     }
     // rows wider than PER_THREAD * blockDim: the tail is not kept in registers
     for (int i = threadIdx.x + PER_THREAD * blockDim.x; i < width; i += blockDim.x) {
-        float a = x[src + i];
-        if (delta) a += delta[src + i];
+        float a = x[src + i], d = 0.f;
+        for (int s = 0; s < n_delta; ++s) d += delta[s * delta_stride + src + i];
+        a += d;
         if (write_back) x[src + i] = a;
         ss += a * a;
     }
@@ -71,7 +74,11 @@ __global__ void k_rms_norm(float* __restrict__ x, const float* __restrict__ delt
     }
     for (int i = threadIdx.x + PER_THREAD * blockDim.x; i < width; i += blockDim.x) {
         float a = x[src + i];
-        if (delta && !write_back) a += delta[src + i];
+        if (!write_back) {
+            float d = 0.f;
+            for (int s = 0; s < n_delta; ++s) d += delta[s * delta_stride + src + i];
+            a += d;
+        }
         store_f32<TOut>(out, dst + i, a * scale * weight[i]);
     }
 }
@@ -79,7 +86,7 @@ __global__ void k_rms_norm(float* __restrict__ x, const float* __restrict__ delt
 // The same for rows whose width is a multiple of 4 and at most 4 * blockDim:
 // one float4 per thread, every load of the row issued before anything waits.
 template <typename TOut>
-__global__ void k_rms_norm_v4(float* __restrict__ x, const float* __restrict__ delta,
+__global__ void k_rms_norm_v4(float* __restrict__ x, const float* __restrict__ delta, int n_delta, size_t delta_stride,
                               const int32_t* __restrict__ rows, const float* __restrict__ weight,
                               TOut* __restrict__ out, int width, float eps, int write_back) {
     __shared__ float scratch[16];
@@ -92,13 +99,18 @@ __global__ void k_rms_norm_v4(float* __restrict__ x, const float* __restrict__ d
     if (in) {
         a = *reinterpret_cast<const float4*>(x + src + i);
         w = *reinterpret_cast<const float4*>(weight + i);
-        if (delta) {
-            const float4 d = *reinterpret_cast<const float4*>(delta + src + i);
-            a.x += d.x;
-            a.y += d.y;
-            a.z += d.z;
-            a.w += d.w;
+        float4 d = make_float4(0.f, 0.f, 0.f, 0.f);   // the slices make up the delta first, then the delta joins x
+        for (int s = 0; s < n_delta; ++s) {
+            const float4 p = *reinterpret_cast<const float4*>(delta + s * delta_stride + src + i);
+            d.x += p.x;
+            d.y += p.y;
+            d.z += p.z;
+            d.w += p.w;
         }
+        a.x += d.x;
+        a.y += d.y;
+        a.z += d.z;
+        a.w += d.w;
         if (write_back) *reinterpret_cast<float4*>(x + src + i) = a;
     }
     // the same order of squares as the scalar kernel would not matter: each kernel is
@@ -114,10 +126,13 @@ __global__ void k_rms_norm_v4(float* __restrict__ x, const float* __restrict__ d
     }
 }
 
-extern "C" int imparo_rms_norm(float* x, const float* delta, const int32_t* rows, const float* weight,
-                               void* out, int out_dtype, int n_rows, int width, float eps, int write_back,
-                               imparo_stream stream) {
+extern "C" int imparo_rms_norm(float* x, const float* delta, int n_delta, int n_x_rows, const int32_t* rows,
+                               const float* weight, void* out, int out_dtype, int n_rows, int width, float eps,
+                               int write_back, imparo_stream stream) {
     if (!x || !weight || !out || n_rows < 0 || width <= 0) return IMPARO_BAD_ARGUMENT;
+    if (n_delta < 0 || n_delta > 64 || (n_delta > 0 && !delta) || n_x_rows < 0) return IMPARO_BAD_ARGUMENT;
+    if (!delta) n_delta = 0;
+    const size_t delta_stride = (size_t)n_x_rows * width;
     if (write_back && rows) return IMPARO_BAD_ARGUMENT;
     if (n_rows == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;
@@ -125,18 +140,22 @@ extern "C" int imparo_rms_norm(float* x, const float* delta, const int32_t* rows
     if (width % 4 == 0 && width >= 512 && width <= 4096 && aligned) {
         const int threads = ((width / 4) + 63) / 64 * 64;
         if (out_dtype == IMPARO_F32)
-            k_rms_norm_v4<float><<<n_rows, threads, 0, s>>>(x, delta, rows, weight, (float*)out, width, eps, write_back);
+            k_rms_norm_v4<float><<<n_rows, threads, 0, s>>>(x, delta, n_delta, delta_stride, rows, weight, (float*)out, width, eps,
+                                                            write_back);
         else if (out_dtype == IMPARO_BF16)
-            k_rms_norm_v4<bf16_t><<<n_rows, threads, 0, s>>>(x, delta, rows, weight, (bf16_t*)out, width, eps, write_back);
+            k_rms_norm_v4<bf16_t><<<n_rows, threads, 0, s>>>(x, delta, n_delta, delta_stride, rows, weight, (bf16_t*)out, width,
+                                                             eps, write_back);
         else
             return IMPARO_BAD_ARGUMENT;
         return launch_status();
     }
     const int threads = width <= 256 ? 64 : 256;
     if (out_dtype == IMPARO_F32)
-        k_rms_norm<float, 8><<<n_rows, threads, 0, s>>>(x, delta, rows, weight, (float*)out, width, eps, write_back);
+        k_rms_norm<float, 8><<<n_rows, threads, 0, s>>>(x, delta, n_delta, delta_stride, rows, weight, (float*)out, width, eps,
+                                                        write_back);
     else if (out_dtype == IMPARO_BF16)
-        k_rms_norm<bf16_t, 8><<<n_rows, threads, 0, s>>>(x, delta, rows, weight, (bf16_t*)out, width, eps, write_back);
+        k_rms_norm<bf16_t, 8><<<n_rows, threads, 0, s>>>(x, delta, n_delta, delta_stride, rows, weight, (bf16_t*)out, width, eps,
+                                                         write_back);
     else
         return IMPARO_BAD_ARGUMENT;
     return launch_status();

@@ -261,20 +261,28 @@ struct SkinnyFrags {
     Frag8 x[MT][4];
 };
 
+// With slices (gridDim.y > 1) block (x, y) sums only K range [y * k_per, (y+1) * k_per) and
+// writes it to Y + y * M * N: the consumer adds the slices in order.
 template <typename TOut, int MT, int NW>
 __global__ __launch_bounds__(NW * 64) void k_gemm_bf16_skinny(const bf16_t* __restrict__ X,
                                                               const bf16_t* __restrict__ W,
                                                               const float* __restrict__ bias,
-                                                              TOut* __restrict__ Y, int M, int N, int K,
-                                                              int epilogue) {
+                                                              TOut* __restrict__ Y, int M, int N, int K_all,
+                                                              int k_per, int epilogue) {
     __shared__ float red[NW][MT][64][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0 = blockIdx.x * 16;
+    const int k_lo = blockIdx.y * k_per;
+    const int K = min(K_all, k_lo + k_per) - k_lo;       // this block's part of K, re-based to 0
+    X += k_lo;
+    W += k_lo;
+    Y += (size_t)blockIdx.y * M * N;
+    if (blockIdx.y > 0) bias = nullptr;                  // the bias belongs to one slice only
     const int r16 = lane & 15, g = lane >> 4;
-    const bf16_t* wrow = W + (size_t)min(n0 + r16, N - 1) * K + g * 8;
+    const bf16_t* wrow = W + (size_t)min(n0 + r16, N - 1) * K_all + g * 8;
     const bf16_t* xrow[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) xrow[mt] = X + (size_t)min(mt * 16 + r16, M - 1) * K + g * 8;
+    for (int mt = 0; mt < MT; ++mt) xrow[mt] = X + (size_t)min(mt * 16 + r16, M - 1) * K_all + g * 8;
     f32x4 acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -347,17 +355,26 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_bf16_skinny(const bf16_t* __re
 
 template <typename TOut, int MT>
 static void launch_skinny(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k,
-                          int epilogue, hipStream_t s) {
-    const unsigned blocks = (unsigned)((n + 15) / 16);
-    // few chunks of 128 per wave: 4 waves up to K = 512, 8 up to 2048, 16 beyond
-    if (k <= 512)
-        k_gemm_bf16_skinny<TOut, MT, 4><<<blocks, 4 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
-    else if (k <= 2048)
-        k_gemm_bf16_skinny<TOut, MT, 8><<<blocks, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+                          int epilogue, int slices, hipStream_t s) {
+    const int k_per = ((k + slices - 1) / slices + 127) / 128 * 128;
+    dim3 grid((unsigned)((n + 15) / 16), (unsigned)((k + k_per - 1) / k_per));
+    // few chunks of 128 per wave: 4 waves up to 512 of K per block, 8 up to 2048, 16 beyond
+    if (k_per <= 512)
+        k_gemm_bf16_skinny<TOut, MT, 4><<<grid, 4 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
+    else if (k_per <= 2048)
+        k_gemm_bf16_skinny<TOut, MT, 8><<<grid, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
     else if (MT <= 2)
-        k_gemm_bf16_skinny<TOut, MT, 16><<<blocks, 16 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+        k_gemm_bf16_skinny<TOut, MT, 16><<<grid, 16 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
     else   // 64 activation rows keep too many fragments in registers for 1024 threads
-        k_gemm_bf16_skinny<TOut, MT, 8><<<blocks, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+        k_gemm_bf16_skinny<TOut, MT, 8><<<grid, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
+}
+
+// Into how many slices of K a few-row product may be cut when its consumer adds the slices:
+// a weight with few rows and a long K (the feed-forward's way back) gives too few blocks
+// otherwise. One slice per 2048 of K, for at most 64 rows and at most 4096 weight rows.
+extern "C" int imparo_gemm_slices(int m, int n, int k, int dtype) {
+    if (dtype != IMPARO_BF16 || m > 64 || n > 4096 || k < 4096) return 1;
+    return (k + 2047) / 2048;
 }
 
 // ------------------------------------------------------------------ bfloat16, few rows, many weight rows
@@ -489,11 +506,11 @@ static void launch_stream(const bf16_t* x, const bf16_t* w, const float* bias, T
 
 template <typename TOut>
 static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
-                       int force, hipStream_t s) {
+                       int force, int slices, hipStream_t s) {
     // 17..64 rows: sharing the activations between the waves of a block matters more than anything
     // else, if the weight has rows enough for enough blocks. (Up to 16 rows the K-split kernel keeps
     // more loads in flight and wins.) `force` (for measurements): 1 = K-split kernel, 2/4/8 = wide with that many waves
-    int nw = (m > 16) ? stream_waves(n) : 0;
+    int nw = (m > 16 && slices == 1) ? stream_waves(n) : 0;
     if (force == 1) nw = 0;
     if (force == 2 || force == 4 || force == 8) nw = force;
     if (m <= 64 && nw) {
@@ -507,11 +524,11 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
     }
     if (m <= 64) {
         if (m <= 16)
-            launch_skinny<TOut, 1>(x, w, bias, y, m, n, k, epilogue, s);
+            launch_skinny<TOut, 1>(x, w, bias, y, m, n, k, epilogue, slices, s);
         else if (m <= 32)
-            launch_skinny<TOut, 2>(x, w, bias, y, m, n, k, epilogue, s);
+            launch_skinny<TOut, 2>(x, w, bias, y, m, n, k, epilogue, slices, s);
         else
-            launch_skinny<TOut, 4>(x, w, bias, y, m, n, k, epilogue, s);
+            launch_skinny<TOut, 4>(x, w, bias, y, m, n, k, epilogue, slices, s);
     } else {
         const int tiles_m = (m + BG_BM - 1) / BG_BM, tiles_n = (n + BG_BN - 1) / BG_BN;
         const long long total = (long long)tiles_m * tiles_n;
@@ -529,8 +546,12 @@ static int g_force_few_row_kernel = 0;
 extern "C" void imparo_gemm_force_kernel(int which) { g_force_few_row_kernel = which; }
 
 extern "C" int imparo_gemm(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
-                           int m, int n, int k, int epilogue, imparo_stream stream) {
+                           int m, int n, int k, int epilogue, int slices, imparo_stream stream) {
     if (!x || !w || !y || m < 0 || n <= 0 || k <= 0) return IMPARO_BAD_ARGUMENT;
+    if (slices < 1) return IMPARO_BAD_ARGUMENT;
+    // slices: only what imparo_gemm_slices allows, float32 out, no epilogue that is not linear
+    if (slices > 1 && (slices != imparo_gemm_slices(m, n, k, dtype) || out_dtype != IMPARO_F32 || epilogue != EPI_NONE))
+        return IMPARO_BAD_ARGUMENT;
     if (epilogue != EPI_NONE && epilogue != EPI_SWIGLU) return IMPARO_BAD_ARGUMENT;
     if (epilogue == EPI_SWIGLU && (n % 2 != 0)) return IMPARO_BAD_ARGUMENT;
     if (m == 0) return IMPARO_OK;
@@ -551,9 +572,9 @@ extern "C" int imparo_gemm(const void* x, const void* w, const float* bias, void
     if (k % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return IMPARO_BAD_ARGUMENT;
     if (out_dtype == IMPARO_F32)
         return launch_bf16<float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)y, m, n, k, epilogue,
-                                  g_force_few_row_kernel, s);
+                                  g_force_few_row_kernel, slices, s);
     if (out_dtype == IMPARO_BF16)
         return launch_bf16<bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)y, m, n, k, epilogue,
-                                   g_force_few_row_kernel, s);
+                                   g_force_few_row_kernel, slices, s);
     return IMPARO_BAD_ARGUMENT;
 }

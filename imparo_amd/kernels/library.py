@@ -22,10 +22,11 @@ F = c_float
 
 _SIGNATURES = {
     "imparo_embed_gather": [P, I, P, P, I, I, I, P],
-    "imparo_rms_norm": [P, P, P, P, P, I, I, I, F, I, P],
+    "imparo_rms_norm": [P, P, I, I, P, P, P, I, I, I, F, I, P],
     "imparo_silu_mul": [P, I, P, I, I, I, P],
     "imparo_add_bias": [P, P, I, I, P],
-    "imparo_gemm": [P, P, P, P, I, I, I, I, I, I, P],
+    "imparo_gemm": [P, P, P, P, I, I, I, I, I, I, I, P],
+    "imparo_gemm_slices": [I, I, I, I],
     "imparo_short_conv_decode": [P, P, P, P, P, P, I, I, I, I, I, P],
     "imparo_qk_norm_rope_store": [P, P, P, F, P, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, P],
     "imparo_attention": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, P],

@@ -70,6 +70,7 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tenso
              delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
              write_back: bool = False) -> torch.Tensor:
     """out[i] = norm(x[src] (+ delta[src])) * weight, src = rows[i] or i.
+    `delta` is shaped like x, or [slices, *x.shape]: slices are added in order.
     write_back stores x + delta into x (only without rows)."""
     width = x.shape[-1]
     n_out = out.shape[0]
@@ -79,8 +80,13 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tenso
         raise KernelArgumentError("rms_norm: one source row index per output row is needed")
     if write_back and (rows is not None or delta is None):
         raise KernelArgumentError("rms_norm: write_back needs a delta and no row selection")
+    n_delta = 0
+    if delta is not None:
+        n_delta = delta.shape[0] if delta.dim() == x.dim() + 1 else 1
+        want = (n_delta,) + tuple(x.shape) if delta.dim() == x.dim() + 1 else tuple(x.shape)
+        _dev(delta, "rms_norm delta", torch.float32, want)
     _check(library().imparo_rms_norm(
-        _dev(x, "rms_norm x", torch.float32), _dev(delta, "rms_norm delta", torch.float32, x.shape),
+        _dev(x, "rms_norm x", torch.float32), _dev(delta, "rms_norm delta", torch.float32), n_delta, x.shape[0],
         _dev(rows, "rms_norm rows", torch.int32), _dev(weight, "rms_norm weight", torch.float32, (width,)),
         _dev(out, "rms_norm out", None, (n_out, width)), _code(out, "rms_norm out"),
         n_out, width, float(eps), int(write_back), _stream()), "rms_norm")
@@ -107,11 +113,17 @@ def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
     return y
 
 
+def gemm_slices(m: int, n: int, k: int, dtype: torch.dtype) -> int:
+    """Into how many slices of K this product may be cut when its consumer adds the slices (1: none)."""
+    return int(library().imparo_gemm_slices(m, n, k, _CODES.get(dtype, -1)))
+
+
 def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
          swiglu: bool = False) -> torch.Tensor:
     """out[m, n] = x[m, k] . w[n, k]^T (+ bias[n]); x and w share a dtype; float32
     accumulate. With `swiglu` the rows of w alternate gate and up and out is
-    [m, n/2] = silu(gate) * up."""
+    [m, n/2] = silu(gate) * up. An `out` of shape [slices, m, n] (slices =
+    gemm_slices(...)) receives the sums over slices of K, to be added by the consumer."""
     m, k = x.shape
     n, kw = w.shape
     if kw != k:
@@ -122,9 +134,17 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[tor
         raise KernelArgumentError(f"gemm: the bfloat16 kernels need the inner size to be a multiple of 8, got {k}")
     if swiglu and n % 2:
         raise KernelArgumentError("gemm: a gate/up weight has an even number of rows")
+    slices = 1
+    if out.dim() == 3:
+        slices = out.shape[0]
+        if slices != gemm_slices(m, n, k, x.dtype) or swiglu or out.dtype != torch.float32:
+            raise KernelArgumentError(f"gemm: this product cannot be cut into {slices} slices of K")
+        _dev(out, "gemm out", torch.float32, (slices, m, n))
+    else:
+        _dev(out, "gemm out", None, (m, n // 2 if swiglu else n))
     _check(library().imparo_gemm(_dev(x, "gemm x"), _dev(w, "gemm weight"), _dev(bias, "gemm bias", torch.float32, (n,)),
-                                 _dev(out, "gemm out", None, (m, n // 2 if swiglu else n)),
-                                 _code(x, "gemm x"), _code(out, "gemm out"), m, n, k, int(swiglu), _stream()), "gemm")
+                                 out.data_ptr(), _code(x, "gemm x"), _code(out, "gemm out"), m, n, k, int(swiglu),
+                                 slices, _stream()), "gemm")
     return out
 
 

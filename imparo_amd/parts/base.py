@@ -83,6 +83,8 @@ class StepContext:
 @dataclass
 class Residual:
     """The residual stream in float32 and a delta not yet added to it. The
-    next norm adds the delta while it reads the row anyway."""
+    next norm adds the delta while it reads the row anyway. The delta is
+    shaped like x, or [slices, *x.shape]: sums over parts of a projection's
+    inner dimension, which the norm adds up in order."""
     x: torch.Tensor
     pending: Optional[torch.Tensor] = None

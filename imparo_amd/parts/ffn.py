@@ -55,7 +55,8 @@ class SwiGlu:
 
     def forward(self, ctx: StepContext, n: torch.Tensor) -> torch.Tensor:
         g = self.gate_up(ctx, n, self.down.in_dtype, "gated", swiglu=True)
-        return self.down(ctx, g, torch.float32, "ffn_out")
+        # the result is a delta for the residual stream, whose next norm adds slices: it may come sliced
+        return self.down(ctx, g, torch.float32, "ffn_out", sliced_ok=True)
 
 
 register_part("feed_forward", "swiglu", SwiGlu)

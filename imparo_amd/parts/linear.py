@@ -28,11 +28,19 @@ class Linear:
         return self.weight.dtype
 
     def __call__(self, ctx: StepContext, x: torch.Tensor, out_dtype: torch.dtype, name: str,
-                 swiglu: bool = False) -> torch.Tensor:
+                 swiglu: bool = False, sliced_ok: bool = False) -> torch.Tensor:
         """`swiglu`: the weight's rows alternate gate and up; the output is
-        silu(gate) * up, half as wide."""
+        silu(gate) * up, half as wide. `sliced_ok`: the caller's consumer adds
+        slices, so the result may come as [slices, rows, out] sums over parts
+        of K (few rows and a long K keep more of the chip busy that way)."""
         width = self.out_features // 2 if swiglu else self.out_features
-        out = ctx.workspace.get(name, (x.shape[0], width), out_dtype)
+        m = x.shape[0]
+        if sliced_ok and not swiglu and out_dtype == torch.float32:
+            slices = ops.gemm_slices(m, self.out_features, self.in_features, self.weight.dtype)
+            if slices > 1:
+                out = ctx.workspace.get(name + "_sliced", (slices, m, width), out_dtype)
+                return ops.gemm(x, self.weight, out, bias=self.bias)
+        out = ctx.workspace.get(name, (m, width), out_dtype)
         return ops.gemm(x, self.weight, out, bias=self.bias, swiglu=swiglu)
 
 

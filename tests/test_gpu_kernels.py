@@ -76,6 +76,40 @@ def test_gemm_epilogues(m):
                                rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("m", [1, 9, 40, 64])
+def test_gemm_in_slices_of_k_and_the_norm_that_adds_them(m):
+    """A few-row product over a long K may leave its result as sums over slices of K, which the
+    norm that consumes it adds up in order."""
+    n, k = 200, 4096 + 264
+    x, w, b = rnd(m, k, seed=1).to(torch.bfloat16), rnd(n, k, seed=2, scale=0.1).to(torch.bfloat16), rnd(n, seed=3)
+    slices = ops().gemm_slices(m, n, k, torch.bfloat16)
+    assert slices == 3 and ops().gemm_slices(m, n, 2048, torch.bfloat16) == 1
+    assert ops().gemm_slices(65, n, k, torch.bfloat16) == 1 and ops().gemm_slices(m, n, k, torch.float32) == 1
+    out = torch.full((slices, m, n), float("nan"), device=DEV)
+    ops().gemm(x.to(DEV), w.to(DEV), out, bias=b.to(DEV))
+    ref = x.double() @ w.double().t() + b.double()
+    torch.testing.assert_close(out.cpu().double().sum(0), ref, rtol=1e-5, atol=1e-5)
+    whole = torch.empty(m, n, device=DEV)
+    ops().gemm(x.to(DEV), w.to(DEV), whole, bias=b.to(DEV))
+    torch.testing.assert_close(out.sum(0), whole, rtol=1e-5, atol=1e-5)
+    # the norm takes the slices as its delta
+    res = rnd(m, n, seed=4)
+    wn = 1 + 0.1 * rnd(n, seed=5)
+    xd = res.to(DEV).clone()
+    normed = torch.empty(m, n, device=DEV)
+    ops().rms_norm(xd, wn.to(DEV), 1e-5, normed, delta=out, write_back=True)
+    total = res + out.cpu().sum(0)
+    torch.testing.assert_close(xd.cpu(), total, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(normed.cpu(), P.rms_norm(total, wn, 1e-5), rtol=1e-5, atol=1e-5)
+    rows = torch.tensor([m - 1, 0], dtype=torch.int32, device=DEV)
+    picked = torch.empty(2, n, device=DEV)
+    ops().rms_norm(res.to(DEV), wn.to(DEV), 1e-5, picked, delta=out, rows=rows)
+    torch.testing.assert_close(picked.cpu(), P.rms_norm(total[[m - 1, 0]], wn, 1e-5), rtol=1e-5, atol=1e-5)
+    from imparo_amd.kernels import KernelArgumentError
+    with pytest.raises(KernelArgumentError, match="slices"):
+        ops().gemm(x.to(DEV), w.to(DEV), torch.empty(2, m, n, device=DEV))
+
+
 def test_gemm_refuses_what_it_cannot_take():
     from imparo_amd.kernels import KernelArgumentError
     x, w = rnd(4, 12).to(torch.bfloat16).to(DEV), rnd(8, 12).to(torch.bfloat16).to(DEV)
