@@ -112,16 +112,16 @@ class _Tables:
         return self._m.table(self._g, req)
 
     def __iter__(self) -> Iterator[Hashable]:
-        return iter(list(self._m._handles))
+        return iter(self._m._live_names())
 
     def __len__(self) -> int:
-        return len(self._m._handles)
+        return len(self._m._live_names())
 
     def __contains__(self, req: Hashable) -> bool:
-        return req in self._m._handles
+        return self._m.is_live(req)
 
     def keys(self):
-        return list(self._m._handles)
+        return self._m._live_names()
 
     def values(self):
         return [self[r] for r in self.keys()]
@@ -154,24 +154,24 @@ class _PerRequest:
         self._m, self._fn = manager, fn
 
     def __getitem__(self, req: Hashable) -> int:
-        if req not in self._m._handles:
+        if not self._m.is_live(req):
             raise KeyError(req)
         return self._fn(self._m._c, self._m._handles[req])
 
     def get(self, req: Hashable, default=None):
-        return self[req] if req in self._m._handles else default
+        return self[req] if self._m.is_live(req) else default
 
     def __contains__(self, req: Hashable) -> bool:
-        return req in self._m._handles
+        return self._m.is_live(req)
 
     def __iter__(self):
-        return iter(list(self._m._handles))
+        return iter(self._m._live_names())
 
     def values(self):
-        return [self[r] for r in list(self._m._handles)]
+        return [self[r] for r in self._m._live_names()]
 
     def items(self):
-        return [(r, self[r]) for r in list(self._m._handles)]
+        return [(r, self[r]) for r in self._m._live_names()]
 
 
 class CacheManager:
@@ -214,6 +214,7 @@ class CacheManager:
         self.n_slots = n_slots
         self.slots = PagePool(0, _borrowed=self._lib.imparo_cache_slot_pool(self._c))
         self._handles: Dict[Hashable, int] = {}
+        self._names: Dict[int, Hashable] = {}
         self._next_handle = 1
         self.length = _PerRequest(self, self._lib.imparo_cache_length)
         self.slot_of = _PerRequest(self, self._lib.imparo_cache_slot)
@@ -225,31 +226,52 @@ class CacheManager:
             self._c = None
 
     def _h(self, req: Hashable) -> int:
-        try:
-            return self._handles[req]
-        except KeyError:
-            raise CacheError(f"request {req!r} is not live") from None
+        h = self._handles.get(req)
+        if h is None or not self._lib.imparo_cache_is_live(self._c, h):
+            raise CacheError(f"request {req!r} is not live")
+        return h
+
+    def handle(self, req: Hashable) -> int:
+        """The 64-bit name the native side knows `req` by (given out on first
+        asking, before the request is live, so that a scheduler can use it)."""
+        h = self._handles.get(req)
+        if h is None:
+            h = self._handles[req] = self._next_handle
+            self._next_handle += 1
+            self._names[h] = req
+        return h
+
+    def name_of(self, handle: int) -> Hashable:
+        return self._names[handle]
+
+    def _live_names(self) -> List[Hashable]:
+        return [r for r, h in self._handles.items() if self._lib.imparo_cache_is_live(self._c, h)]
 
     # ------------------------------------------------------------ requests
     def is_live(self, req: Hashable) -> bool:
-        return req in self._handles
+        h = self._handles.get(req)
+        return h is not None and bool(self._lib.imparo_cache_is_live(self._c, h))
 
     def admit(self, req: Hashable) -> int:
         """Takes a state slot for a new request; its tables start empty. The
         caller zeroes the slot's device state."""
-        if req in self._handles:
+        if self.is_live(req):
             raise CacheError(f"request {req!r} is already live")
-        h = self._next_handle
-        slot = self._lib.imparo_cache_admit(self._c, h)
+        slot = self._lib.imparo_cache_admit(self._c, self.handle(req))
         if slot == N.E_OUT_OF_PAGES:
             raise OutOfPages(f"all {self.n_slots} request slots are in use")
-        self._next_handle += 1
-        self._handles[req] = h
         return slot
 
     def release(self, req: Hashable) -> None:
         self._lib.imparo_cache_release(self._c, self._h(req))
-        del self._handles[req]
+        self.forget(req)
+
+    def forget(self, req: Hashable) -> None:
+        """Drops the name of a request that is not live (any more)."""
+        h = self._handles.get(req)
+        if h is not None and not self._lib.imparo_cache_is_live(self._c, h):
+            del self._handles[req]
+            del self._names[h]
 
     # ------------------------------------------------------------ growth
     def pages_needed(self, req: Hashable, new_length: int) -> List[int]:

@@ -240,6 +240,8 @@ int imparo_cache_first_needed_page(const ImparoCache* c, int group, int next_pos
     return c->first_needed_page(group, next_position);
 }
 int imparo_cache_n_live(const ImparoCache* c) { return (int)c->live.size(); }
+int imparo_cache_page_size(const ImparoCache* c) { return c->page_size; }
+int imparo_cache_n_groups(const ImparoCache* c) { return (int)c->pools.size(); }
 int imparo_cache_live_requests(const ImparoCache* c, int64_t* out, int capacity) {
     if ((int)c->live.size() > capacity) return IMPARO_E_CAPACITY;
     int i = 0;

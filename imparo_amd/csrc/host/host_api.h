@@ -56,6 +56,8 @@ int imparo_cache_table_copy(const ImparoCache* c, int group, int64_t req, int32_
 int imparo_cache_pages_needed(const ImparoCache* c, int64_t req, int new_length, int32_t* per_group);
 int imparo_cache_first_needed_page(const ImparoCache* c, int group, int next_position);
 int imparo_cache_n_live(const ImparoCache* c);
+int imparo_cache_page_size(const ImparoCache* c);
+int imparo_cache_n_groups(const ImparoCache* c);
 int imparo_cache_live_requests(const ImparoCache* c, int64_t* out, int capacity);
 int imparo_cache_check(const ImparoCache* c);
 
@@ -68,6 +70,40 @@ int imparo_cache_check(const ImparoCache* c);
 int64_t imparo_cache_pack(const ImparoCache* c, int n_rows, const int64_t* reqs, const int32_t* n_tokens,
                           const int32_t* tokens, const int32_t* n_want, const int32_t* want, int table_width,
                           int32_t* out, int64_t capacity, int32_t* layout);
+
+// ---- the scheduler's decisions (admission, portions under a token budget, pre-emption).
+// It knows requests by the same handles the cache manager uses, and only their sizes: how
+// many tokens wait to be fed, how many were fed, how many were generated. Token values,
+// sampling and the model step stay with the caller:
+//     n = imparo_sched_plan(...)      choose this step's batch (admits, pre-empts)
+//     ... run the step ...
+//     imparo_sched_advance(s)         the step ran
+//     imparo_sched_token(s, id, ..)   once per request whose logits were sampled
+typedef struct ImparoSched ImparoSched;
+
+#define IMPARO_EV_ADMIT 1
+#define IMPARO_EV_WAIT 2       // the head of the line does not fit yet
+#define IMPARO_EV_PREEMPT 3    // gave back its pages and slot; recomputes prompt ++ generated later
+#define IMPARO_EV_FAIL 4       // does not fit the cache even alone; it has left
+
+ImparoSched* imparo_sched_new(ImparoCache* cache, int max_batch_tokens, int max_running, int portion);
+void imparo_sched_delete(ImparoSched* s);
+// 0 queued | 1 finished at once (max_tokens <= 0) | IMPARO_E_ALREADY_LIVE
+int imparo_sched_add(ImparoSched* s, int64_t id, int prompt_len, int max_tokens);
+// Fills one line per planned request: offset into its pending tokens (-1: its sampled
+// token), how many tokens, whether logits are wanted at the last one. Events (what was
+// decided on the way) go to ev_ids/ev_kinds. Returns the number of planned requests.
+int imparo_sched_plan(ImparoSched* s, int64_t* ids, int32_t* offsets, int32_t* counts, int32_t* wants, int capacity,
+                      int64_t* ev_ids, int32_t* ev_kinds, int ev_capacity, int32_t* n_events);
+void imparo_sched_advance(ImparoSched* s);
+// A token was sampled for `id`: is_stop ends the reply unsent. Returns 0 (goes on), 1 (finished: stop),
+// 2 (finished: reached max_tokens; the token counts). The caller frees what a finished request holds.
+int imparo_sched_token(ImparoSched* s, int64_t id, int is_stop);
+int imparo_sched_drop_waiting_head(ImparoSched* s, int64_t* id);   // 1 and the id, or 0 if nobody waits
+int imparo_sched_n_waiting(const ImparoSched* s);
+int imparo_sched_n_running(const ImparoSched* s);
+int imparo_sched_waiting(const ImparoSched* s, int64_t* out, int capacity);
+int imparo_sched_running(const ImparoSched* s, int64_t* out, int capacity);
 
 #ifdef __cplusplus
 }

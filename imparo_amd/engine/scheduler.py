@@ -15,6 +15,7 @@ request that cannot fit even alone ends with an error.
 """
 from __future__ import annotations
 
+import ctypes
 import os
 from collections import deque
 from dataclasses import dataclass, field
@@ -63,17 +64,27 @@ class Planned:
 class Scheduler:
     """`engine` needs: step(entries) -> logits rows or None, release(id),
     cache (a CacheManager), page_size. `pick(logits, temperatures, uniforms)`
-    turns logits rows into token ids."""
+    turns logits rows into token ids.
+
+    The decisions (whom to admit, what each request feeds under the budget,
+    whom to pre-empt) are taken by the native scheduler core
+    (csrc/host/scheduler.cpp), which knows requests by size only; token
+    values, sampling and the model step are handled here."""
 
     def __init__(self, engine, pick: Callable, max_batch_tokens: int = 2048, max_running: int = 64,
                  portion: Optional[int] = None, entry_type=None):
+        from ..cache import native as N
+        self._N = N
+        self._lib = N.host_library()
         self.engine = engine
         self.pick = pick
         self.max_batch_tokens = max_batch_tokens
         self.max_running = max_running
         self.portion = portion or prefill_portion()
-        self.waiting: Deque[Request] = deque()
-        self.running: List[Request] = []
+        self._s = self._lib.imparo_sched_new(engine.cache._c, max_batch_tokens, max_running, self.portion)
+        if not self._s:
+            raise ValueError("the scheduler refused its sizes")
+        self._requests: Dict[int, Request] = {}          # by native handle: waiting or running
         self.finished: Dict[Hashable, Request] = {}
         self._arrivals = 0
         if entry_type is None:
@@ -81,6 +92,20 @@ class Scheduler:
             entry_type = StepEntry
         self._entry = entry_type
         self.log: List[Tuple] = []      # decisions, for tests and --verbose
+        cap = max(64, max_running + 8)
+        self._cap = cap
+        self._ids = (ctypes.c_int64 * cap)()
+        self._offs = (ctypes.c_int32 * cap)()
+        self._counts = (ctypes.c_int32 * cap)()
+        self._wants = (ctypes.c_int32 * cap)()
+        self._ev_ids = (ctypes.c_int64 * (4 * cap))()
+        self._ev_kinds = (ctypes.c_int32 * (4 * cap))()
+        self._n_ev = ctypes.c_int32(0)
+
+    def __del__(self):
+        if getattr(self, "_s", None):
+            self._lib.imparo_sched_delete(self._s)
+            self._s = None
 
     # ------------------------------------------------------------ intake
     def add(self, request_id: Hashable, prompt: Sequence[int], params: SamplingParams) -> Request:
@@ -88,103 +113,72 @@ class Scheduler:
             raise ValueError("a request needs at least one prompt token")
         r = Request(request_id, list(prompt), params, pending=list(prompt), arrival=self._arrivals)
         self._arrivals += 1
-        if params.max_tokens <= 0:
+        h = self.engine.cache.handle(request_id)
+        rc = self._lib.imparo_sched_add(self._s, h, len(prompt), params.max_tokens)
+        if rc == 1:
             self._finish(r, "length")
             return r
-        self.waiting.append(r)
+        if rc < 0:
+            raise ValueError(f"request {request_id!r} is already queued")
+        self._requests[h] = r
         return r
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self._lib.imparo_sched_n_waiting(self._s) or self._lib.imparo_sched_n_running(self._s))
+
+    def _listed(self, fn) -> List[Request]:
+        buf = (ctypes.c_int64 * max(1, len(self._requests)))()
+        n = fn(self._s, buf, len(buf))
+        return [self._requests[buf[i]] for i in range(max(n, 0))]
+
+    @property
+    def waiting(self) -> List[Request]:
+        return self._listed(self._lib.imparo_sched_waiting)
+
+    @property
+    def running(self) -> List[Request]:
+        return self._listed(self._lib.imparo_sched_running)
 
     # ------------------------------------------------------------ decisions
-    def _pages_for(self, n_tokens: int) -> int:
-        ps = self.engine.page_size
-        return (n_tokens + ps - 1) // ps
-
-    def _free_pages(self) -> int:
-        free = self.engine.cache.free_pages()
-        return min(free) if free else 1 << 30
-
-    def _next_tokens(self, r: Request, budget: int) -> Tuple[List[int], bool]:
-        """What `r` would feed next under `budget` tokens, and whether that
-        ends in a place whose logits are needed."""
-        if r.fed < len(r.pending):
-            n = min(self.portion, budget, len(r.pending) - r.fed)
-            return r.pending[r.fed:r.fed + n], r.fed + n == len(r.pending) and r.next_token is None
-        return [r.next_token], True
-
-    def _pages_needed(self, p: Planned) -> int:
-        cache = self.engine.cache
-        if cache.is_live(p.request.id):
-            need = cache.pages_needed(p.request.id, cache.length[p.request.id] + len(p.tokens))
-            return max(need) if need else 0
-        return self._pages_for(len(p.tokens))
-
     def plan(self) -> List[Planned]:
         """Chooses this step's batch; admits and pre-empts as needed."""
-        budget = self.max_batch_tokens
-        planned: List[Planned] = []
-        # 1. running requests: decoders first, then prompts in progress
-        order = sorted(self.running, key=lambda r: (r.fed < len(r.pending), r.arrival))
-        for r in order:
-            if budget <= 0:
-                break
-            toks, wants = self._next_tokens(r, budget)
-            planned.append(Planned(r, toks, wants))
-            budget -= len(toks)
-        spoken_for = sum(self._pages_needed(p) for p in planned)
-        # 2. admissions, first come first served; the head of the line blocks the rest.
-        # A newcomer needs the pages of its first portion and leaves one page of
-        # headroom per running request
-        # (/root/reference/crates/imparo-server/src/main.rs:2230-2246).
-        while self.waiting and budget > 0 and len(self.running) < self.max_running:
-            r = self.waiting[0]
-            toks, wants = self._next_tokens(r, budget)
-            need = self._pages_for(len(toks)) + len(self.running)
-            if self.engine.cache.slots.n_free == 0 or (self.running and need > self._free_pages() - spoken_for):
+        n = self._lib.imparo_sched_plan(self._s, self._ids, self._offs, self._counts, self._wants, self._cap,
+                                        self._ev_ids, self._ev_kinds, 4 * self._cap, ctypes.byref(self._n_ev))
+        if n < 0:
+            raise RuntimeError(f"the scheduler could not plan a step (code {n})")
+        N = self._N
+        for i in range(min(self._n_ev.value, 4 * self._cap)):
+            h, kind = self._ev_ids[i], self._ev_kinds[i]
+            r = self._requests[h]
+            if kind == N.EV_ADMIT:
+                self.log.append(("admit", r.id))
+            elif kind == N.EV_WAIT:
                 self.log.append(("wait", r.id))
-                break
-            self.waiting.popleft()
-            self.running.append(r)
-            self.log.append(("admit", r.id))
-            planned.append(Planned(r, toks, wants))
-            spoken_for += self._pages_for(len(toks))
-            budget -= len(toks)
-        # 3. do the pages suffice? if not, the youngest running request goes back in line
-        while planned:
-            if sum(self._pages_needed(p) for p in planned) <= self._free_pages():
-                break
-            if len(self.running) == 1:
-                r = self.running[0]
-                self._leave(r)
+            elif kind == N.EV_PREEMPT:
+                # it gave back everything it held; it will recompute prompt ++ generated
+                self.engine.release(r.id)
+                r.pending = r.prompt + r.generated
+                r.fed = 0
+                r.next_token = None
+                r.preemptions += 1
+                self.log.append(("preempt", r.id))
+            elif kind == N.EV_FAIL:
+                self.engine.release(r.id)
+                del self._requests[h]
                 self._finish(r, "error: the request does not fit the cache even alone")
-                planned = []
-                break
-            victim = max(self.running, key=lambda r: r.arrival)
-            self.preempt(victim)
-            planned = [p for p in planned if p.request is not victim]
+        planned = []
+        for i in range(n):
+            r = self._requests[self._ids[i]]
+            off, count = self._offs[i], self._counts[i]
+            tokens = [r.next_token] if off < 0 else r.pending[off:off + count]
+            planned.append(Planned(r, tokens, bool(self._wants[i])))
         return planned
-
-    def preempt(self, r: Request) -> None:
-        """Gives back everything `r` holds; it will recompute prompt ++ generated."""
-        self._leave(r)
-        r.pending = r.prompt + r.generated
-        r.fed = 0
-        r.next_token = None
-        r.preemptions += 1
-        self.waiting.appendleft(r)
-        self.log.append(("preempt", r.id))
-
-    def _leave(self, r: Request) -> None:
-        if r in self.running:
-            self.running.remove(r)
-        self.engine.release(r.id)
 
     def _finish(self, r: Request, reason: str) -> None:
         r.finished = True
         r.finish_reason = reason
         self.finished[r.id] = r
+        self.engine.cache.forget(r.id)
         self.log.append(("finish", r.id, reason))
 
     # ------------------------------------------------------------ one iteration
@@ -197,6 +191,7 @@ class Scheduler:
         entries = [self._entry(p.request.id, p.tokens, [len(p.tokens) - 1] if p.wants_logits else [])
                    for p in planned]
         logits = self.engine.step(entries)
+        self._lib.imparo_sched_advance(self._s)
         for p in planned:
             r = p.request
             if r.fed < len(r.pending):
@@ -211,26 +206,32 @@ class Scheduler:
             picks = self.pick(logits, temps, unis)
             for r, tok in zip(askers, picks):
                 tok = int(tok)
-                if tok in r.params.stop_token_ids:     # a stop token ends the reply unsent
-                    self._leave(r)
-                    self._finish(r, "stop")
-                    continue
-                r.generated.append(tok)
-                out.append((r.id, tok))
-                if len(r.generated) >= r.params.max_tokens:   # the last token needs no forward
-                    self._leave(r)
-                    self._finish(r, "length")
-                else:
+                h = self.engine.cache.handle(r.id)
+                is_stop = tok in r.params.stop_token_ids      # a stop token ends the reply unsent
+                outcome = self._lib.imparo_sched_token(self._s, h, int(is_stop))
+                if not is_stop:
+                    r.generated.append(tok)
+                    out.append((r.id, tok))
+                if outcome == 0:
                     r.next_token = tok
+                else:                                          # 1: stop; 2: the last token needs no forward
+                    self.engine.release(r.id)
+                    del self._requests[h]
+                    self._finish(r, "stop" if outcome == 1 else "length")
         return out
 
     def run(self) -> Dict[Hashable, Request]:
         while self.has_work():
-            before = (len(self.waiting), len(self.running), len(self.finished))
+            n_running = self._lib.imparo_sched_n_running(self._s)
+            before = (self._lib.imparo_sched_n_waiting(self._s), n_running, len(self.finished))
             self.step()
-            if not self.running and self.waiting and before == (len(self.waiting), 0, len(self.finished)):
-                r = self.waiting.popleft()      # nothing runs and the head still cannot start
-                self._finish(r, "error: the request does not fit the cache even alone")
+            after = (self._lib.imparo_sched_n_waiting(self._s), self._lib.imparo_sched_n_running(self._s),
+                     len(self.finished))
+            if after[1] == 0 and after[0] and before == after and n_running == 0:
+                head = ctypes.c_int64(0)                       # nothing runs and the head still cannot start
+                if self._lib.imparo_sched_drop_waiting_head(self._s, ctypes.byref(head)):
+                    r = self._requests.pop(head.value)
+                    self._finish(r, "error: the request does not fit the cache even alone")
         return self.finished
 
 

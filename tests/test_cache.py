@@ -179,3 +179,30 @@ def test_random_orders_never_lose_or_share_a_page(seed):
         m.release(rid)
     m.check()
     assert m.free_pages() == [24, 24] and m.slots.n_free == 4
+
+
+def test_pack_lays_out_a_step():
+    """The native packer: tokens | positions | row_of_token | seg_start | seg_len | slot | row lists |
+    want | tables, positions counted from each request's length before the step."""
+    m = CacheManager([PagedSpec(1, 16), FixedSpec((4,)), PagedSpec(1, 16, window=6)], page_size=4, n_pages=16, n_slots=4)
+    m.admit("a"), m.admit("b"), m.admit("c")
+    m.reserve("a", 9), m.commit("a", 9)
+    m.reserve("a", 10), m.reserve("b", 3), m.reserve("c", 1)
+    arr, lay = m.pack(["a", "b", "c"], [[7], [1, 2, 3], [4]], [[0], [2, 0], []])
+    T, R, W, G, P = (lay[k] for k in "TRWGP")
+    assert (T, R, W, G) == (5, 3, 3, 2) and P == 3 and lay["n_single"] == 2 and lay["n_multi"] == 1
+    assert lay["max_seg_len"] == 3 and lay["max_context"] == 10 and lay["n_prefill_tiles"] == 1
+    a = arr.tolist()
+    assert a[0:5] == [7, 1, 2, 3, 4]                      # tokens
+    assert a[5:10] == [9, 0, 1, 2, 0]                     # positions
+    assert a[10:15] == [0, 1, 1, 1, 2]                    # row of token
+    assert a[15:18] == [0, 1, 4] and a[18:21] == [1, 3, 1] and a[21:24] == [0, 1, 2]   # start, len, slot
+    assert a[24:27] == [0, 2, 1]                          # rows with one token, then the others
+    assert a[27:30] == [0, 3, 1]                          # wanted places as indices into the batch
+    tables = arr[30:].reshape(G, R, P).tolist()
+    assert tables[0] == [m.table(0, "a"), m.table(0, "b") + [-1, -1], m.table(0, "c") + [-1, -1]]
+    assert tables[1][0] == m.table(1, "a") and tables[1][0][0] == -1      # behind the window of 6 at length 9
+    fixed, lay2 = m.pack(["a"], [[7]], [[0]], table_width=8)
+    assert lay2["P"] == 8 and fixed[-8:].tolist() == m.table(1, "a") + [-1] * 5
+    with pytest.raises(CacheError):
+        m.pack(["zzz"], [[1]], [[0]])

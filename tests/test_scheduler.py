@@ -123,6 +123,18 @@ def test_arrival_order_and_running_cap():
     assert all(done[n].generated == expected([ord(n)] * 3, 3) for n in "abc")
 
 
+def test_newcomers_of_one_step_do_not_share_a_slot():
+    eng = FakeEngine(64, n_slots=2)
+    s = Scheduler(eng, pick, entry_type=Entry, max_batch_tokens=64, max_running=8)
+    for name in "abc":
+        s.add(name, [ord(name)] * 3, SamplingParams(max_tokens=2))
+    s.step()
+    assert [r.id for r in s.running] == ["a", "b"] and [r.id for r in s.waiting] == ["c"]
+    done = s.run()
+    assert all(done[n].generated == expected([ord(n)] * 3, 2) for n in "abc")
+    assert eng.cache.slots.n_free == 2
+
+
 def test_stop_token_ends_the_reply_unsent():
     want = expected([5, 6], 5)
     eng, s = make()
