@@ -1,0 +1,80 @@
+"""Long contexts and a serving workload, where the plain implementation cannot
+follow: the bfloat16 matrix-core path is held to the engine's own float32 path
+(itself held to the plain implementation at short lengths elsewhere), and
+continuous batching under page pressure is held to each request run alone."""
+import random
+
+import pytest
+import torch
+
+from conftest import prompt_tokens
+from gpu_helpers import make_engine
+from tolerances import check_logits
+
+pytestmark = pytest.mark.gpu
+
+LONG = dict(
+    architectures=["Lfm2ForCausalLM"], model_type="lfm2", vocab_size=512, hidden_size=256,
+    num_hidden_layers=4, layer_types=["conv", "full_attention", "sliding_attention", "full_attention"],
+    num_attention_heads=4, num_key_value_heads=2, block_auto_adjust_ff_dim=False, block_ff_dim=512,
+    conv_L_cache=3, conv_bias=False, rope_theta=1000000.0, tie_embedding=True, norm_eps=1e-5,
+    max_position_embeddings=32768, sliding_window=700,
+)
+
+
+@pytest.fixture(scope="module")
+def long_model(tmp_path_factory):
+    from imparo_amd import write_random_model
+    d = str(tmp_path_factory.mktemp("long"))
+    write_random_model(LONG, 5, d)
+    return d
+
+
+def test_long_context_bfloat16_against_float32(long_model):
+    """16,500 tokens in portions of 2,048 (tiles of 64 queries over hundreds of
+    key tiles, a window of 700 that gives pages back), then single tokens over
+    more than 64 splits of 256 keys, through captured steps."""
+    from imparo_amd.engine import StepEntry
+    N = 16500
+    toks = prompt_tokens(512, N + 40, 99)
+    runs = {}
+    for dtype in ("float32", "bfloat16"):
+        eng = make_engine(long_model, dtype, page_size=64, max_tokens=N + 128, max_requests=2)
+        out = []
+        for lo in range(0, N, 2048):
+            hi = min(N, lo + 2048)
+            out.append(eng.step([StepEntry("l", toks[lo:hi], list(range(hi - lo - 8, hi - lo)))]).cpu())
+        for i in range(N, N + 40):
+            out.append(eng.step([StepEntry("l", toks[i:i + 1], [0])]).cpu().clone())
+        held = eng.cache.held_pages("l")
+        assert held[0] == (N + 40 + 63) // 64 and held[1] <= 700 // 64 + 2     # the window's group holds a dozen pages
+        runs[dtype] = torch.cat(out)
+    check_logits(runs["bfloat16"], runs["float32"], "bfloat16", "long context")
+
+
+def test_serving_workload_under_page_pressure(long_model):
+    """32 requests in waves, prompts of 20..600 tokens, 5..40 new tokens each, a pool that holds
+    about a third of them at once: every output equals the request's output when it runs alone."""
+    from imparo_amd.engine import Engine
+    from imparo_amd.engine.scheduler import Scheduler, generate
+    from imparo_amd.sampling import Sampler, SamplingParams
+    rng = random.Random(3)
+    reqs = [(prompt_tokens(512, rng.randint(20, 600), 500 + i), rng.randint(5, 40)) for i in range(32)]
+    eng = Engine(long_model, dtype="float32", page_size=16, max_tokens=3200, max_requests=12)
+    sched = Scheduler(eng, Sampler(eng.device).pick, max_batch_tokens=512, max_running=12, portion=128)
+    pending = list(enumerate(reqs))
+    while pending or sched.has_work():
+        if pending and (not sched.has_work() or rng.random() < 0.3):
+            for _ in range(min(8, len(pending))):                 # a wave arrives
+                i, (prompt, n) = pending.pop(0)
+                sched.add(i, prompt, SamplingParams(max_tokens=n))
+        if sched.has_work():
+            sched.step()
+            eng.cache.check()
+    assert any(e[0] == "preempt" for e in sched.log) and any(e[0] == "wait" for e in sched.log)
+    assert eng.free_pages() == [200, 200] and eng.cache.slots.n_free == 12
+    alone = Engine(long_model, dtype="float32", page_size=16, max_tokens=1024, max_requests=2)
+    for i in rng.sample(range(32), 10):
+        prompt, n = reqs[i]
+        assert sched.finished[i].finish_reason == "length"
+        assert sched.finished[i].generated == generate(alone, [prompt], max_tokens=n)[0], f"request {i}"
