@@ -113,10 +113,17 @@ __global__ __launch_bounds__(256) void k_gemm_f32(const float* __restrict__ X, c
 template <typename TOut>
 __global__ __launch_bounds__(256, 2) void k_gemm_bf16_tile(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                            const float* __restrict__ bias, TOut* __restrict__ Y,
-                                                           int M, int N, int K, int tiles_m, int tiles_n,
-                                                           int epilogue) {
+                                                           int M, int N, int K_all, int tiles_m, int tiles_n,
+                                                           int epilogue, int k_per) {
     __shared__ __attribute__((aligned(16))) bf16_t As[2][BG_BM * BG_LD];
     __shared__ __attribute__((aligned(16))) bf16_t Bs[2][BG_BN * BG_LD];
+    // slices of K (gridDim.y > 1): block (x, y) sums K range [y * k_per, (y+1) * k_per) into Y + y * M * N
+    const int k_lo = blockIdx.y * k_per;
+    const int K = min(K_all, k_lo + k_per) - k_lo;
+    X += k_lo;
+    W += k_lo;
+    Y += (size_t)blockIdx.y * M * N;
+    if (blockIdx.y > 0) bias = nullptr;
     // block id -> tile: consecutive logical ids on one XCD, grouped over 8 tile rows
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + N_XCD - 1) / N_XCD;
@@ -141,8 +148,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_bf16_tile(const bf16_t* __restr
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int row = (tid >> 3) + 32 * j;
-        pa[j] = X + (size_t)min(m0 + row, M - 1) * K + kc8;
-        pb[j] = W + (size_t)min(n0 + row, N - 1) * K + kc8;
+        pa[j] = X + (size_t)min(m0 + row, M - 1) * K_all + kc8;
+        pb[j] = W + (size_t)min(n0 + row, N - 1) * K_all + kc8;
         lds_off[j] = row * BG_LD + kc8;
     }
     const int nk = (K + BG_BK - 1) / BG_BK;
@@ -373,7 +380,16 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, const float* bias, T
 // a weight with few rows and a long K (the feed-forward's way back) gives too few blocks
 // otherwise. One slice per 2048 of K, for at most 64 rows and at most 4096 weight rows.
 extern "C" int imparo_gemm_slices(int m, int n, int k, int dtype) {
-    if (dtype != IMPARO_BF16 || m > 64 || n > 4096 || k < 4096) return 1;
+    if (dtype != IMPARO_BF16) return 1;
+    if (m > 64) {
+        // many rows: with about one tile of 128x128 per CU or fewer, a block has a CU to itself and
+        // nothing hides its waits; slices of K (at least 1024 each, at most 4) multiply the blocks
+        const long long tiles = (long long)((m + BG_BM - 1) / BG_BM) * ((n + BG_BN - 1) / BG_BN);
+        int slices = 1;
+        while (slices < 4 && tiles * slices * 2 <= 512 && k / (slices * 2) >= 1024) slices *= 2;
+        return slices;
+    }
+    if (n > 4096 || k < 4096) return 1;
     return (k + 2047) / 2048;
 }
 
@@ -534,7 +550,9 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
         const long long total = (long long)tiles_m * tiles_n;
         if (total > 0x7fffff00LL) return IMPARO_BAD_ARGUMENT;
         const unsigned blocks = (unsigned)(((total + N_XCD - 1) / N_XCD) * N_XCD);
-        k_gemm_bf16_tile<TOut><<<blocks, 256, 0, s>>>(x, w, bias, y, m, n, k, tiles_m, tiles_n, epilogue);
+        const int k_per = ((k + slices - 1) / slices + BG_BK - 1) / BG_BK * BG_BK;
+        dim3 grid(blocks, (unsigned)((k + k_per - 1) / k_per));
+        k_gemm_bf16_tile<TOut><<<grid, 256, 0, s>>>(x, w, bias, y, m, n, k, tiles_m, tiles_n, epilogue, k_per);
     }
     return launch_status();
 }

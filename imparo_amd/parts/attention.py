@@ -114,7 +114,8 @@ class Attention:
                           v_transposed=vt)
         if o.dtype != self.out.in_dtype:
             raise ValueError("the output projection's weight dtype differs from the attention output's")
-        return self.out(ctx, o, torch.float32, "mixer_out")
+        # a delta for the residual stream: the next norm adds slices, so it may come sliced
+        return self.out(ctx, o, torch.float32, "mixer_out", sliced_ok=True)
 
 
 register_part("mixer", "attention", Attention)

@@ -70,7 +70,8 @@ class ShortConv:
         y = ctx.workspace.get("conv_out", (T, self.width), self.out_proj.in_dtype)
         ops.short_conv(bcx, self.conv_weight, self.conv_bias, ctx.fixed_state(site), ctx.row_of_token,
                        ctx.seg_start, ctx.seg_len, ctx.slot, y, single_tokens=ctx.max_seg_len == 1)
-        return self.out_proj(ctx, y, torch.float32, "mixer_out")
+        # a delta for the residual stream: the next norm adds slices, so it may come sliced
+        return self.out_proj(ctx, y, torch.float32, "mixer_out", sliced_ok=True)
 
 
 register_part("mixer", "short_conv", ShortConv)

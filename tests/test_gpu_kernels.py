@@ -84,7 +84,14 @@ def test_gemm_in_slices_of_k_and_the_norm_that_adds_them(m):
     x, w, b = rnd(m, k, seed=1).to(torch.bfloat16), rnd(n, k, seed=2, scale=0.1).to(torch.bfloat16), rnd(n, seed=3)
     slices = ops().gemm_slices(m, n, k, torch.bfloat16)
     assert slices == 3 and ops().gemm_slices(m, n, 2048, torch.bfloat16) == 1
-    assert ops().gemm_slices(65, n, k, torch.bfloat16) == 1 and ops().gemm_slices(m, n, k, torch.float32) == 1
+    assert ops().gemm_slices(m, n, k, torch.float32) == 1
+    # many rows and few tiles: the 128x128 kernel takes slices too (at least 1024 of K each, at most 4)
+    assert ops().gemm_slices(300, n, k, torch.bfloat16) == 4 and ops().gemm_slices(300, n, 2048, torch.bfloat16) == 2
+    assert ops().gemm_slices(2048, 16384, 2048, torch.bfloat16) == 1
+    x3 = rnd(300, k, seed=7).to(torch.bfloat16)
+    out3 = torch.full((4, 300, n), float("nan"), device=DEV)
+    ops().gemm(x3.to(DEV), w.to(DEV), out3, bias=b.to(DEV))
+    torch.testing.assert_close(out3.cpu().double().sum(0), x3.double() @ w.double().t() + b.double(), rtol=1e-5, atol=1e-5)
     out = torch.full((slices, m, n), float("nan"), device=DEV)
     ops().gemm(x.to(DEV), w.to(DEV), out, bias=b.to(DEV))
     ref = x.double() @ w.double().t() + b.double()
