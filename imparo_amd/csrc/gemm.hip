@@ -184,22 +184,37 @@ __global__ __launch_bounds__(256, 2) void k_gemm_bf16_tile(const bf16_t* __restr
     const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
     const int a_base = (wm * 64 + frag_row) * BG_LD + frag_k;
     const int b_base = (wn * 64 + frag_row) * BG_LD + frag_k;
-    auto compute = [&](int buf) {
+    // The operand fragments of K-sub-step ks+1 are read from LDS while the products of sub-step ks
+    // run: without that every sub-step waits a full LDS latency before its first product.
+    auto read_frags = [&](int buf, int ks, Frag8 (&fa)[2], Frag8 (&fb)[2]) {
 #pragma unroll
-        for (int ks = 0; ks < BG_BK / 16; ++ks) {
-            Frag8 fa[2], fb[2];
+        for (int ii = 0; ii < 2; ++ii)
+            fa[ii].u = *reinterpret_cast<const uint4*>(&As[buf][a_base + ii * 32 * BG_LD + ks * 16]);
 #pragma unroll
-            for (int ii = 0; ii < 2; ++ii)
-                fa[ii].u = *reinterpret_cast<const uint4*>(&As[buf][a_base + ii * 32 * BG_LD + ks * 16]);
+        for (int jj = 0; jj < 2; ++jj)
+            fb[jj].u = *reinterpret_cast<const uint4*>(&Bs[buf][b_base + jj * 32 * BG_LD + ks * 16]);
+    };
+    auto multiply = [&](const Frag8 (&fa)[2], const Frag8 (&fb)[2]) {
+#pragma unroll
+        for (int ii = 0; ii < 2; ++ii)
 #pragma unroll
             for (int jj = 0; jj < 2; ++jj)
-                fb[jj].u = *reinterpret_cast<const uint4*>(&Bs[buf][b_base + jj * 32 * BG_LD + ks * 16]);
-#pragma unroll
-            for (int ii = 0; ii < 2; ++ii)
-#pragma unroll
-                for (int jj = 0; jj < 2; ++jj)
-                    acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ii].v, fb[jj].v, acc[ii][jj], 0, 0, 0);
-        }
+                acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ii].v, fb[jj].v, acc[ii][jj], 0, 0, 0);
+    };
+    auto compute = [&](int buf) {
+        Frag8 fa0[2], fb0[2], fa1[2], fb1[2];
+        read_frags(buf, 0, fa0, fb0);
+        read_frags(buf, 1, fa1, fb1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(fa0, fb0);
+        read_frags(buf, 2, fa0, fb0);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(fa1, fb1);
+        read_frags(buf, 3, fa1, fb1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(fa0, fb0);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(fa1, fb1);
     };
     // K-step i: the next step's tile goes from its registers to LDS, those registers
     // take the load of step i+1+BG_PF, then step i is multiplied out of LDS
@@ -250,6 +265,161 @@ __global__ __launch_bounds__(256, 2) void k_gemm_bf16_tile(const bf16_t* __restr
                 if (m < M) store_f32<TOut>(Y, (size_t)m * N + n, acc[i][j][r] + bn);
             }
         }
+}
+
+// ------------------------------------------------------------------ bfloat16, many rows, large tiles
+// The 128x128 kernel moves (128 + 128) rows of K per 128 x 128 outputs through L2: 64 flops a byte,
+// which at this chip's L2 bandwidth caps it near 650 TFLOP/s whatever the matrix cores could do.
+// This kernel takes a WM x WN grid of waves, each TM x TN MFMA tiles of 32x32, so that a block's
+// tile is (WM TM 32) x (WN TN 32): 256 x 256 moves half the bytes per flop. One block per CU
+// (its LDS holds two K-steps of both operands), global loads two K-steps ahead in registers.
+template <typename TOut, int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(WM * WN * 64) void k_gemm_bf16_big(const bf16_t* __restrict__ X,
+                                                                const bf16_t* __restrict__ W,
+                                                                const float* __restrict__ bias,
+                                                                TOut* __restrict__ Y, int M, int N, int K,
+                                                                int tiles_m, int tiles_n, int epilogue) {
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32, NT = WM * WN * 64;
+    constexpr int PA = BM * 8 / NT, PB = BN * 8 / NT;      // 16-byte pieces of a K-step per thread
+    static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile rows must divide over the threads");
+    extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
+    bf16_t* As = lds;                                      // [2][BM * BG_LD]
+    bf16_t* Bs = lds + 2 * BM * BG_LD;                     // [2][BN * BG_LD]
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + N_XCD - 1) / N_XCD;
+    const int logical = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;
+    if (logical >= total) return;
+    const int per_group = BG_GROUP_M * tiles_n;
+    const int first_m = (logical / per_group) * BG_GROUP_M;
+    const int gsize = min(tiles_m - first_m, BG_GROUP_M);
+    const int tile_m = first_m + (logical % per_group) % gsize;
+    const int tile_n = (logical % per_group) / gsize;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int kc8 = (tid & 7) * 8;
+    const bf16_t* pa[PA];
+    const bf16_t* pb[PB];
+    int la[PA], lb[PB];
+#pragma unroll
+    for (int j = 0; j < PA; ++j) {
+        const int row = (tid >> 3) + (NT / 8) * j;
+        pa[j] = X + (size_t)min(m0 + row, M - 1) * K + kc8;
+        la[j] = row * BG_LD + kc8;
+    }
+#pragma unroll
+    for (int j = 0; j < PB; ++j) {
+        const int row = (tid >> 3) + (NT / 8) * j;
+        pb[j] = W + (size_t)min(n0 + row, N - 1) * K + kc8;
+        lb[j] = row * BG_LD + kc8;
+    }
+    const int nk = (K + BG_BK - 1) / BG_BK;
+    uint4 a0[PA], b0[PB], a1[PA], b1[PB];
+    auto fetch = [&](int kt, uint4 (&a)[PA], uint4 (&b)[PB]) {
+        const bool in = kt * BG_BK + kc8 < K;
+        const size_t off = (size_t)kt * BG_BK;
+#pragma unroll
+        for (int j = 0; j < PA; ++j) a[j] = in ? *reinterpret_cast<const uint4*>(pa[j] + off) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < PB; ++j) b[j] = in ? *reinterpret_cast<const uint4*>(pb[j] + off) : make_uint4(0, 0, 0, 0);
+    };
+    auto stash = [&](int buf, const uint4 (&a)[PA], const uint4 (&b)[PB]) {
+#pragma unroll
+        for (int j = 0; j < PA; ++j) *reinterpret_cast<uint4*>(&As[buf * BM * BG_LD + la[j]]) = a[j];
+#pragma unroll
+        for (int j = 0; j < PB; ++j) *reinterpret_cast<uint4*>(&Bs[buf * BN * BG_LD + lb[j]]) = b[j];
+    };
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
+    const int a_base = (wm * TM * 32 + frag_row) * BG_LD + frag_k;
+    const int b_base = (wn * TN * 32 + frag_row) * BG_LD + frag_k;
+    auto compute = [&](int buf) {
+#pragma unroll
+        for (int ks = 0; ks < BG_BK / 16; ++ks) {
+            Frag8 fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                fa[i].u = *reinterpret_cast<const uint4*>(&As[buf * BM * BG_LD + a_base + i * 32 * BG_LD + ks * 16]);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                fb[j].u = *reinterpret_cast<const uint4*>(&Bs[buf * BN * BG_LD + b_base + j * 32 * BG_LD + ks * 16]);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i].v, fb[j].v, acc[i][j], 0, 0, 0);
+        }
+    };
+    auto step = [&](int i, uint4 (&na)[PA], uint4 (&nb)[PB]) {
+        const int buf = i & 1;
+        if (i + 1 < nk) {
+            stash(buf ^ 1, na, nb);
+            fetch(i + 3, na, nb);
+        }
+        compute(buf);
+        __syncthreads();
+    };
+    fetch(0, a0, b0);
+    fetch(1, a1, b1);
+    stash(0, a0, b0);
+    fetch(2, a0, b0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; kt += 2) {
+        step(kt, a1, b1);
+        if (kt + 1 < nk) step(kt + 1, a0, b0);
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + (wn * TN + j) * 32 + (lane & 31);
+            const float bn = (bias && n < N) ? bias[n] : 0.f;
+            if (epilogue == EPI_SWIGLU) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float mine = acc[i][j][r] + bn;
+                    const float other = __shfl_xor(mine, 1, WAVE);
+                    const int m = m0 + (wm * TM + i) * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                    if (!(lane & 1) && n + 1 < N && m < M)
+                        store_f32<TOut>(Y, (size_t)m * (N / 2) + n / 2, silu_mul_f(mine, other));
+                }
+                continue;
+            }
+            if (n >= N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + (wm * TM + i) * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                if (m < M) store_f32<TOut>(Y, (size_t)m * N + n, acc[i][j][r] + bn);
+            }
+        }
+}
+
+template <typename TOut, int WM, int WN, int TM, int TN>
+static int launch_big(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
+                      hipStream_t s) {
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    constexpr size_t lds_bytes = (size_t)2 * (BM + BN) * BG_LD * sizeof(bf16_t);
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)k_gemm_bf16_big<TOut, WM, WN, TM, TN>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
+            return IMPARO_LAUNCH_FAILED;
+        configured = true;
+    }
+    const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
+    const long long total = (long long)tiles_m * tiles_n;
+    const unsigned blocks = (unsigned)(((total + N_XCD - 1) / N_XCD) * N_XCD);
+    k_gemm_bf16_big<TOut, WM, WN, TM, TN><<<blocks, WM * WN * 64, lds_bytes, s>>>(x, w, bias, y, m, n, k, tiles_m,
+                                                                                 tiles_n, epilogue);
+    return launch_status();
 }
 
 // ------------------------------------------------------------------ bfloat16, few rows
@@ -520,6 +690,13 @@ static void launch_stream(const bf16_t* x, const bf16_t* w, const float* bias, T
         k_gemm_bf16_stream<TOut, MT, 2><<<blocks, 2 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
 }
 
+// The 256x256 tile (one block per CU) pays once its tiles keep most of the chip's 256 CUs busy:
+// measured, from about 160 tiles on (192 tiles: +15% over 128x128; 96 tiles: -30%).
+static bool big_tile_pays(int m, int n, int k) {
+    (void)k;
+    return (long long)((m + 255) / 256) * ((n + 255) / 256) >= 160;
+}
+
 template <typename TOut>
 static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
                        int force, int slices, hipStream_t s) {
@@ -546,6 +723,11 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
         else
             launch_skinny<TOut, 4>(x, w, bias, y, m, n, k, epilogue, slices, s);
     } else {
+        // `force` 256: the 256x256 tile; 257: 256x128 (for measurements); otherwise by shape
+        if (slices == 1 && (force == 256 || (force == 0 && big_tile_pays(m, n, k))))
+            return launch_big<TOut, 2, 4, 4, 2>(x, w, bias, y, m, n, k, epilogue, s);
+        if (slices == 1 && force == 257)
+            return launch_big<TOut, 4, 2, 2, 2>(x, w, bias, y, m, n, k, epilogue, s);
         const int tiles_m = (m + BG_BM - 1) / BG_BM, tiles_n = (n + BG_BN - 1) / BG_BN;
         const long long total = (long long)tiles_m * tiles_n;
         if (total > 0x7fffff00LL) return IMPARO_BAD_ARGUMENT;
