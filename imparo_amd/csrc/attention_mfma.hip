@@ -36,27 +36,49 @@ struct Paged {
 
 __device__ __forceinline__ short pack_bf16(float f) { return (short)f32_to_bf16(f); }
 
-// One tile of 16 keys starting at key_base (a multiple of 16). [lo_q, hi_q] is
-// the key range of this lane's query, [lo_all, hi_all] the live keys any query
-// of the wave may read (addresses are clamped into it; values outside it are
-// forced to zero, never multiplied). `full`: every key of the tile is inside
-// every query's range, so no masking is needed.
+// The operands of one tile of 16 keys: K rows and V^T rows as the products take
+// them. Loading is apart from computing so that a wave can have the loads of
+// several tiles in flight before it waits for the first.
 template <int ND>
-__device__ __forceinline__ void attn_tile(WaveState<ND>& st, const Paged& kv, int key_base, int lo_q, int hi_q,
-                                          int lo_all, int hi_all, bool full, float scale, int lane) {
+struct TileRegs {
+    s16x4 k[ND];
+    s16x4 v[ND];
+};
+
+// Issues the loads of the tile starting at key_base (a multiple of 16).
+// [lo_all, hi_all] are the live keys any query of the wave may read: addresses
+// are clamped into it (what lies outside is forced to zero before use).
+template <int ND>
+__device__ __forceinline__ void load_tile(TileRegs<ND>& r, const Paged& kv, int key_base, int lo_all, int hi_all,
+                                          int lane) {
     constexpr int D = ND * 16;
     const int c = lane & 15, g = lane >> 4;
-    // ---- scores
     const int key = min(max(key_base + c, lo_all), hi_all);
     int page = kv.table[key / kv.page_size];
     page = min(max(page, 0), kv.n_pages - 1);
     const bf16_t* krow = kv.k + (((size_t)page * kv.kv_heads + kv.kvh) * kv.page_size + (key % kv.page_size)) * D + 4 * g;
+    const int kgc = min(max(key_base + 4 * g, lo_all & ~3), hi_all & ~3);
+    int vpage = kv.table[kgc / kv.page_size];
+    vpage = min(max(vpage, 0), kv.n_pages - 1);
+    const bf16_t* vbase = kv.v + ((size_t)vpage * kv.kv_heads + kv.kvh) * kv.page_size * D + (kgc % kv.page_size);
+#pragma unroll
+    for (int dk = 0; dk < ND; ++dk) r.k[dk] = *reinterpret_cast<const s16x4*>(krow + dk * 16);
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt)
+        r.v[dt] = *reinterpret_cast<const s16x4*>(vbase + (size_t)(dt * 16 + c) * kv.page_size);
+}
+
+// One softmax step over a loaded tile. [lo_q, hi_q] is the key range of this
+// lane's query. `full`: every key of the tile is inside every query's range,
+// so no masking is needed.
+template <int ND>
+__device__ __forceinline__ void attn_tile(WaveState<ND>& st, const TileRegs<ND>& r, int key_base, int lo_q, int hi_q,
+                                          int lo_all, int hi_all, bool full, float scale, int lane) {
+    const int g = lane >> 4;
+    // ---- scores
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int dk = 0; dk < ND; ++dk) {
-        const s16x4 a = *reinterpret_cast<const s16x4*>(krow + dk * 16);
-        s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, st.q[dk], s, 0, 0, 0);
-    }
+    for (int dk = 0; dk < ND; ++dk) s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(r.k[dk], st.q[dk], s, 0, 0, 0);
     const int kg = key_base + 4 * g;          // this lane's 4 keys: kg .. kg+3
     float sv[4];
 #pragma unroll
@@ -74,22 +96,18 @@ __device__ __forceinline__ void attn_tile(WaveState<ND>& st, const Paged& kv, in
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const float p = (sv[i] == -INFINITY) ? 0.f : __expf(sv[i] - m_new);
-        const bf16_t r = f32_to_bf16(p);
-        pb[i] = (short)r;
-        psum += bf16_to_f32(r);               // the denominator sums what the product uses
+        const bf16_t rb = f32_to_bf16(p);
+        pb[i] = (short)rb;
+        psum += bf16_to_f32(rb);              // the denominator sums what the product uses
     }
     psum += __shfl_xor(psum, 16, WAVE);
     psum += __shfl_xor(psum, 32, WAVE);
     st.l = st.l * corr + psum;
     st.m = m_new;
     // ---- weighted values
-    const int kgc = min(max(kg, lo_all & ~3), hi_all & ~3);
-    int vpage = kv.table[kgc / kv.page_size];
-    vpage = min(max(vpage, 0), kv.n_pages - 1);
-    const bf16_t* vbase = kv.v + ((size_t)vpage * kv.kv_heads + kv.kvh) * kv.page_size * D + (kgc % kv.page_size);
 #pragma unroll
     for (int dt = 0; dt < ND; ++dt) {
-        s16x4 a = *reinterpret_cast<const s16x4*>(vbase + (size_t)(dt * 16 + c) * kv.page_size);
+        s16x4 a = r.v[dt];
         if (!full) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -114,17 +132,21 @@ __device__ __forceinline__ void load_q(WaveState<ND>& st, const bf16_t* __restri
 
 // ---------------------------------------------------------------- decode
 // grid (split, kv head x passes of 16 query heads, decode row). The four waves
-// of a block take the split's key tiles in turn; their partial results meet in
-// LDS and are merged in wave order; one partial (max, sum, O) per split goes to
-// scratch for the merge kernel.
+// of a block take the split's key tiles in turn, each with the loads of its
+// tiles in flight before the first product; their partial results meet in LDS
+// and are merged in wave order; one partial (max, sum, O) per split goes to
+// scratch for the merge kernel. With a single split the block writes the
+// normalised result itself and no merge follows.
 template <int ND>
 __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_decode(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
-    float* __restrict__ part_o, float* __restrict__ part_ml, const int32_t* __restrict__ rows,
-    const int32_t* __restrict__ seg_start, const int32_t* __restrict__ positions,
+    float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out,
+    const int32_t* __restrict__ rows, const int32_t* __restrict__ seg_start, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int n_pages,
     float scale, int window, int n_splits) {
     constexpr int D = ND * 16;
+    constexpr int TILES = DEC_SPLIT / (MFMA_WAVES * 16);   // tiles a wave takes at most
+    constexpr int DEPTH = ND <= 4 ? TILES : 2;             // of which this many are loaded ahead
     __shared__ float sm[MFMA_WAVES][16], sl[MFMA_WAVES][16];
     __shared__ float so[MFMA_WAVES][16][D + 1];
     const int split = blockIdx.x, ri = blockIdx.z;
@@ -146,9 +168,22 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_decode(
     load_q<ND>(st, q + ((size_t)t * heads + head) * D, qvalid, lane);
     Paged kv{k_cache, v_cache, block_table + (size_t)row * table_stride, page_size, kv_heads, kvh, n_pages};
     const int hi_q = qvalid ? pos : -1;
-    for (int kb = k_begin + wave * 16; kb < k_end; kb += MFMA_WAVES * 16) {
-        const bool full = kb >= lo && kb + 15 <= pos;
-        attn_tile<ND>(st, kv, kb, lo, hi_q, lo, pos, full, scale, lane);
+#pragma unroll
+    for (int j0 = 0; j0 < TILES; j0 += DEPTH) {
+        TileRegs<ND> regs[DEPTH];
+#pragma unroll
+        for (int j = 0; j < DEPTH; ++j) {
+            const int kb = k_begin + (wave + (j0 + j) * MFMA_WAVES) * 16;
+            if (kb < k_end) load_tile<ND>(regs[j], kv, kb, lo, pos, lane);
+        }
+#pragma unroll
+        for (int j = 0; j < DEPTH; ++j) {
+            const int kb = k_begin + (wave + (j0 + j) * MFMA_WAVES) * 16;
+            if (kb < k_end) {
+                const bool full = kb >= lo && kb + 15 <= pos;
+                attn_tile<ND>(st, regs[j], kb, lo, hi_q, lo, pos, full, scale, lane);
+            }
+        }
     }
     if (g == 0) {
         sm[wave][c] = st.m;
@@ -172,7 +207,12 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_decode(
             acc += so[w][qc][d] * f;
             ls += sl[w][qc] * f;
         }
-        const size_t slot = ((size_t)ri * heads + kvh * G + pass * 16 + qc) * n_splits + split;
+        const int head_out = kvh * G + pass * 16 + qc;
+        if (n_splits == 1) {
+            out[((size_t)t * heads + head_out) * D + d] = f32_to_bf16(ls > 0.f ? acc / ls : 0.f);
+            continue;
+        }
+        const size_t slot = ((size_t)ri * heads + head_out) * n_splits + split;
         part_o[slot * D + d] = acc;
         if (d == 0) {
             part_ml[slot * 2] = ms;
@@ -183,12 +223,14 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_decode(
 
 // One wave per (decode row, head): merges the splits in split order. Lane s
 // first fetches split s's (max, sum), so the weights of up to 64 splits are
-// known after one round trip; the sums over splits then run with the loads of
-// several splits in flight.
+// known after one round trip; the partial outputs then come eight splits at a
+// time, all loads of a group issued before the first is used, and are added in
+// split order.
 __global__ void k_attn_decode_merge(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                     bf16_t* __restrict__ out, const int32_t* __restrict__ rows,
                                     const int32_t* __restrict__ seg_start, const int32_t* __restrict__ positions,
                                     int heads, int head_dim, int n_splits, int window) {
+    constexpr int GROUP = 8, NJ = 2;          // head_dim <= NJ * WAVE
     const int ri = blockIdx.x / heads, head = blockIdx.x % heads;
     const int lane = threadIdx.x;
     const int t = seg_start[rows[ri]];
@@ -202,9 +244,9 @@ __global__ void k_attn_decode_merge(const float* __restrict__ part_o, const floa
         ms = fmaxf(ms, s <= s_hi ? part_ml[(base + s) * 2] : -INFINITY);
     }
     ms = wave_max(ms);
-    float acc[8];
+    float acc[NJ];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    for (int j = 0; j < NJ; ++j) acc[j] = 0.f;
     float ls = 0.f;
     for (int s0 = s_lo; s0 <= s_hi; s0 += WAVE) {
         const int s = s0 + lane;
@@ -214,23 +256,32 @@ __global__ void k_attn_decode_merge(const float* __restrict__ part_o, const floa
             wgt = (m == -INFINITY) ? 0.f : __expf(m - ms);
             l = part_ml[(base + s) * 2 + 1] * wgt;
         }
-        // sum in split order: lane by lane
         const int n_here = min(WAVE, s_hi - s0 + 1);
-        for (int k = 0; k < n_here; ++k) ls += __shfl(l, k, WAVE);
-#pragma unroll 4
-        for (int k = 0; k < n_here; ++k) {
-            const float wk = __shfl(wgt, k, WAVE);
-            const float* po = part_o + (base + s0 + k) * head_dim;
+        for (int k0 = 0; k0 < n_here; k0 += GROUP) {
+            float v[GROUP][NJ];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int d = lane + j * WAVE;
-                if (d < head_dim) acc[j] += po[d] * wk;
+            for (int i = 0; i < GROUP; ++i) {
+                const float* po = part_o + (base + s0 + min(k0 + i, n_here - 1)) * head_dim;
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    const int d = lane + j * WAVE;
+                    v[i][j] = d < head_dim ? po[d] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < GROUP; ++i) {
+                const bool on = k0 + i < n_here;
+                const int src = min(k0 + i, WAVE - 1);
+                const float wk = on ? __shfl(wgt, src, WAVE) : 0.f;
+                ls += on ? __shfl(l, src, WAVE) : 0.f;
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) acc[j] += v[i][j] * wk;
             }
         }
     }
     const float inv = ls > 0.f ? 1.0f / ls : 0.f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < NJ; ++j) {
         const int d = lane + j * WAVE;
         if (d < head_dim) out[((size_t)t * heads + head) * head_dim + d] = f32_to_bf16(acc[j] * inv);
     }
@@ -473,9 +524,10 @@ extern "C" int imparo_attention_decode(const void* q, const void* k_cache, const
     const int G = heads / kv_heads;
     dim3 grid(n_splits, kv_heads * ((G + 15) / 16), n_rows);
     DISPATCH_ND(head_dim / 16, (k_attn_decode<ND><<<grid, MFMA_WAVES * 64, 0, s>>>(
-        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, part_o, part_ml, rows, seg_start, positions,
-        block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, n_splits)));
+        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, part_o, part_ml, (bf16_t*)out, rows, seg_start,
+        positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, n_splits)));
     if (launch_status()) return IMPARO_LAUNCH_FAILED;
+    if (n_splits == 1) return IMPARO_OK;
     k_attn_decode_merge<<<n_rows * heads, 64, 0, s>>>(part_o, part_ml, (bf16_t*)out, rows, seg_start, positions, heads,
                                                       head_dim, n_splits, window);
     return launch_status();
