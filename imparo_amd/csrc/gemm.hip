@@ -546,9 +546,10 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, const float* bias, T
         k_gemm_bf16_skinny<TOut, MT, 8><<<grid, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
 }
 
-// Into how many slices of K a few-row product may be cut when its consumer adds the slices:
-// a weight with few rows and a long K (the feed-forward's way back) gives too few blocks
-// otherwise. One slice per 2048 of K, for at most 64 rows and at most 4096 weight rows.
+// Into how many slices of K a product may be cut when its consumer adds the slices. A weight
+// with few rows gives too few blocks to keep the memory system busy otherwise (one CU draws
+// about 50 GB/s at best, so it takes all of them): the measured optimum, with cold weights,
+// is about 256 blocks.
 extern "C" int imparo_gemm_slices(int m, int n, int k, int dtype) {
     if (dtype != IMPARO_BF16) return 1;
     if (m > 64) {
@@ -559,93 +560,149 @@ extern "C" int imparo_gemm_slices(int m, int n, int k, int dtype) {
         while (slices < 4 && tiles * slices * 2 <= 512 && k / (slices * 2) >= 1024) slices *= 2;
         return slices;
     }
-    if (n > 4096 || k < 4096) return 1;
-    return (k + 2047) / 2048;
+    if (n > 4096) return 1;
+    if (m <= 16) {            // one block per 16 weight rows
+        if (k >= 4096) return (k + 2047) / 2048;
+        return k >= 2048 ? 2 : 1;
+    }
+    return k >= 2048 ? 4 : (k >= 1024 ? 2 : 1);   // one block per 32 weight rows
 }
 
-// ------------------------------------------------------------------ bfloat16, few rows, many weight rows
-// For weights with so many rows that one block per 128 of them fills the chip
-// (the output head): a block of 8 waves takes 128 weight rows (16 per wave) and
-// walks all of K. The activation chunk [rows x 128] is staged in LDS once per
-// block and shared by the 8 waves, so activations cost an eighth of the L2
-// traffic they cost when every wave fetches its own; every output element is
-// summed by one wave in k order.
+// ------------------------------------------------------------------ bfloat16, some rows (17..64)
+// A block of ST_WAVES waves takes 16 weight rows per wave and up to 16*MT
+// activation rows, and walks its part of K in chunks of 128. The activation
+// chunk is staged in LDS once per block and shared by the waves (with more
+// than 16 rows every wave fetching its own activations costs several times the
+// weight traffic); weights go from memory straight into the MFMA operand
+// registers. Loads run three chunks ahead of the products: four register sets
+// in rotation, the activation part of a set goes to LDS one step before its
+// chunk is multiplied. With slices (gridDim.y > 1) block (x, y) sums K range
+// [y * k_per, (y+1) * k_per) into Y + y * M * N and the consumer adds the slices.
 #define ST_BK 128
 #define ST_LD (ST_BK + 8)   // LDS row stride in elements: 272 bytes, 16 rows of 16-byte reads on distinct banks
+
+template <int XP>
+struct StreamSet {
+    Frag8 w[4];       // this wave's weight rows, chunk columns s*32 + g*8
+    uint4 x[XP];      // this thread's pieces of the activation chunk
+};
 
 template <typename TOut, int MT, int ST_WAVES>
 __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, const float* __restrict__ bias,
-    TOut* __restrict__ Y, int M, int N, int K, int epilogue) {
+    TOut* __restrict__ Y, int M, int N, int K_all, int k_per, int epilogue) {
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16 * ST_LD];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.x * (ST_WAVES * 16) + wave * 16;
-    const bf16_t* wrow = W + (size_t)min(n0 + r16, N - 1) * K + g * 8;
+    const int k_lo = blockIdx.y * k_per;
+    const int K = min(K_all, k_lo + k_per) - k_lo;       // this block's part of K, re-based to 0
+    X += k_lo;
+    W += k_lo;
+    Y += (size_t)blockIdx.y * M * N;
+    if (blockIdx.y > 0) bias = nullptr;                  // the bias belongs to one slice only
+    const bf16_t* wrow = W + (size_t)min(n0 + r16, N - 1) * K_all;
 
-    // staging of the activation chunk: MT*16 rows x 16 pieces of 16 bytes
+    // the activation chunk: MT*16 rows x 16 pieces of 16 bytes, XP pieces per thread
     constexpr int PIECES = MT * 16 * (ST_BK / 8);
-    constexpr int PER_THREAD = (PIECES + ST_WAVES * 64 - 1) / (ST_WAVES * 64);
-    auto stage_load = [&](int k0, uint4 (&r)[PER_THREAD]) {
+    constexpr int XP = (PIECES + ST_WAVES * 64 - 1) / (ST_WAVES * 64);
+    const bf16_t* xsrc[XP];
+    int xdst[XP], xkc[XP];
 #pragma unroll
-        for (int j = 0; j < PER_THREAD; ++j) {
-            const int p = tid + j * ST_WAVES * 64;
-            const int row = p / (ST_BK / 8), kc = (p % (ST_BK / 8)) * 8;
-            const bool in = p < PIECES && k0 + kc < K;
-            r[j] = in ? *reinterpret_cast<const uint4*>(X + (size_t)min(row, M - 1) * K + k0 + kc)
-                      : make_uint4(0, 0, 0, 0);
-        }
+    for (int j = 0; j < XP; ++j) {
+        const int p = min(tid + j * ST_WAVES * 64, PIECES - 1);
+        const int row = p / (ST_BK / 8);
+        xkc[j] = (p % (ST_BK / 8)) * 8;
+        xsrc[j] = X + (size_t)min(row, M - 1) * K_all;
+        xdst[j] = row * ST_LD + xkc[j];
+    }
+    const int nk = (K + ST_BK - 1) / ST_BK;
+    // The walk along K is free of branches: a load under a branch, or a step under one, makes
+    // the compiler wait for every load in flight at the next use of any. So every load is
+    // issued unconditionally from an address clamped into the row, what a chunk reads at or
+    // beyond K is zeroed before use, and the number of steps is rounded up to the four
+    // register sets (a chunk past the end reads the last one again and counts as zeros).
+    // Blocks start their walk at different chunks and wrap around: rows are a power of two
+    // apart in memory, so blocks in step would ask the same few cache channels for the same
+    // activation chunk at the same time.
+    const int rot = (blockIdx.x + blockIdx.y) % nk;
+    auto chunk_of = [&](int kt) {                        // kt >= nk: past the end
+        const int c = kt + rot;
+        return kt >= nk ? kt : (c >= nk ? c - nk : c);
     };
-    auto stage_store = [&](int buf, const uint4 (&r)[PER_THREAD]) {
+    auto fetch = [&](int kt, StreamSet<XP>& f) {
+        const int k0 = min(chunk_of(kt), nk - 1) * ST_BK;
 #pragma unroll
-        for (int j = 0; j < PER_THREAD; ++j) {
-            const int p = tid + j * ST_WAVES * 64;
-            if (p < PIECES) {
-                const int row = p / (ST_BK / 8), kc = (p % (ST_BK / 8)) * 8;
-                *reinterpret_cast<uint4*>(&xs[buf][row * ST_LD + kc]) = r[j];
-            }
-        }
-    };
-    auto load_w = [&](int k0, Frag8 (&f)[4]) {
+        for (int s2 = 0; s2 < 4; ++s2)
+            f.w[s2].u = *reinterpret_cast<const uint4*>(wrow + min(k0 + s2 * 32 + g * 8, K - 8));
 #pragma unroll
-        for (int s2 = 0; s2 < 4; ++s2) {
-            const int k = k0 + s2 * 32;
-            f[s2].u = (k + g * 8 < K) ? *reinterpret_cast<const uint4*>(wrow + k) : make_uint4(0, 0, 0, 0);
-        }
+        for (int j = 0; j < XP; ++j) f.x[j] = *reinterpret_cast<const uint4*>(xsrc[j] + min(k0 + xkc[j], K - 8));
     };
-
+    auto zero_if = [](bool out, uint4 v) {
+        return make_uint4(out ? 0u : v.x, out ? 0u : v.y, out ? 0u : v.z, out ? 0u : v.w);
+    };
+    auto stash = [&](int kt, int buf, const StreamSet<XP>& f) {
+        const int k0 = chunk_of(kt) * ST_BK;
+#pragma unroll
+        for (int j = 0; j < XP; ++j)     // threads beyond the last piece repeat it: same value, same place
+            *reinterpret_cast<uint4*>(&xs[buf][xdst[j]]) = zero_if(k0 + xkc[j] >= K, f.x[j]);
+    };
     f32x4 acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    uint4 xr[PER_THREAD];
-    Frag8 wcur[4], wnxt[4];
-    stage_load(0, xr);
-    load_w(0, wcur);
-    stage_store(0, xr);
-    __syncthreads();
-    int buf = 0;
-    for (int k0 = 0; k0 < K; k0 += ST_BK) {
-        const int k1 = k0 + ST_BK;
-        if (k1 < K) {
-            stage_load(k1, xr);
-            load_w(k1, wnxt);
-        }
+    // The activation fragments of K-sub-step s2+1 are read from LDS while the products of
+    // sub-step s2 run: a block may be alone on its CU, with nothing else to hide the LDS latency.
+    auto read_x = [&](int buf, int s2, Frag8 (&xf)[MT]) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
+            xf[mt].u = *reinterpret_cast<const uint4*>(&xs[buf][(mt * 16 + r16) * ST_LD + s2 * 32 + g * 8]);
+    };
+    auto multiply = [&](const Frag8& wf, const Frag8 (&xf)[MT]) {
 #pragma unroll
-            for (int s2 = 0; s2 < 4; ++s2) {
-                Frag8 xf;
-                xf.u = *reinterpret_cast<const uint4*>(&xs[buf][(mt * 16 + r16) * ST_LD + s2 * 32 + g * 8]);
-                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wcur[s2].v, xf.v, acc[mt], 0, 0, 0);
-            }
-        if (k1 < K) {
-            stage_store(buf ^ 1, xr);
-#pragma unroll
-            for (int s2 = 0; s2 < 4; ++s2) wcur[s2] = wnxt[s2];
-        }
+        for (int mt = 0; mt < MT; ++mt)
+            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, xf[mt].v, acc[mt], 0, 0, 0);
+    };
+    auto compute = [&](int kt, int buf, const StreamSet<XP>& f) {
+        const int k0 = chunk_of(kt) * ST_BK + g * 8;
+        Frag8 xa[MT], xb[MT], wf;
+        read_x(buf, 0, xa);
+        read_x(buf, 1, xb);
+        __builtin_amdgcn_sched_barrier(0);
+        wf.u = zero_if(k0 >= K, f.w[0].u);
+        multiply(wf, xa);
+        read_x(buf, 2, xa);
+        __builtin_amdgcn_sched_barrier(0);
+        wf.u = zero_if(k0 + 32 >= K, f.w[1].u);
+        multiply(wf, xb);
+        read_x(buf, 3, xb);
+        __builtin_amdgcn_sched_barrier(0);
+        wf.u = zero_if(k0 + 64 >= K, f.w[2].u);
+        multiply(wf, xa);
+        __builtin_amdgcn_sched_barrier(0);
+        wf.u = zero_if(k0 + 96 >= K, f.w[3].u);
+        multiply(wf, xb);
+    };
+    // chunk i: the next chunk's activations go from their registers to LDS, the set that
+    // chunk i-1 used takes the loads of chunk i+3, then chunk i is multiplied
+    auto step = [&](int i, const StreamSet<XP>& cur, const StreamSet<XP>& next, StreamSet<XP>& refill) {
+        const int buf = i & 1;
+        stash(i + 1, buf ^ 1, next);
+        fetch(i + 3, refill);
+        compute(i, buf, cur);
         __syncthreads();
-        buf ^= 1;
+    };
+    StreamSet<XP> s0, s1, s2, s3;
+    fetch(0, s0);
+    fetch(1, s1);
+    fetch(2, s2);
+    stash(0, 0, s0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; kt += 4) {
+        step(kt, s0, s1, s3);
+        step(kt + 1, s1, s2, s0);
+        step(kt + 2, s2, s3, s1);
+        step(kt + 3, s3, s0, s2);
     }
     // D layout of the 16x16 tile: lane holds column lane%16 (an activation row), rows 4*(lane/16)+i (weight rows)
     const int nq = n0 + g * 4;
@@ -668,26 +725,28 @@ __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
     }
 }
 
-// Waves per block for the wide kernel, or 0 for "use the K-split kernel". Measured with cold
-// weights (they never stay in cache between decode steps): the wide kernel wins from about
-// 12k weight rows on, with 2 waves a block, and with 4 from about 32k rows on; below that
-// its walk along K (one chunk of 128 per round trip) costs more than shared activations save.
-static int stream_waves(int n) {
-    if (n >= 32768) return 4;
-    if (n >= 12288) return 2;
+// Which kernel takes a product of up to 64 rows: 0 for the K-split kernel, else the waves per
+// block of the shared-activation kernel. Measured with cold weights (they never stay in cache
+// between decode steps): from about 12k weight rows on the shared-activation kernel wins at
+// any number of rows; below that it wins when every wave would fetch its own copy of more
+// than 16 activation rows, or when K is long.
+static int stream_waves(int m, int n, int k) {
+    if (n >= 12288) return 4;
+    if (m > 16 || k >= 4096) return 2;
     return 0;
 }
 
 template <typename TOut, int MT>
 static void launch_stream(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k,
-                          int epilogue, int nw, hipStream_t s) {
-    const unsigned blocks = (unsigned)((n + nw * 16 - 1) / (nw * 16));
+                          int epilogue, int nw, int slices, hipStream_t s) {
+    const int k_per = ((k + slices - 1) / slices + ST_BK - 1) / ST_BK * ST_BK;
+    dim3 grid((unsigned)((n + nw * 16 - 1) / (nw * 16)), (unsigned)((k + k_per - 1) / k_per));
     if (nw == 8)
-        k_gemm_bf16_stream<TOut, MT, 8><<<blocks, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+        k_gemm_bf16_stream<TOut, MT, 8><<<grid, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
     else if (nw == 4)
-        k_gemm_bf16_stream<TOut, MT, 4><<<blocks, 4 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+        k_gemm_bf16_stream<TOut, MT, 4><<<grid, 4 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
     else
-        k_gemm_bf16_stream<TOut, MT, 2><<<blocks, 2 * 64, 0, s>>>(x, w, bias, y, m, n, k, epilogue);
+        k_gemm_bf16_stream<TOut, MT, 2><<<grid, 2 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
 }
 
 // The 256x256 tile (one block per CU) pays once its tiles keep most of the chip's 256 CUs busy:
@@ -700,19 +759,17 @@ static bool big_tile_pays(int m, int n, int k) {
 template <typename TOut>
 static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
                        int force, int slices, hipStream_t s) {
-    // 17..64 rows: sharing the activations between the waves of a block matters more than anything
-    // else, if the weight has rows enough for enough blocks. (Up to 16 rows the K-split kernel keeps
-    // more loads in flight and wins.) `force` (for measurements): 1 = K-split kernel, 2/4/8 = wide with that many waves
-    int nw = (m > 16 && slices == 1) ? stream_waves(n) : 0;
+    // `force` (for measurements): 1 = K-split kernel, 2/4/8 = shared activations with that many waves
+    int nw = stream_waves(m, n, k);
     if (force == 1) nw = 0;
     if (force == 2 || force == 4 || force == 8) nw = force;
     if (m <= 64 && nw) {
         if (m <= 16)
-            launch_stream<TOut, 1>(x, w, bias, y, m, n, k, epilogue, nw, s);
+            launch_stream<TOut, 1>(x, w, bias, y, m, n, k, epilogue, nw, slices, s);
         else if (m <= 32)
-            launch_stream<TOut, 2>(x, w, bias, y, m, n, k, epilogue, nw, s);
+            launch_stream<TOut, 2>(x, w, bias, y, m, n, k, epilogue, nw, slices, s);
         else
-            launch_stream<TOut, 4>(x, w, bias, y, m, n, k, epilogue, nw, s);
+            launch_stream<TOut, 4>(x, w, bias, y, m, n, k, epilogue, nw, slices, s);
         return launch_status();
     }
     if (m <= 64) {
@@ -740,17 +797,23 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
 }
 
 static int g_force_few_row_kernel = 0;
+static int g_force_slices = 0;
 
-// For measurements only: 0 lets the library choose the few-row kernel, 1 forces the K-split
-// kernel, 2, 4 or 8 the wide kernel with that many waves.
-extern "C" void imparo_gemm_force_kernel(int which) { g_force_few_row_kernel = which; }
+// For measurements only: 0 lets the library choose the kernel, 1 forces the K-split kernel,
+// 2, 4 or 8 the shared-activation kernel with that many waves, 256/257 the large tiles;
+// plus 1000 times a number of K slices that imparo_gemm then accepts whatever the shape.
+extern "C" void imparo_gemm_force_kernel(int which) {
+    g_force_slices = which / 1000;
+    g_force_few_row_kernel = which % 1000;
+}
 
 extern "C" int imparo_gemm(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
                            int m, int n, int k, int epilogue, int slices, imparo_stream stream) {
     if (!x || !w || !y || m < 0 || n <= 0 || k <= 0) return IMPARO_BAD_ARGUMENT;
     if (slices < 1) return IMPARO_BAD_ARGUMENT;
     // slices: only what imparo_gemm_slices allows, float32 out, no epilogue that is not linear
-    if (slices > 1 && (slices != imparo_gemm_slices(m, n, k, dtype) || out_dtype != IMPARO_F32 || epilogue != EPI_NONE))
+    const int slices_ok = g_force_slices ? g_force_slices : imparo_gemm_slices(m, n, k, dtype);
+    if (slices > 1 && (slices != slices_ok || out_dtype != IMPARO_F32 || epilogue != EPI_NONE))
         return IMPARO_BAD_ARGUMENT;
     if (epilogue != EPI_NONE && epilogue != EPI_SWIGLU) return IMPARO_BAD_ARGUMENT;
     if (epilogue == EPI_SWIGLU && (n % 2 != 0)) return IMPARO_BAD_ARGUMENT;

@@ -83,7 +83,9 @@ def test_gemm_in_slices_of_k_and_the_norm_that_adds_them(m):
     n, k = 200, 4096 + 264
     x, w, b = rnd(m, k, seed=1).to(torch.bfloat16), rnd(n, k, seed=2, scale=0.1).to(torch.bfloat16), rnd(n, seed=3)
     slices = ops().gemm_slices(m, n, k, torch.bfloat16)
-    assert slices == 3 and ops().gemm_slices(m, n, 2048, torch.bfloat16) == 1
+    # up to 16 rows: one slice per 2048 of K; 17..64 rows: four
+    assert slices == (3 if m <= 16 else 4) and ops().gemm_slices(m, n, 2048, torch.bfloat16) == (2 if m <= 16 else 4)
+    assert ops().gemm_slices(m, 8192, k, torch.bfloat16) == 1       # a weight with many rows fills the chip by itself
     assert ops().gemm_slices(m, n, k, torch.float32) == 1
     # many rows and few tiles: the 128x128 kernel takes slices too (at least 1024 of K each, at most 4)
     assert ops().gemm_slices(300, n, k, torch.bfloat16) == 4 and ops().gemm_slices(300, n, 2048, torch.bfloat16) == 2
@@ -115,6 +117,24 @@ def test_gemm_in_slices_of_k_and_the_norm_that_adds_them(m):
     from imparo_amd.kernels import KernelArgumentError
     with pytest.raises(KernelArgumentError, match="slices"):
         ops().gemm(x.to(DEV), w.to(DEV), torch.empty(2, m, n, device=DEV))
+
+
+@pytest.mark.parametrize("m", [3, 16, 24, 64])
+@pytest.mark.parametrize("k", [264, 1024])
+def test_gemm_with_many_weight_rows(m, k):
+    """From about 12k weight rows on, few-row products go to the kernel that shares the
+    activations between the waves of a block: ragged K, a last block that is cut, bias, SwiGLU."""
+    n = 12288 + 2 * 37
+    x, w, b = rnd(m, k, seed=1).to(torch.bfloat16), rnd(n, k, seed=2, scale=0.1).to(torch.bfloat16), rnd(n, seed=3)
+    y = x.double() @ w.double().t() + b.double()
+    out = torch.full((m, n), float("nan"), device=DEV)
+    ops().gemm(x.to(DEV), w.to(DEV), out, bias=b.to(DEV))
+    assert (out.cpu().double() - y).abs().max() <= 1e-6 * math.sqrt(k) * y.abs().max()
+    act = torch.full((m, n // 2), float("nan"), device=DEV)
+    ops().gemm(x.to(DEV), w.to(DEV), act, bias=b.to(DEV), swiglu=True)
+    # silu(gate) * up: an accumulation error e in gate or up shows as at most about e * max|y|
+    ref = y[:, 0::2] / (1 + torch.exp(-y[:, 0::2])) * y[:, 1::2]
+    assert (act.cpu().double() - ref).abs().max() <= 1e-6 * math.sqrt(k) * y.abs().max() * max(1.0, y.abs().max().item())
 
 
 def test_gemm_refuses_what_it_cannot_take():
