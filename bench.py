@@ -3,8 +3,10 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-A step is one decode step of the whole batch through the engine's own loop:
-step function, sampling kernel, the sampled tokens read back and fed again.
+A step is one decode step of the whole batch through the engine's own loop, as
+generation runs it: step function, sampling kernel, the sampled tokens fed to
+the next step on the device and read back by the host one step late (while the
+GPU runs that next step).
 Default: batch 8, every request's context ending at 4096 tokens, random
 bfloat16 weights (seed 2), synthetic token ids uniform over the vocabulary.
 The JSON line also carries a 2,048-token prefill, the decode step's HBM
@@ -53,7 +55,7 @@ def model_numbers(cfg):
 def decode_run(engine, sampler, batch, context, steps, warmup, vocab, seed):
     """Fills `batch` requests up to context - steps - warmup tokens, then times `steps` decode steps."""
     import torch
-    from imparo_amd.engine import StepEntry
+    from imparo_amd.engine import DeviceToken, StepEntry
     g = torch.Generator().manual_seed(seed)
     start = context - steps - warmup
     ids = [f"d{i}" for i in range(batch)]
@@ -65,18 +67,22 @@ def decode_run(engine, sampler, batch, context, steps, warmup, vocab, seed):
             out = engine.step([StepEntry(rid, prompt[lo:hi], [hi - lo - 1] if hi == start else [])])
         last = out if last is None else torch.cat([last, out])
     temps, unis = [0.0] * batch, [0.0] * batch
-    tokens = sampler.pick(last, temps, unis)
+    picked = sampler.pick_async(last, temps, unis)
 
-    def one_step(tokens):
-        logits = engine.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, tokens)])
-        return sampler.pick(logits, temps, unis)
+    def one_step(picked):
+        logits = engine.step([StepEntry(rid, [DeviceToken(picked.on_device, i)], [0]) for i, rid in enumerate(ids)])
+        following = sampler.pick_async(logits, temps, unis)
+        picked.tokens()                                # the step before's tokens, read while this one runs
+        return following
 
     for _ in range(warmup):
-        tokens = one_step(tokens)
+        picked = one_step(picked)
+    picked.tokens()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        tokens = one_step(tokens)
+        picked = one_step(picked)
+    picked.tokens()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     for rid in ids:

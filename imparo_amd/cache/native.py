@@ -30,11 +30,13 @@ _SIGNATURES = {
     "imparo_cache_pages_needed": ([P, c_int64, I, P], I), "imparo_cache_first_needed_page": ([P, I, I], I),
     "imparo_cache_n_live": ([P], I), "imparo_cache_live_requests": ([P, P, I], I), "imparo_cache_check": ([P], I),
     "imparo_cache_pack": ([P, I, P, P, P, P, P, I, P, c_int64, P], c_int64),
+    "imparo_cache_begin_step": ([P, I, P, P, P, P, P, I, I, P, P], I),
+    "imparo_cache_abort_step": ([P, I, P, P], I), "imparo_cache_end_step": ([P, I, P, P], I),
     "imparo_sched_new": ([P, I, I, I], P), "imparo_sched_delete": ([P], None),
     "imparo_sched_add": ([P, c_int64, I, I], I),
     "imparo_sched_plan": ([P, P, P, P, P, I, P, P, I, P], I),
     "imparo_sched_advance": ([P], None), "imparo_sched_token": ([P, c_int64, I], I),
-    "imparo_sched_drop_waiting_head": ([P, P], I),
+    "imparo_sched_drop_waiting_head": ([P, P], I), "imparo_sched_retract": ([P, c_int64], I),
     "imparo_sched_n_waiting": ([P], I), "imparo_sched_n_running": ([P], I),
     "imparo_sched_waiting": ([P, P, I], I), "imparo_sched_running": ([P, P, I], I),
 }
@@ -42,6 +44,7 @@ EV_ADMIT, EV_WAIT, EV_PREEMPT, EV_FAIL = 1, 2, 3, 4
 
 E_OUT_OF_PAGES, E_NOT_LIVE, E_ALREADY_LIVE, E_SHRINK, E_DOUBLE_FREE, E_RANGE, E_BUSY, E_CAPACITY = range(-1, -9, -1)
 E_LOST_PAGE, E_SHARED_PAGE, E_SLOTS = -9, -10, -11
+E_TWICE, E_EMPTY, E_POSITIONS, E_TOKEN, E_WANT = -12, -13, -14, -15, -16
 
 
 def host_library() -> ctypes.CDLL:

@@ -14,6 +14,7 @@ from __future__ import annotations
 
 import ctypes
 from dataclasses import dataclass
+from itertools import chain
 from typing import Dict, Hashable, Iterator, List, Optional, Sequence, Tuple, Union
 
 import numpy as np
@@ -333,6 +334,55 @@ class CacheManager:
         if rc == N.E_SLOTS:
             raise CacheError("state slots are lost or held twice")
 
+    # ------------------------------------------------------------ a step, as flat arrays
+    def batch(self, requests: Sequence[Hashable], token_lists: Sequence[Sequence[int]],
+              want_lists: Sequence[Sequence[int]]) -> "StepBatch":
+        """The rows of a step as the native side takes them: handles, counts,
+        and all token ids and wanted places end to end."""
+        R = len(requests)
+        b = StepBatch()
+        b.requests = list(requests)
+        b.reqs = np.fromiter(map(self.handle, requests), dtype=np.int64, count=R)
+        b.n_tok = np.fromiter(map(len, token_lists), dtype=np.int32, count=R)
+        b.n_want = np.fromiter(map(len, want_lists), dtype=np.int32, count=R)
+        b.T, b.W = int(b.n_tok.sum()), int(b.n_want.sum())
+        try:
+            b.tokens = np.fromiter(chain.from_iterable(token_lists), dtype=np.int32, count=b.T)
+            b.want = np.fromiter(chain.from_iterable(want_lists), dtype=np.int32, count=b.W)
+        except (OverflowError, TypeError, ValueError) as e:
+            raise CacheError(f"token ids and wanted places must be integers that fit 32 bits: {e}") from None
+        b.new_slots = np.full(R, -1, dtype=np.int32)
+        b.widest = 1
+        b.device_tokens = None
+        return b
+
+    def begin_step(self, b: "StepBatch", vocab: int, max_position: int) -> Tuple[int, int]:
+        """Checks the batch, admits its new requests and reserves every row's
+        pages, all or nothing. Returns (0, -1) or (the native code of what is
+        wrong, the row); raises OutOfPages. b.new_slots then names the slots
+        whose device state the caller has to clear, b.widest the widest block
+        table in pages."""
+        info = np.zeros(3, dtype=np.int32)
+        rc = self._lib.imparo_cache_begin_step(self._c, len(b.requests), b.reqs.ctypes.data, b.n_tok.ctypes.data,
+                                               b.tokens.ctypes.data, b.n_want.ctypes.data, b.want.ctypes.data,
+                                               vocab, max_position, b.new_slots.ctypes.data, info.ctypes.data)
+        row = int(info[0])
+        if rc == N.E_OUT_OF_PAGES:
+            req = b.requests[row]
+            if info[2]:
+                raise OutOfPages(f"all {self.n_slots} request slots are in use")
+            raise OutOfPages(f"request {req!r} needs pages for {int(b.n_tok[row])} more positions and the pool "
+                             f"has none left")
+        b.widest = int(info[1])
+        return rc, row
+
+    def abort_step(self, b: "StepBatch") -> None:
+        self._lib.imparo_cache_abort_step(self._c, len(b.requests), b.reqs.ctypes.data, b.new_slots.ctypes.data)
+
+    def end_step(self, b: "StepBatch") -> None:
+        """The step ran: every row's request now holds its tokens; pages a window has passed are given back."""
+        self._lib.imparo_cache_end_step(self._c, len(b.requests), b.reqs.ctypes.data, b.n_tok.ctypes.data)
+
     # ------------------------------------------------------------ a step's index arrays
     LAYOUT = ("T", "R", "W", "G", "P", "n_single", "n_multi", "n_prefill_tiles", "max_seg_len", "max_context", "total")
 
@@ -342,21 +392,27 @@ class CacheManager:
         tokens | positions | row_of_token | seg_start | seg_len | slot | row
         lists | want | tables[group][row][page], and the sizes of its parts.
         Lengths are those before the step."""
-        R = len(requests)
-        reqs = np.fromiter((self._h(r) for r in requests), dtype=np.int64, count=R)
-        n_tok = np.fromiter((len(t) for t in token_lists), dtype=np.int32, count=R)
-        n_want = np.fromiter((len(w) for w in want_lists), dtype=np.int32, count=R)
-        T, W = int(n_tok.sum()), int(n_want.sum())
-        tokens = np.fromiter((t for ts in token_lists for t in ts), dtype=np.int32, count=T)
-        want = np.fromiter((w for ws in want_lists for w in ws), dtype=np.int32, count=W)
+        b = self.batch(requests, token_lists, want_lists)
+        if table_width <= 0:
+            b.widest = max([1] + [self._lib.imparo_cache_table_len(self._c, g, int(h))
+                                  for h in b.reqs for g in range(len(self.groups))])
+        return self.pack_batch(b, table_width)
+
+    def pack_batch(self, b: "StepBatch", table_width: int = 0) -> Tuple[np.ndarray, Dict[str, int]]:
+        R = len(b.requests)
         layout = np.zeros(len(self.LAYOUT), dtype=np.int32)
-        P = table_width if table_width > 0 else max(
-            [1] + [self._lib.imparo_cache_table_len(self._c, g, int(h)) for h in reqs for g in range(len(self.groups))])
-        capacity = 3 * T + 4 * R + W + len(self.groups) * R * P
+        P = table_width if table_width > 0 else b.widest
+        capacity = 3 * b.T + 4 * R + b.W + len(self.groups) * R * P
         out = np.empty(capacity, dtype=np.int32)
-        n = self._lib.imparo_cache_pack(self._c, R, reqs.ctypes.data, n_tok.ctypes.data, tokens.ctypes.data,
-                                        n_want.ctypes.data, want.ctypes.data, table_width, out.ctypes.data,
+        n = self._lib.imparo_cache_pack(self._c, R, b.reqs.ctypes.data, b.n_tok.ctypes.data, b.tokens.ctypes.data,
+                                        b.n_want.ctypes.data, b.want.ctypes.data, table_width, out.ctypes.data,
                                         capacity, layout.ctypes.data)
         if n < 0:
             raise CacheError(f"packing the step failed with code {n}")
         return out[:n], dict(zip(self.LAYOUT, layout.tolist()))
+
+
+class StepBatch:
+    """The rows of one step as flat arrays (see CacheManager.batch)."""
+    __slots__ = ("requests", "reqs", "n_tok", "n_want", "tokens", "want", "T", "W", "new_slots", "widest",
+                 "device_tokens")     # device_tokens: (source vector, places in `tokens`, indices into the source) or None

@@ -15,6 +15,12 @@ typedef void* imparo_stream;
 int imparo_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* x,
                         int n_tokens, int width, int vocab, imparo_stream stream);
 
+// ids[dst[i]] = src[src_index[i]] for i < n, clamped into [0, vocab): token ids sampled by the
+// step before that are still on the device. The caller guarantees dst[i] < len(ids) and
+// src_index[i] < len(src).
+int imparo_place_tokens(int32_t* ids, const int32_t* dst, const int32_t* src, const int32_t* src_index,
+                        int n, int vocab, imparo_stream stream);
+
 // Row-wise RMS norm. For output row i the source row is rows ? rows[i] : i.
 // If delta is given the row is x + delta[0] + delta[1] + ... first (n_delta
 // slices, each [n_x_rows, width], added in order); with write_back (rows must

@@ -29,6 +29,23 @@ extern "C" int imparo_embed_gather(const void* table, int table_dtype, const int
     return launch_status();
 }
 
+// Token ids that are still on the device (sampled by the step before, not yet read back):
+// ids[dst[i]] = src[src_index[i]], clamped into the vocabulary.
+__global__ void k_place_tokens(int32_t* __restrict__ ids, const int32_t* __restrict__ dst,
+                               const int32_t* __restrict__ src, const int32_t* __restrict__ src_index, int n,
+                               int vocab) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) ids[dst[i]] = min(max(src[src_index[i]], 0), vocab - 1);
+}
+
+extern "C" int imparo_place_tokens(int32_t* ids, const int32_t* dst, const int32_t* src, const int32_t* src_index,
+                                   int n, int vocab, imparo_stream stream) {
+    if (!ids || !dst || !src || !src_index || n < 0 || vocab <= 0) return IMPARO_BAD_ARGUMENT;
+    if (n == 0) return IMPARO_OK;
+    k_place_tokens<<<(n + 255) / 256, 256, 0, (hipStream_t)stream>>>(ids, dst, src, src_index, n, vocab);
+    return launch_status();
+}
+
 // ---------------------------------------------------------------- RMS norm
 // One block per output row. Sum of squares in float32, reduced in an order
 // fixed by the block size. Two passes over the row; the second re-reads what

@@ -23,6 +23,10 @@ union Frag8 {
 
 __device__ __forceinline__ float silu_mul_f(float g, float u) { return g / (1.0f + expf(-g)) * u; }
 
+__device__ __forceinline__ uint4 zero_if(bool out, uint4 v) {
+    return make_uint4(out ? 0u : v.x, out ? 0u : v.y, out ? 0u : v.z, out ? 0u : v.w);
+}
+
 // ------------------------------------------------------------------ float32
 #define F32_BM 64
 #define F32_BN 64
@@ -148,24 +152,34 @@ __global__ __launch_bounds__(256, 2) void k_gemm_bf16_tile(const bf16_t* __restr
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int row = (tid >> 3) + 32 * j;
-        pa[j] = X + (size_t)min(m0 + row, M - 1) * K_all + kc8;
-        pb[j] = W + (size_t)min(n0 + row, N - 1) * K_all + kc8;
+        pa[j] = X + (size_t)min(m0 + row, M - 1) * K_all;
+        pb[j] = W + (size_t)min(n0 + row, N - 1) * K_all;
         lds_off[j] = row * BG_LD + kc8;
     }
     const int nk = (K + BG_BK - 1) / BG_BK;
     // three register sets, one per K-step in flight (named apart so that they stay in registers)
     uint4 a0[4], b0[4], a1[4], b1[4], a2[4], b2[4];
 
+    // No load sits under a branch (the compiler would wait for every load in flight at the
+    // next use of any): addresses are clamped into the row, a step past the end reads the
+    // last one again, and what a cut step reads at or beyond K is zeroed on its way to LDS.
     auto fetch = [&](int kt, uint4 (&a)[4], uint4 (&b)[4]) {
-        const bool in = kt * BG_BK + kc8 < K;
-        const size_t off = (size_t)kt * BG_BK;
+        const int k = min(min(kt, nk - 1) * BG_BK + kc8, K - 8);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            a[j] = in ? *reinterpret_cast<const uint4*>(pa[j] + off) : make_uint4(0, 0, 0, 0);
-            b[j] = in ? *reinterpret_cast<const uint4*>(pb[j] + off) : make_uint4(0, 0, 0, 0);
+            a[j] = *reinterpret_cast<const uint4*>(pa[j] + k);
+            b[j] = *reinterpret_cast<const uint4*>(pb[j] + k);
         }
     };
-    auto stash = [&](int buf, const uint4 (&a)[4], const uint4 (&b)[4]) {
+    auto stash = [&](int kt, int buf, uint4 (&a)[4], uint4 (&b)[4]) {
+        if ((kt + 1) * BG_BK > K) {                               // only a cut step, or one past the end
+            const bool out = kt * BG_BK + kc8 >= K;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                a[j] = zero_if(out, a[j]);
+                b[j] = zero_if(out, b[j]);
+            }
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             *reinterpret_cast<uint4*>(&As[buf][lds_off[j]]) = a[j];
@@ -220,10 +234,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_bf16_tile(const bf16_t* __restr
     // take the load of step i+1+BG_PF, then step i is multiplied out of LDS
     auto step = [&](int i, uint4 (&na)[4], uint4 (&nb)[4]) {
         const int buf = i & 1;
-        if (i + 1 < nk) {
-            stash(buf ^ 1, na, nb);
-            fetch(i + 1 + BG_PF, na, nb);
-        }
+        stash(i + 1, buf ^ 1, na, nb);
+        fetch(i + 1 + BG_PF, na, nb);
         compute(buf);
         __syncthreads();
     };
@@ -231,13 +243,18 @@ __global__ __launch_bounds__(256, 2) void k_gemm_bf16_tile(const bf16_t* __restr
     fetch(0, a0, b0);
     fetch(1, a1, b1);
     fetch(2, a2, b2);
-    stash(0, a0, b0);
+    stash(0, 0, a0, b0);
     fetch(3, a0, b0);
     __syncthreads();
-    for (int kt = 0; kt < nk; kt += BG_PF) {
+    int kt = 0;
+    for (; kt + BG_PF <= nk; kt += BG_PF) {        // whole rounds of the three sets, free of branches
+        step(kt, a1, b1);
+        step(kt + 1, a2, b2);
+        step(kt + 2, a0, b0);
+    }
+    if (kt < nk) {
         step(kt, a1, b1);
         if (kt + 1 < nk) step(kt + 1, a2, b2);
-        if (kt + 2 < nk) step(kt + 2, a0, b0);
     }
     // D layout of the 32x32 tile: lane holds column lane%32, rows 8*(r/4) + 4*(lane/32) + r%4
 #pragma unroll
@@ -306,26 +323,33 @@ __global__ __launch_bounds__(WM * WN * 64) void k_gemm_bf16_big(const bf16_t* __
 #pragma unroll
     for (int j = 0; j < PA; ++j) {
         const int row = (tid >> 3) + (NT / 8) * j;
-        pa[j] = X + (size_t)min(m0 + row, M - 1) * K + kc8;
+        pa[j] = X + (size_t)min(m0 + row, M - 1) * K;
         la[j] = row * BG_LD + kc8;
     }
 #pragma unroll
     for (int j = 0; j < PB; ++j) {
         const int row = (tid >> 3) + (NT / 8) * j;
-        pb[j] = W + (size_t)min(n0 + row, N - 1) * K + kc8;
+        pb[j] = W + (size_t)min(n0 + row, N - 1) * K;
         lb[j] = row * BG_LD + kc8;
     }
     const int nk = (K + BG_BK - 1) / BG_BK;
     uint4 a0[PA], b0[PB], a1[PA], b1[PB];
+    // as in the 128x128 kernel: no load under a branch, addresses clamped, cut steps zeroed on the way to LDS
     auto fetch = [&](int kt, uint4 (&a)[PA], uint4 (&b)[PB]) {
-        const bool in = kt * BG_BK + kc8 < K;
-        const size_t off = (size_t)kt * BG_BK;
+        const int k = min(min(kt, nk - 1) * BG_BK + kc8, K - 8);
 #pragma unroll
-        for (int j = 0; j < PA; ++j) a[j] = in ? *reinterpret_cast<const uint4*>(pa[j] + off) : make_uint4(0, 0, 0, 0);
+        for (int j = 0; j < PA; ++j) a[j] = *reinterpret_cast<const uint4*>(pa[j] + k);
 #pragma unroll
-        for (int j = 0; j < PB; ++j) b[j] = in ? *reinterpret_cast<const uint4*>(pb[j] + off) : make_uint4(0, 0, 0, 0);
+        for (int j = 0; j < PB; ++j) b[j] = *reinterpret_cast<const uint4*>(pb[j] + k);
     };
-    auto stash = [&](int buf, const uint4 (&a)[PA], const uint4 (&b)[PB]) {
+    auto stash = [&](int kt, int buf, uint4 (&a)[PA], uint4 (&b)[PB]) {
+        if ((kt + 1) * BG_BK > K) {
+            const bool out = kt * BG_BK + kc8 >= K;
+#pragma unroll
+            for (int j = 0; j < PA; ++j) a[j] = zero_if(out, a[j]);
+#pragma unroll
+            for (int j = 0; j < PB; ++j) b[j] = zero_if(out, b[j]);
+        }
 #pragma unroll
         for (int j = 0; j < PA; ++j) *reinterpret_cast<uint4*>(&As[buf * BM * BG_LD + la[j]]) = a[j];
 #pragma unroll
@@ -360,22 +384,22 @@ __global__ __launch_bounds__(WM * WN * 64) void k_gemm_bf16_big(const bf16_t* __
     };
     auto step = [&](int i, uint4 (&na)[PA], uint4 (&nb)[PB]) {
         const int buf = i & 1;
-        if (i + 1 < nk) {
-            stash(buf ^ 1, na, nb);
-            fetch(i + 3, na, nb);
-        }
+        stash(i + 1, buf ^ 1, na, nb);
+        fetch(i + 3, na, nb);
         compute(buf);
         __syncthreads();
     };
     fetch(0, a0, b0);
     fetch(1, a1, b1);
-    stash(0, a0, b0);
+    stash(0, 0, a0, b0);
     fetch(2, a0, b0);
     __syncthreads();
-    for (int kt = 0; kt < nk; kt += 2) {
+    int kt = 0;
+    for (; kt + 2 <= nk; kt += 2) {                // whole rounds of the two sets, free of branches
         step(kt, a1, b1);
-        if (kt + 1 < nk) step(kt + 1, a0, b0);
+        step(kt + 1, a0, b0);
     }
+    if (kt < nk) step(kt, a1, b1);
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -638,9 +662,6 @@ __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
             f.w[s2].u = *reinterpret_cast<const uint4*>(wrow + min(k0 + s2 * 32 + g * 8, K - 8));
 #pragma unroll
         for (int j = 0; j < XP; ++j) f.x[j] = *reinterpret_cast<const uint4*>(xsrc[j] + min(k0 + xkc[j], K - 8));
-    };
-    auto zero_if = [](bool out, uint4 v) {
-        return make_uint4(out ? 0u : v.x, out ? 0u : v.y, out ? 0u : v.z, out ? 0u : v.w);
     };
     auto stash = [&](int kt, int buf, const StreamSet<XP>& f) {
         const int k0 = chunk_of(kt) * ST_BK;

@@ -273,6 +273,87 @@ int imparo_cache_check(const ImparoCache* c) {
     return 0;
 }
 
+int imparo_cache_begin_step(ImparoCache* c, int n_rows, const int64_t* reqs, const int32_t* n_tokens,
+                            const int32_t* tokens, const int32_t* n_want, const int32_t* want, int vocab,
+                            int max_position, int32_t* new_slots, int32_t* info) {
+    int bad_row = -1, widest = 1, code = 0, no_slot = 0;
+    // ---- what can be refused without touching anything
+    {
+        std::unordered_map<int64_t, int> seen;
+        int64_t t = 0, w = 0;
+        for (int r = 0; r < n_rows && !code; ++r) {
+            const int n = n_tokens[r];
+            auto it = c->live.find(reqs[r]);
+            const int length = it == c->live.end() ? 0 : it->second.length;
+            if (!seen.emplace(reqs[r], r).second) code = IMPARO_E_TWICE;
+            else if (n <= 0) code = IMPARO_E_EMPTY;
+            else if ((int64_t)length + n > max_position) code = IMPARO_E_POSITIONS;
+            for (int i = 0; i < n && !code; ++i)
+                if (tokens[t + i] < 0 || tokens[t + i] >= vocab) code = IMPARO_E_TOKEN;
+            for (int i = 0; i < n_want[r] && !code; ++i)
+                if (want[w + i] < 0 || want[w + i] >= n) code = IMPARO_E_WANT;
+            if (code) bad_row = r;
+            t += std::max(n, 0);
+            w += n_want[r];
+        }
+    }
+    // ---- slots and pages, all or nothing
+    int done = 0;
+    for (; done < n_rows && !code; ++done) {
+        new_slots[done] = -1;
+        if (!c->live.count(reqs[done])) {
+            const int slot = imparo_cache_admit(c, reqs[done]);
+            if (slot < 0) {
+                code = IMPARO_E_OUT_OF_PAGES;
+                bad_row = done;
+                no_slot = 1;
+                break;
+            }
+            new_slots[done] = slot;
+        }
+        Request& r = c->live[reqs[done]];
+        const int rc = imparo_cache_reserve(c, reqs[done], r.length + n_tokens[done]);
+        if (rc < 0) {
+            if (new_slots[done] >= 0) imparo_cache_release(c, reqs[done]);
+            code = rc;
+            bad_row = done;
+            break;
+        }
+        for (const auto& table : r.tables) widest = std::max(widest, (int)table.size());
+    }
+    if (code) {
+        for (int r = done - 1; r >= 0; --r) {     // rows before the failing one
+            if (new_slots[r] >= 0) imparo_cache_release(c, reqs[r]);
+            else c->undo(c->live[reqs[r]]);
+        }
+    }
+    if (info) {
+        info[0] = bad_row;
+        info[1] = widest;
+        info[2] = no_slot;
+    }
+    return code;
+}
+
+int imparo_cache_abort_step(ImparoCache* c, int n_rows, const int64_t* reqs, const int32_t* new_slots) {
+    for (int r = n_rows - 1; r >= 0; --r) {
+        auto it = c->live.find(reqs[r]);
+        if (it == c->live.end()) continue;
+        if (new_slots[r] >= 0) imparo_cache_release(c, reqs[r]);
+        else c->undo(it->second);
+    }
+    return 0;
+}
+
+int imparo_cache_end_step(ImparoCache* c, int n_rows, const int64_t* reqs, const int32_t* n_tokens) {
+    for (int r = 0; r < n_rows; ++r) {
+        auto it = c->live.find(reqs[r]);
+        if (it == c->live.end()) return IMPARO_E_NOT_LIVE;
+        imparo_cache_commit(c, reqs[r], it->second.length + n_tokens[r]);
+    }
+    return 0;
+}
+
 int64_t imparo_cache_pack(const ImparoCache* c, int n_rows, const int64_t* reqs, const int32_t* n_tokens,
                           const int32_t* tokens, const int32_t* n_want, const int32_t* want, int table_width,
                           int32_t* out, int64_t capacity, int32_t* layout) {

@@ -21,6 +21,11 @@ extern "C" {
 #define IMPARO_E_LOST_PAGE (-9)      // check: a page is neither free nor held
 #define IMPARO_E_SHARED_PAGE (-10)   // check: a page is held twice, or held and free
 #define IMPARO_E_SLOTS (-11)         // check: slots lost or held twice
+#define IMPARO_E_TWICE (-12)         // begin_step: a request appears twice
+#define IMPARO_E_EMPTY (-13)         // begin_step: a request brings no tokens
+#define IMPARO_E_POSITIONS (-14)     // begin_step: a request would pass the model's positions
+#define IMPARO_E_TOKEN (-15)         // begin_step: a token id outside the vocabulary
+#define IMPARO_E_WANT (-16)          // begin_step: a wanted place outside the request's tokens
 
 typedef struct ImparoPool ImparoPool;
 typedef struct ImparoCache ImparoCache;
@@ -61,6 +66,20 @@ int imparo_cache_n_groups(const ImparoCache* c);
 int imparo_cache_live_requests(const ImparoCache* c, int64_t* out, int capacity);
 int imparo_cache_check(const ImparoCache* c);
 
+// ---- a step's bookkeeping, one call for the whole batch (rows as for imparo_cache_pack).
+// begin: checks the batch (no request twice, at least one token each, length + tokens within
+// max_position, token ids in [0, vocab), wanted places inside the row's tokens), then admits
+// the requests that are not live (new_slots[r] = the slot taken, else -1: the caller clears
+// that slot's device state) and reserves pages for every row's new length. All or nothing: on
+// failure everything this call did is undone. info = {the failing row or -1, the widest block
+// table of the batch in pages, 1 if what ran out was slots}. Returns 0, IMPARO_E_OUT_OF_PAGES (pages, or slots) or the
+// check's code. abort undoes a begin whose step did not run; end commits every row.
+int imparo_cache_begin_step(ImparoCache* c, int n_rows, const int64_t* reqs, const int32_t* n_tokens,
+                            const int32_t* tokens, const int32_t* n_want, const int32_t* want, int vocab,
+                            int max_position, int32_t* new_slots, int32_t* info);
+int imparo_cache_abort_step(ImparoCache* c, int n_rows, const int64_t* reqs, const int32_t* new_slots);
+int imparo_cache_end_step(ImparoCache* c, int n_rows, const int64_t* reqs, const int32_t* n_tokens);
+
 // ---- a step's index arrays, packed for one host-to-device copy.
 // Layout (int32): tokens[T] | positions[T] | row_of_token[T] | seg_start[R] | seg_len[R] | slot[R] |
 // row lists[R] (rows with one token first, then the others) | want[W] | tables[G][R][P].
@@ -99,6 +118,10 @@ void imparo_sched_advance(ImparoSched* s);
 // A token was sampled for `id`: is_stop ends the reply unsent. Returns 0 (goes on), 1 (finished: stop),
 // 2 (finished: reached max_tokens; the token counts). The caller frees what a finished request holds.
 int imparo_sched_token(ImparoSched* s, int64_t id, int is_stop);
+// For a caller that reports tokens before it has read them (is_stop = 0, while the next step
+// is queued already): the token turned out to be a stop token. The request leaves, wherever
+// it stands, running or back in the waiting line. The caller frees what it holds.
+int imparo_sched_retract(ImparoSched* s, int64_t id);
 int imparo_sched_drop_waiting_head(ImparoSched* s, int64_t* id);   // 1 and the id, or 0 if nobody waits
 int imparo_sched_n_waiting(const ImparoSched* s);
 int imparo_sched_n_running(const ImparoSched* s);

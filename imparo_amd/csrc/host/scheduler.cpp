@@ -215,6 +215,17 @@ int imparo_sched_token(ImparoSched* s, int64_t id, int is_stop) {
     return outcome;
 }
 
+int imparo_sched_retract(ImparoSched* s, int64_t id) {
+    auto it = s->reqs.find(id);
+    if (it == s->reqs.end()) return IMPARO_E_NOT_LIVE;
+    s->running.erase(std::remove(s->running.begin(), s->running.end(), id), s->running.end());
+    s->waiting.erase(std::remove(s->waiting.begin(), s->waiting.end(), id), s->waiting.end());
+    s->planned.erase(std::remove_if(s->planned.begin(), s->planned.end(), [&](const Planned& p) { return p.id == id; }),
+                     s->planned.end());
+    s->reqs.erase(it);
+    return 0;
+}
+
 int imparo_sched_drop_waiting_head(ImparoSched* s, int64_t* id) {
     if (s->waiting.empty()) return 0;
     *id = s->waiting.front();

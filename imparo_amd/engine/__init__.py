@@ -1,2 +1,2 @@
-from .engine import Engine, StepEntry, StepError
+from .engine import DeviceToken, Engine, StepEntry, StepError
 from .model import Model, declared_tensors

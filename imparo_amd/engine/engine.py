@@ -18,10 +18,10 @@ from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-from ..cache.pages import CacheManager, OutOfPages
+from ..cache.pages import CacheError, CacheManager, OutOfPages
 from ..cache.storage import CacheStorage
 from ..config import plan_from_config, read_config_json
-from ..kernels import library
+from ..kernels import library, ops
 from ..parts.base import StepContext, Workspace
 from ..weights import load_weights
 from .model import Model, declared_tensors
@@ -36,8 +36,18 @@ class StepError(ValueError):
 @dataclass
 class StepEntry:
     request: Hashable
-    tokens: Sequence[int]
+    tokens: Sequence[int]          # token ids; a lone DeviceToken stands for one that was not read back yet
     want: Sequence[int] = ()       # places among `tokens` whose logits are wanted
+
+
+@dataclass(frozen=True)
+class DeviceToken:
+    """A token id that the sampling kernel left on the device: element `index`
+    of `source`, an int32 tensor. A request may bring one as its only token;
+    the step then takes the id from there, so that the host need not wait for
+    the step before to end before it queues the next."""
+    source: torch.Tensor
+    index: int
 
 
 class _Upload:
@@ -146,73 +156,78 @@ class Engine:
         """Runs one batch. Returns float32 logits [wanted, vocab] on the
         device, in the order of the entries and of each entry's `want`, or
         None when nothing is wanted."""
-        entries = [e for e in entries]
-        seen = set()
-        for e in entries:
-            if e.request in seen:
-                raise StepError(f"request {e.request!r} appears twice in one step")
-            seen.add(e.request)
-            if len(e.tokens) == 0:
-                raise StepError(f"request {e.request!r} brings no tokens")
-            for tok in e.tokens:
-                if not 0 <= int(tok) < self.vocab_size:
-                    raise StepError(f"request {e.request!r}: token id {tok} is outside the vocabulary "
-                                    f"of {self.vocab_size}")
-            for w in e.want:
-                if not 0 <= int(w) < len(e.tokens):
-                    raise StepError(f"request {e.request!r}: wanted place {w} is outside its "
-                                    f"{len(e.tokens)} tokens")
-            if self.length(e.request) + len(e.tokens) > self.max_position:
-                raise StepError(f"request {e.request!r} would pass the model's {self.max_position} positions")
+        entries = list(entries)
         if not entries:
             return None
-
-        # pages and slots, all or nothing
-        admitted: List[Hashable] = []
-        taken: List[Tuple[Hashable, list]] = []
+        # the native side checks the batch, admits, and reserves pages and slots, all or nothing
+        token_lists = [e.tokens for e in entries]
+        on_device = [(row, e.tokens[0]) for row, e in enumerate(entries)
+                     if len(e.tokens) == 1 and isinstance(e.tokens[0], DeviceToken)]
+        for row, tok in on_device:
+            if (tok.source.dtype != torch.int32 or tok.source.dim() != 1 or tok.source.device != self.device
+                    or not 0 <= tok.index < tok.source.shape[0] or tok.source is not on_device[0][1].source):
+                raise StepError(f"request {entries[row].request!r}: a device token must be an element of one "
+                                f"int32 vector on {self.device}, the same for the whole step")
+            token_lists[row] = (0,)          # a placeholder until the id is copied in on the device
         try:
-            for e in entries:
-                if not self.cache.is_live(e.request):
-                    slot = self.cache.admit(e.request)
-                    admitted.append(e.request)
-                    self.storage.zero_slot(slot)
-                got = self.cache.reserve(e.request, self.cache.length[e.request] + len(e.tokens))
-                taken.append((e.request, got))
-        except OutOfPages:
-            for req, got in reversed(taken):
-                self.cache.rollback(req, got)
-            for req in admitted:
-                self.cache.release(req)
+            batch = self.cache.batch([e.request for e in entries], token_lists, [e.want for e in entries])
+        except CacheError as err:
+            raise StepError(str(err)) from None
+        if on_device:
+            starts = np.cumsum(batch.n_tok) - batch.n_tok
+            batch.device_tokens = (on_device[0][1].source,
+                                   np.array([starts[row] for row, _ in on_device], dtype=np.int32),
+                                   np.array([tok.index for _, tok in on_device], dtype=np.int32))
+        code, row = self.cache.begin_step(batch, self.vocab_size, self.max_position)
+        if code:
+            raise StepError(self._refusal(code, entries[row]))
+        try:
+            for slot in batch.new_slots[batch.new_slots >= 0].tolist():
+                self.storage.zero_slot(slot)
+            if (self.use_graphs and self.model.graph_safe and batch.T == len(entries)
+                    and bool((batch.n_want == 1).all())):
+                logits = self._decode_step(entries, batch)       # one token each, wanted
+            else:
+                ctx, token_ids, want_rows = self._pack(batch)
+                logits = self.model.forward(ctx, token_ids, want_rows)
+        except BaseException:
+            self.cache.abort_step(batch)
             raise
-
-        if (self.use_graphs and self.model.graph_safe
-                and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)):
-            logits = self._decode_step(entries)
-        else:
-            ctx, token_ids, want_rows = self._pack(entries)
-            logits = self.model.forward(ctx, token_ids, want_rows)
-        for e in entries:
-            self.cache.commit(e.request, self.cache.length[e.request] + len(e.tokens))
+        self.cache.end_step(batch)
         self.steps_run += 1
         return logits
 
-    def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def _refusal(self, code: int, e: StepEntry) -> str:
+        from ..cache import native as N
+        if code == N.E_TWICE:
+            return f"request {e.request!r} appears twice in one step"
+        if code == N.E_EMPTY:
+            return f"request {e.request!r} brings no tokens"
+        if code == N.E_POSITIONS:
+            return f"request {e.request!r} would pass the model's {self.max_position} positions"
+        if code == N.E_TOKEN:
+            bad = next(t for t in e.tokens if not 0 <= int(t) < self.vocab_size)
+            return f"request {e.request!r}: token id {bad} is outside the vocabulary of {self.vocab_size}"
+        if code == N.E_WANT:
+            bad = next(w for w in e.want if not 0 <= int(w) < len(e.tokens))
+            return f"request {e.request!r}: wanted place {bad} is outside its {len(e.tokens)} tokens"
+        return f"request {e.request!r}: the cache manager refused the step with code {code}"
+
+    def _decode_step(self, entries: Sequence[StepEntry], batch) -> torch.Tensor:
         """A step of single tokens. The first step of a batch shape runs
         launch by launch (so that every kernel it needs has been loaded), the
         second is captured, later ones replay the capture."""
-        G = len(self.cache.groups)
-        widest = max([self.cache.table_len(g, e.request) for e in entries for g in range(G)] or [1])
-        width = -(-widest // TABLE_BUCKET) * TABLE_BUCKET
+        width = -(-batch.widest // TABLE_BUCKET) * TABLE_BUCKET
         key = (len(entries), width)
         g = self._graphs.setdefault(key, _DecodeGraph())
         g.seen += 1
         if g.seen == 1:
-            ctx, token_ids, want_rows = self._pack(entries)
+            ctx, token_ids, want_rows = self._pack(batch)
             return self.model.forward(ctx, token_ids, want_rows)
         if g.graph is None:
             g.workspace = Workspace(self.device)
             # the capture fixes grid sizes: they are sized for the widest context the tables can hold
-            ctx, token_ids, want_rows = self._pack(entries, table_width=width, workspace=g.workspace, graph=g)
+            ctx, token_ids, want_rows = self._pack(batch, table_width=width, workspace=g.workspace, graph=g)
             if self._graph_pool is None:
                 self._graph_pool = torch.cuda.graph_pool_handle()
             graph = torch.cuda.CUDAGraph()
@@ -220,18 +235,20 @@ class Engine:
                 g.logits = self.model.forward(ctx, token_ids, want_rows)
             g.graph = graph
         else:
-            self._pack(entries, table_width=width, workspace=g.workspace, graph=g)
+            self._pack(batch, table_width=width, workspace=g.workspace, graph=g)
         g.graph.replay()
         return g.logits
 
-    def _pack(self, entries: Sequence[StepEntry], table_width: Optional[int] = None,
+    def _pack(self, batch, table_width: Optional[int] = None,
               workspace: Optional[Workspace] = None, graph: Optional[_DecodeGraph] = None):
         """Builds the step's index arrays, sends them to the device in one
         copy and wraps them in a StepContext. For a captured step the arrays go
         to the capture's own fixed buffer and sizes are the capture's bounds."""
-        a, lay = self.cache.pack([e.request for e in entries], [e.tokens for e in entries],
-                                 [e.want for e in entries], table_width or 0)
+        a, lay = self.cache.pack_batch(batch, table_width or 0)
         T, R, W, G, P, total = lay["T"], lay["R"], lay["W"], lay["G"], lay["P"], lay["total"]
+        placed = batch.device_tokens
+        if placed is not None:               # where the ids go, and where they come from, ride along
+            a = np.concatenate([a, placed[1], placed[2]])
         o_pos, o_row = T, 2 * T
         o_start, o_len, o_slot = 3 * T, 3 * T + R, 3 * T + 2 * R
         o_lists = 3 * T + 3 * R
@@ -241,10 +258,14 @@ class Engine:
         n_dec = lay["n_single"]
         if graph is not None:
             if graph.meta is None:
-                graph.meta = torch.empty(total, dtype=torch.int32, device=self.device)
+                graph.meta = torch.empty(total + 2 * R, dtype=torch.int32, device=self.device)
             dev = self._upload.send(a, into=graph.meta)
         else:
             dev = self._upload.send(a)
+        if placed is not None:
+            n = placed[1].shape[0]
+            ops.place_tokens(dev[o_tok:o_tok + T], dev[total:total + n], placed[0], dev[total + n:total + 2 * n],
+                             self.vocab_size)
         block_tables = {g: dev[o_tab + g * R * P:o_tab + (g + 1) * R * P].view(R, P) for g in range(G)}
         ctx = StepContext(
             n_tokens=T, n_rows=R,

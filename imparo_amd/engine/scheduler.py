@@ -52,6 +52,11 @@ class Request:
     finish_reason: str = ""
     preemptions: int = 0
     arrival: int = 0
+    drawn: int = 0                   # tokens sampled for it that count, read back or not
+    # while its last sampled token has not been read back:
+    unread: bool = False
+    ended_by_length: bool = False    # that token is its last; it has left the engine already
+    repend: bool = False             # it was pre-empted meanwhile: `pending` lacks that token
 
 
 @dataclass
@@ -69,15 +74,26 @@ class Scheduler:
     The decisions (whom to admit, what each request feeds under the budget,
     whom to pre-empt) are taken by the native scheduler core
     (csrc/host/scheduler.cpp), which knows requests by size only; token
-    values, sampling and the model step are handled here."""
+    values, sampling and the model step are handled here.
+
+    With `pick_async` (logits, temperatures, uniforms -> an object with
+    `on_device`, the int32 vector the tokens land in, and `tokens()`, which
+    waits for them) the loop does not wait for a step's tokens before it
+    queues the next step: a request's next token is fed from the device, the
+    host reads it one step late, while the GPU is busy. Every sampled token is
+    then counted as "goes on" at first; when it turns out to be a stop token
+    the request is taken out (it has run one step in vain). What is generated
+    is the same either way."""
 
     def __init__(self, engine, pick: Callable, max_batch_tokens: int = 2048, max_running: int = 64,
-                 portion: Optional[int] = None, entry_type=None):
+                 portion: Optional[int] = None, entry_type=None, pick_async: Optional[Callable] = None):
         from ..cache import native as N
         self._N = N
         self._lib = N.host_library()
         self.engine = engine
         self.pick = pick
+        self.pick_async = pick_async
+        self._unread = None              # (requests and their places, the pending pick) of the last step
         self.max_batch_tokens = max_batch_tokens
         self.max_running = max_running
         self.portion = portion or prefill_portion()
@@ -124,7 +140,8 @@ class Scheduler:
         return r
 
     def has_work(self) -> bool:
-        return bool(self._lib.imparo_sched_n_waiting(self._s) or self._lib.imparo_sched_n_running(self._s))
+        return bool(self._lib.imparo_sched_n_waiting(self._s) or self._lib.imparo_sched_n_running(self._s)
+                    or self._unread is not None)
 
     def _listed(self, fn) -> List[Request]:
         buf = (ctypes.c_int64 * max(1, len(self._requests)))()
@@ -158,6 +175,7 @@ class Scheduler:
                 # it gave back everything it held; it will recompute prompt ++ generated
                 self.engine.release(r.id)
                 r.pending = r.prompt + r.generated
+                r.repend = r.unread            # its latest token joins `pending` when it has been read
                 r.fed = 0
                 r.next_token = None
                 r.preemptions += 1
@@ -187,7 +205,7 @@ class Scheduler:
         every token handed out in this iteration."""
         planned = self.plan()
         if not planned:
-            return []
+            return self._read_back()
         entries = [self._entry(p.request.id, p.tokens, [len(p.tokens) - 1] if p.wants_logits else [])
                    for p in planned]
         logits = self.engine.step(entries)
@@ -199,25 +217,89 @@ class Scheduler:
             else:
                 r.next_token = None           # the decoded token is in the cache now
         askers = [p.request for p in planned if p.wants_logits]
+        if not askers:
+            return self._read_back()
+        temps = [r.params.temperature for r in askers]
+        unis = [uniform_for(r.params.seed, r.drawn) for r in askers]
+        if self.pick_async is not None:
+            pending = self.pick_async(logits, temps, unis)
+            out = self._read_back()          # the step before's tokens, while this step runs
+            self._count_unread(askers, pending)
+            return out
         out: List[Tuple[Hashable, int]] = []
-        if askers:
-            temps = [r.params.temperature for r in askers]
-            unis = [uniform_for(r.params.seed, len(r.generated)) for r in askers]
-            picks = self.pick(logits, temps, unis)
-            for r, tok in zip(askers, picks):
-                tok = int(tok)
-                h = self.engine.cache.handle(r.id)
-                is_stop = tok in r.params.stop_token_ids      # a stop token ends the reply unsent
-                outcome = self._lib.imparo_sched_token(self._s, h, int(is_stop))
+        picks = self.pick(logits, temps, unis)
+        for r, tok in zip(askers, picks):
+            tok = int(tok)
+            h = self.engine.cache.handle(r.id)
+            is_stop = tok in r.params.stop_token_ids      # a stop token ends the reply unsent
+            outcome = self._lib.imparo_sched_token(self._s, h, int(is_stop))
+            if not is_stop:
+                r.drawn += 1
+                r.generated.append(tok)
+                out.append((r.id, tok))
+            if outcome == 0:
+                r.next_token = tok
+            else:                                          # 1: stop; 2: the last token needs no forward
+                self.engine.release(r.id)
+                del self._requests[h]
+                self._finish(r, "stop" if outcome == 1 else "length")
+        return out
+
+    def _count_unread(self, askers: List[Request], pending) -> None:
+        """Counts tokens that were asked for but not read yet, as tokens after which the reply goes on."""
+        from .engine import DeviceToken
+        places = []
+        for i, r in enumerate(askers):
+            if r.finished:                     # a late stop token ended it while this step ran
+                continue
+            h = self.engine.cache.handle(r.id)
+            outcome = self._lib.imparo_sched_token(self._s, h, 0)
+            r.drawn += 1
+            r.unread = True
+            if outcome == 0:
+                r.next_token = DeviceToken(pending.on_device, i)
+            else:                              # 2: its last token; it needs no forward and leaves the engine now
+                self.engine.release(r.id)
+                del self._requests[h]
+                r.ended_by_length = True
+            places.append((r, i))
+        self._unread = (places, pending)
+
+    def _read_back(self) -> List[Tuple[Hashable, int]]:
+        """Waits for the tokens of the step before and hands them out."""
+        if self._unread is None:
+            return []
+        places, pending = self._unread
+        self._unread = None
+        tokens = pending.tokens()
+        out: List[Tuple[Hashable, int]] = []
+        for r, i in places:
+            tok = int(tokens[i])
+            r.unread = False
+            is_stop = tok in r.params.stop_token_ids
+            if r.finished:                                 # it failed meanwhile: the token still counts
                 if not is_stop:
                     r.generated.append(tok)
                     out.append((r.id, tok))
-                if outcome == 0:
-                    r.next_token = tok
-                else:                                          # 1: stop; 2: the last token needs no forward
+                continue
+            if is_stop:                                    # ends the reply unsent, one step late
+                if not r.ended_by_length:
+                    h = self.engine.cache.handle(r.id)
+                    self._lib.imparo_sched_retract(self._s, h)
                     self.engine.release(r.id)
-                    del self._requests[h]
-                    self._finish(r, "stop" if outcome == 1 else "length")
+                    self._requests.pop(h, None)
+                self._finish(r, "stop")
+                continue
+            r.generated.append(tok)
+            out.append((r.id, tok))
+            if r.ended_by_length:
+                self._finish(r, "length")
+                continue
+            if r.next_token is not None and not isinstance(r.next_token, int):
+                r.next_token = tok                         # not fed yet: the host's copy will do
+            if r.repend:
+                r.pending = r.prompt + r.generated
+                r.repend = False
         return out
 
     def run(self) -> Dict[Hashable, Request]:
@@ -227,7 +309,7 @@ class Scheduler:
             self.step()
             after = (self._lib.imparo_sched_n_waiting(self._s), self._lib.imparo_sched_n_running(self._s),
                      len(self.finished))
-            if after[1] == 0 and after[0] and before == after and n_running == 0:
+            if after[1] == 0 and after[0] and before == after and n_running == 0 and self._unread is None:
                 head = ctypes.c_int64(0)                       # nothing runs and the head still cannot start
                 if self._lib.imparo_sched_drop_waiting_head(self._s, ctypes.byref(head)):
                     r = self._requests.pop(head.value)
@@ -238,11 +320,13 @@ class Scheduler:
 def generate(model, input_ids: Sequence[Sequence[int]], max_tokens: int = 16, temperature: float = 0.0,
              seed: int = 0, stop_token_ids: Optional[Sequence[int]] = None, dtype: str = "bfloat16",
              ctx: Optional[int] = None, parallel: int = 64, max_batch_tokens: int = 2048,
-             page_size: int = 64) -> List[List[int]]:
+             page_size: int = 64, overlap: bool = True) -> List[List[int]]:
     """Tokens in, tokens out. `model` is a model folder or an Engine; returns
     the generated ids of every prompt, in order. Request `i` samples with seed
     `seed + i`. `ctx` is the most tokens one request may hold (the reference's
-    -c/--ctx), `parallel` the most requests that run at once (-np/--parallel)."""
+    -c/--ctx), `parallel` the most requests that run at once (-np/--parallel).
+    `overlap`: queue each step before the tokens of the step before are read
+    back (the same tokens come out; False waits after every step)."""
     from .engine import Engine
     from ..sampling.sampler import Sampler
     if isinstance(model, Engine):
@@ -257,7 +341,8 @@ def generate(model, input_ids: Sequence[Sequence[int]], max_tokens: int = 16, te
     stops = tuple(stop_token_ids) if stop_token_ids is not None else tuple(engine.plan.stop_token_ids)
     sampler = Sampler(engine.device)
     sched = Scheduler(engine, sampler.pick, max_batch_tokens=max_batch_tokens,
-                      max_running=min(parallel, engine.cache.n_slots))
+                      max_running=min(parallel, engine.cache.n_slots),
+                      pick_async=sampler.pick_async if overlap else None)
     for i, prompt in enumerate(input_ids):
         sched.add(i, prompt, SamplingParams(temperature=temperature, max_tokens=max_tokens, seed=seed + i,
                                             stop_token_ids=stops))

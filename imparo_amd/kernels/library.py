@@ -22,6 +22,7 @@ F = c_float
 
 _SIGNATURES = {
     "imparo_embed_gather": [P, I, P, P, I, I, I, P],
+    "imparo_place_tokens": [P, P, P, P, I, I, P],
     "imparo_rms_norm": [P, P, I, I, P, P, P, I, I, I, F, I, P],
     "imparo_silu_mul": [P, I, P, I, I, I, P],
     "imparo_add_bias": [P, P, I, I, P],

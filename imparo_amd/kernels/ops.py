@@ -66,6 +66,18 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> t
     return out
 
 
+def place_tokens(ids: torch.Tensor, dst: torch.Tensor, src: torch.Tensor, src_index: torch.Tensor,
+                 vocab: int) -> torch.Tensor:
+    """ids[dst[i]] = src[src_index[i]]: token ids that the step before sampled and that were
+    not read back. The caller has checked the indices on the host (they come from there)."""
+    n = dst.shape[0]
+    _check(library().imparo_place_tokens(
+        _dev(ids, "token ids", torch.int32), _dev(dst, "places", torch.int32, (n,)),
+        _dev(src, "sampled tokens", torch.int32), _dev(src_index, "indices of sampled tokens", torch.int32, (n,)),
+        n, vocab, _stream()), "place_tokens")
+    return ids
+
+
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
              delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
              write_back: bool = False) -> torch.Tensor:

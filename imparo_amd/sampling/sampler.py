@@ -44,6 +44,24 @@ class SamplingParams:
     stop_token_ids: Tuple[int, ...] = ()
 
 
+class PendingPick:
+    """Token ids that the sampling kernel has been asked for. `on_device` is
+    the int32 vector they land in (to feed the next step from, without
+    waiting); `tokens()` waits for the copy to the host and returns them."""
+
+    def __init__(self, on_device, host, event):
+        self.on_device = on_device
+        self._host = host
+        self._event = event
+        self._tokens: Optional[List[int]] = None
+
+    def tokens(self) -> List[int]:
+        if self._tokens is None:
+            self._event.synchronize()
+            self._tokens = self._host.tolist()
+        return self._tokens
+
+
 class Sampler:
     """Runs the sampling kernels over the logits rows a step returned."""
 
@@ -52,7 +70,8 @@ class Sampler:
         self.device = device
         self._torch = torch
 
-    def pick(self, logits, temperatures: Sequence[float], uniforms: Sequence[float]) -> List[int]:
+    def pick_async(self, logits, temperatures: Sequence[float], uniforms: Sequence[float]) -> PendingPick:
+        """Queues the kernel and the copy of its result to the host; returns at once."""
         torch = self._torch
         from ..kernels import ops
         n = logits.shape[0]
@@ -63,4 +82,11 @@ class Sampler:
             host = torch.tensor([list(temperatures), list(uniforms)], dtype=torch.float32, pin_memory=True)
             dev = host.to(logits.device, non_blocking=True)
             ops.sample_rows(logits, dev[0], dev[1], out)
-        return out.cpu().tolist()
+        back = torch.empty(n, dtype=torch.int32, pin_memory=True)
+        back.copy_(out, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        return PendingPick(out, back, event)
+
+    def pick(self, logits, temperatures: Sequence[float], uniforms: Sequence[float]) -> List[int]:
+        return self.pick_async(logits, temperatures, uniforms).tokens()

@@ -206,3 +206,74 @@ def test_pack_lays_out_a_step():
     assert lay2["P"] == 8 and fixed[-8:].tolist() == m.table(1, "a") + [-1] * 5
     with pytest.raises(CacheError):
         m.pack(["zzz"], [[1]], [[0]])
+
+
+def snapshot(m, names):
+    return (m.free_pages(), m.slots.n_free, sorted(n for n in names if m.is_live(n)),
+            {n: [m.table(g, n) for g in range(len(m.groups))] for n in names if m.is_live(n)},
+            {n: m.length[n] for n in names if m.is_live(n)})
+
+
+def test_a_whole_step_is_booked_in_one_call():
+    """begin_step admits, reserves and checks for the whole batch; end_step commits it. The
+    result is what admit/reserve/commit give one request at a time."""
+    from imparo_amd.cache import native as N
+    specs = [PagedSpec(1, 16), FixedSpec((4,)), PagedSpec(1, 16, window=6)]
+    m = CacheManager(specs, page_size=4, n_pages=16, n_slots=3)
+    one = CacheManager(specs, page_size=4, n_pages=16, n_slots=3)
+    steps = [(["a", "b"], [[1] * 9, [2] * 3]), (["b", "a", "c"], [[5], [6, 7], [8] * 5]), (["c", "a"], [[1], [2]])]
+    for names, toks in steps:
+        b = m.batch(names, toks, [[0]] * len(names))
+        assert m.begin_step(b, vocab=10, max_position=64) == (0, -1)
+        new = [n for n, s in zip(names, b.new_slots.tolist()) if s >= 0]
+        for n, t in zip(names, toks):
+            if not one.is_live(n):
+                assert n in new and one.admit(n) == int(b.new_slots[names.index(n)])
+            else:
+                assert n not in new
+            one.reserve(n, one.length[n] + len(t))
+        assert b.widest == max(len(one.table(g, n)) for n in names for g in range(2))
+        arr, lay = m.pack_batch(b)
+        arr1, lay1 = one.pack(names, toks, [[0]] * len(names))
+        assert lay == lay1 and arr.tolist() == arr1.tolist()
+        m.end_step(b)
+        for n, t in zip(names, toks):
+            one.commit(n, one.length[n] + len(t))
+        assert snapshot(m, "abc") == snapshot(one, "abc")
+        m.check()
+    # what is wrong with a batch is said before anything is touched
+    before = snapshot(m, "abcd")
+    for names, toks, want, code, row in (
+            (["a", "d", "a"], [[1], [1], [1]], [[0], [0], [0]], N.E_TWICE, 2),
+            (["a", "d"], [[1], []], [[0], []], N.E_EMPTY, 1),
+            (["d", "a"], [[1], [1] * 60], [[0], [0]], N.E_POSITIONS, 1),
+            (["d", "a"], [[1, 10], [1]], [[0], [0]], N.E_TOKEN, 0),
+            (["d", "a"], [[1, -1], [1]], [[0], [0]], N.E_TOKEN, 0),
+            (["d", "a"], [[1], [1, 2]], [[0], [2]], N.E_WANT, 1)):
+        assert m.begin_step(m.batch(names, toks, want), vocab=10, max_position=64) == (code, row)
+        assert snapshot(m, "abcd") == before
+    with pytest.raises(CacheError, match="32 bits"):
+        m.batch(["a"], [[2 ** 40]], [[0]])
+
+
+def test_a_step_that_does_not_fit_changes_nothing():
+    m = CacheManager([PagedSpec(1, 16), PagedSpec(1, 16, window=6)], page_size=4, n_pages=6, n_slots=2)
+    b = m.batch(["a"], [[1] * 10], [[9]])
+    assert m.begin_step(b, 10, 64) == (0, -1)
+    m.end_step(b)
+    before = snapshot(m, "abc")
+    # a's 6 more fit (1 page of 3 free), new b's 12 do not: neither advances, b is not admitted
+    with pytest.raises(OutOfPages, match="pages"):
+        m.begin_step(m.batch(["a", "b"], [[1] * 6, [1] * 12], [[0], [0]]), 10, 64)
+    assert snapshot(m, "abc") == before
+    # slots: b fits, c finds no slot; b leaves again
+    with pytest.raises(OutOfPages, match="slots"):
+        m.begin_step(m.batch(["b", "c", "a"], [[1], [1], [1]], [[0], [0], [0]]), 10, 64)
+    assert snapshot(m, "abc") == before
+    # a step that was booked and then did not run
+    b = m.batch(["a", "b"], [[1] * 3, [1] * 4], [[0], [0]])
+    assert m.begin_step(b, 10, 64) == (0, -1)
+    assert m.is_live("b") and snapshot(m, "abc") != before
+    m.abort_step(b)
+    assert snapshot(m, "abc") == before
+    m.check()

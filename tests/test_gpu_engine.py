@@ -269,6 +269,43 @@ def test_a_step_that_does_not_fit_changes_nothing(zoo):
     assert eng.free_pages() == [8]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_tokens_fed_from_the_device(zoo, dtype):
+    """A request's single token may be named as an element of an int32 vector on the device
+    (where the sampling kernel left it): the step gives the logits it gives for the id itself,
+    launch by launch, captured, and beside a portion of a prompt."""
+    from imparo_amd.engine import StepEntry, DeviceToken, StepError
+    vocab = vocab_of(zoo, "B")
+    prompts = [prompt_tokens(vocab, n, 30 + n) for n in (12, 7, 20)]
+    nxt = [prompt_tokens(vocab, 6, 90 + i) for i in range(3)]
+    runs = []
+    for from_device in (False, True):
+        eng = make_engine(zoo[0]["B"], dtype, page_size=8, max_tokens=256, max_requests=4)
+        for i in (0, 1):
+            eng.step([StepEntry(i, prompts[i], [])])
+        out = []
+        for s in range(6):                     # steps 0..: eager, capture, replays; step 4 brings a prompt along
+            ids = [nxt[0][s], nxt[1][s]]
+            src = torch.tensor([7, ids[1], 3, ids[0]], dtype=torch.int32, device=eng.device)
+            toks = [[DeviceToken(src, 3)], [DeviceToken(src, 1)]] if from_device else [[ids[0]], [ids[1]]]
+            entries = [StepEntry(0, toks[0], [0]), StepEntry(1, toks[1], [0])]
+            if s == 4:
+                entries.insert(1, StepEntry(2, prompts[2], [19]))
+            out.append(eng.step(entries))
+        runs.append(torch.cat(out).cpu())
+        if from_device:
+            with pytest.raises(StepError, match="device token"):
+                eng.step([StepEntry(0, [DeviceToken(src, 4)], [0])])
+            with pytest.raises(StepError, match="device token"):
+                eng.step([StepEntry(0, [DeviceToken(src.long(), 0)], [0])])
+            with pytest.raises(StepError, match="device token"):
+                eng.step([StepEntry(0, [DeviceToken(src, 0)], [0]), StepEntry(1, [DeviceToken(src.clone(), 0)], [0])])
+            assert eng.length(0) == 12 + 6
+    assert torch.equal(runs[0], runs[1])
+    ref = zoo[1]["B"](prompts[0] + nxt[0])
+    check_logits(runs[0][0:1], ref[12:13], dtype, "first decoded row")
+
+
 def test_refused_batches(zoo, engines):
     from imparo_amd.engine import StepEntry, StepError
     eng = engines("A", "float32")

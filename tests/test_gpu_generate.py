@@ -80,14 +80,16 @@ def test_temperature_sampling_tiny_b(model_dirs, plain_models):
     assert alone == want[:2]          # a request's draws do not depend on its batch
 
 
-def test_preemption_by_recompute_keeps_greedy_outputs(model_dirs, plain_models):
+@pytest.mark.parametrize("overlap", [False, True])
+def test_preemption_by_recompute_keeps_greedy_outputs(model_dirs, plain_models, overlap):
     from imparo_amd.engine import Engine
     from imparo_amd.engine.scheduler import Scheduler
     from imparo_amd.sampling import Sampler, SamplingParams
     prompts = [prompt_tokens(256, n, 80 + n) for n in (20, 22, 18)]
     want = [plain_models["A"].greedy(p, 20) for p in prompts]
     eng = Engine(model_dirs["A"], dtype="float32", page_size=8, max_tokens=10 * 8, max_requests=4)
-    sched = Scheduler(eng, Sampler(eng.device).pick, max_batch_tokens=64)
+    sampler = Sampler(eng.device)
+    sched = Scheduler(eng, sampler.pick, max_batch_tokens=64, pick_async=sampler.pick_async if overlap else None)
     for i, p in enumerate(prompts):
         sched.add(i, p, SamplingParams(max_tokens=20))
     done = sched.run()
@@ -102,6 +104,26 @@ def test_stop_token_and_entry_point_defaults(model_dirs, plain_models):
     full = plain_models["A"].greedy(p, 10)
     got = generate(model_dirs["A"], [p], max_tokens=10, dtype="float32", stop_token_ids=[full[4]])
     assert got == [full[:full.index(full[4])]]
+
+
+def test_waiting_after_every_step_generates_the_same(model_dirs, plain_models):
+    """By default a step is queued before the tokens of the step before are read back (they
+    are fed from the device); overlap=False waits after every step. Same tokens either way:
+    greedy and sampled, with a stop token that is noticed a step late, in both dtypes."""
+    from imparo_amd import generate
+    prompts = [prompt_tokens(384, n, 60 + n) for n in (3, 9, 40, 21, 2)]
+    for dtype in ("float32", "bfloat16"):
+        for kw in (dict(), dict(temperature=0.8, seed=5)):
+            free = generate(model_dirs["B"], prompts, max_tokens=20, dtype=dtype, page_size=8, parallel=3,
+                            max_batch_tokens=16, overlap=False, **kw)
+            assert generate(model_dirs["B"], prompts, max_tokens=20, dtype=dtype, page_size=8, parallel=3,
+                            max_batch_tokens=16, **kw) == free
+            stops = [free[0][3], free[2][7], free[3][-1]]
+            a = generate(model_dirs["B"], prompts, max_tokens=20, dtype=dtype, page_size=8, parallel=3,
+                         max_batch_tokens=16, stop_token_ids=stops, overlap=False, **kw)
+            b = generate(model_dirs["B"], prompts, max_tokens=20, dtype=dtype, page_size=8, parallel=3,
+                         max_batch_tokens=16, stop_token_ids=stops, **kw)
+            assert a == b and len(a[0]) <= 3 and all(t not in stops for out in a for t in out)
 
 
 def test_command_line(model_dirs, plain_models, tmp_path):

@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 from imparo_amd.cache import CacheManager, PagedSpec, FixedSpec, OutOfPages
+from imparo_amd.engine.engine import DeviceToken
 from imparo_amd.engine.scheduler import Scheduler, Request
 from imparo_amd.sampling import SamplingParams, uniform_for
 
@@ -50,6 +51,8 @@ class FakeEngine:
             raise AssertionError("the scheduler sent a step that does not fit")
         rows = []
         for e in entries:
+            # a token that "is still on the device" is looked up where the fake sampler left it
+            e.tokens = [t.source[t.index] if isinstance(t, DeviceToken) else t for t in e.tokens]
             self.history[e.request].extend(e.tokens)
             self.cache.commit(e.request, len(self.history[e.request]))
             for w in e.want:
@@ -80,9 +83,25 @@ def expected(prompt, n):
     return out
 
 
-def make(n_pages=64, **kw):
+class FakePending:
+    """What an asynchronous sampler hands back: the tokens "on the device", and a wait for them."""
+    reads = 0
+
+    def __init__(self, tokens):
+        self.on_device = tokens
+
+    def tokens(self):
+        FakePending.reads += 1
+        return self.on_device
+
+
+def pick_async(logits, temperatures, uniforms):
+    return FakePending(pick(logits, temperatures, uniforms))
+
+
+def make(n_pages=64, overlap=False, **kw):
     eng = FakeEngine(n_pages)
-    return eng, Scheduler(eng, pick, entry_type=Entry, **kw)
+    return eng, Scheduler(eng, pick, entry_type=Entry, pick_async=pick_async if overlap else None, **kw)
 
 
 def test_one_request_prompt_in_portions_then_decode():
@@ -226,3 +245,84 @@ def test_uniform_numbers_depend_on_seed_and_index_only():
     assert all(0.0 <= u < 1.0 for u in a) and len(set(a)) > 90
     assert a != [uniform_for(4, i) for i in range(100)]
     assert 0.35 < sum(a) / 100 < 0.65
+
+
+# ---------------------------------------------------------------- the next step queued before the tokens are read
+def test_overlapped_steps_feed_tokens_from_the_device_and_read_them_a_step_late():
+    eng, s = make(overlap=True, max_batch_tokens=8, portion=5)
+    s.add("a", list(range(12)), SamplingParams(max_tokens=4))
+    assert s.step() == [] and s.step() == [] and s.step() == []     # the prompt; its token is not read yet
+    want = expected(range(12), 4)
+    assert s.step() == [("a", want[0])]          # the first decode step is queued, then token 0 is read
+    assert s.step() == [("a", want[1])]
+    assert s.step() == [("a", want[2])]          # the third decode step; a's last token needs no forward
+    assert eng.cache.free_pages() == [64] and s.has_work()          # it left the engine; its token is unread
+    assert s.step() == [("a", want[3])] and not s.has_work()
+    assert s.finished["a"].generated == want and s.finished["a"].finish_reason == "length"
+    assert eng.steps == [[("a", 5, False)], [("a", 5, False)], [("a", 2, True)],
+                         [("a", 1, True)], [("a", 1, True)], [("a", 1, True)]]
+
+
+def test_a_late_stop_token_costs_one_step_and_changes_nothing_else():
+    want = expected([5, 6], 5)
+    eng, s = make(overlap=True)
+    s.add("a", [5, 6], SamplingParams(max_tokens=5, stop_token_ids=(want[2],)))
+    done = s.run()
+    assert done["a"].generated == want[:2] and done["a"].finish_reason == "stop"
+    assert len(eng.steps) == 4                   # prompt, two decodes, and one in vain (3 without overlap)
+    assert eng.cache.free_pages() == [64] and eng.cache.slots.n_free == 4
+    # a stop token as the last token allowed: the reason is the stop, the token stays unsent
+    eng, s = make(overlap=True)
+    s.add("a", [5, 6], SamplingParams(max_tokens=3, stop_token_ids=(want[2],)))
+    done = s.run()
+    assert done["a"].generated == want[:2] and done["a"].finish_reason == "stop"
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_overlapped_and_waiting_loops_generate_the_same(seed):
+    """Random arrivals, stop tokens, so few pages that requests are pre-empted and some fail."""
+    runs = []
+    for overlap in (False, True):
+        rng = np.random.default_rng(seed)
+        eng, s = make(n_pages=12, overlap=overlap, max_batch_tokens=24, portion=7, max_running=3)
+        pending = []
+        for i in range(12):
+            prompt = rng.integers(0, VOCAB, size=int(rng.integers(1, 20))).tolist()
+            n = int(rng.integers(1, 14))
+            stops = tuple(rng.integers(0, VOCAB, size=int(rng.integers(0, 6))).tolist())
+            pending.append((i, prompt, n, stops))
+        while pending or s.has_work():
+            for _ in range(int(rng.integers(0, 3))):
+                if pending:
+                    i, prompt, n, stops = pending.pop(0)
+                    s.add(i, prompt, SamplingParams(max_tokens=n, stop_token_ids=stops))
+            if s.has_work():
+                s.step()
+                assert len(s.running) <= 3
+        assert eng.cache.free_pages() == [12] and eng.cache.slots.n_free == 4
+        runs.append({i: (r.generated, r.finish_reason) for i, r in s.finished.items()})
+        # against the plain recurrence
+        rng = np.random.default_rng(seed)
+        for i in range(12):
+            prompt = rng.integers(0, VOCAB, size=int(rng.integers(1, 20))).tolist()
+            n = int(rng.integers(1, 14))
+            stops = tuple(rng.integers(0, VOCAB, size=int(rng.integers(0, 6))).tolist())
+            got, reason = runs[-1][i]
+            if reason.startswith("error"):
+                continue
+            full = expected(prompt, n)
+            cut = next((j for j, t in enumerate(full) if t in stops), None)
+            assert got == (full if cut is None else full[:cut]) and reason == ("length" if cut is None else "stop")
+    assert runs[0] == runs[1]
+    assert any(len(g) for g, _ in runs[0].values())
+
+
+def test_overlapped_preemption_keeps_the_unread_token():
+    eng, s = make(n_pages=5, overlap=True, max_batch_tokens=64, portion=64)
+    s.add("old", list(range(6)), SamplingParams(max_tokens=8))
+    s.add("young", list(range(10, 16)), SamplingParams(max_tokens=8))
+    done = s.run()
+    assert ("preempt", "young") in s.log
+    assert done["old"].generated == expected(range(6), 8)
+    assert done["young"].generated == expected(range(10, 16), 8)
+    assert eng.cache.free_pages() == [5] and eng.cache.slots.n_free == 4
