@@ -36,88 +36,6 @@ struct Paged {
 
 __device__ __forceinline__ short pack_bf16(float f) { return (short)f32_to_bf16(f); }
 
-// The operands of one tile of 16 keys: K rows and V^T rows as the products take
-// them. Loading is apart from computing so that a wave can have the loads of
-// several tiles in flight before it waits for the first.
-template <int ND>
-struct TileRegs {
-    s16x4 k[ND];
-    s16x4 v[ND];
-};
-
-// Issues the loads of the tile starting at key_base (a multiple of 16).
-// [lo_all, hi_all] are the live keys any query of the wave may read: addresses
-// are clamped into it (what lies outside is forced to zero before use).
-template <int ND>
-__device__ __forceinline__ void load_tile(TileRegs<ND>& r, const Paged& kv, int key_base, int lo_all, int hi_all,
-                                          int lane) {
-    constexpr int D = ND * 16;
-    const int c = lane & 15, g = lane >> 4;
-    const int key = min(max(key_base + c, lo_all), hi_all);
-    int page = kv.table[key / kv.page_size];
-    page = min(max(page, 0), kv.n_pages - 1);
-    const bf16_t* krow = kv.k + (((size_t)page * kv.kv_heads + kv.kvh) * kv.page_size + (key % kv.page_size)) * D + 4 * g;
-    const int kgc = min(max(key_base + 4 * g, lo_all & ~3), hi_all & ~3);
-    int vpage = kv.table[kgc / kv.page_size];
-    vpage = min(max(vpage, 0), kv.n_pages - 1);
-    const bf16_t* vbase = kv.v + ((size_t)vpage * kv.kv_heads + kv.kvh) * kv.page_size * D + (kgc % kv.page_size);
-#pragma unroll
-    for (int dk = 0; dk < ND; ++dk) r.k[dk] = *reinterpret_cast<const s16x4*>(krow + dk * 16);
-#pragma unroll
-    for (int dt = 0; dt < ND; ++dt)
-        r.v[dt] = *reinterpret_cast<const s16x4*>(vbase + (size_t)(dt * 16 + c) * kv.page_size);
-}
-
-// One softmax step over a loaded tile. [lo_q, hi_q] is the key range of this
-// lane's query. `full`: every key of the tile is inside every query's range,
-// so no masking is needed.
-template <int ND>
-__device__ __forceinline__ void attn_tile(WaveState<ND>& st, const TileRegs<ND>& r, int key_base, int lo_q, int hi_q,
-                                          int lo_all, int hi_all, bool full, float scale, int lane) {
-    const int g = lane >> 4;
-    // ---- scores
-    f32x4 s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int dk = 0; dk < ND; ++dk) s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(r.k[dk], st.q[dk], s, 0, 0, 0);
-    const int kg = key_base + 4 * g;          // this lane's 4 keys: kg .. kg+3
-    float sv[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const bool ok = full || (kg + i >= lo_q && kg + i <= hi_q);
-        sv[i] = ok ? s[i] * scale : -INFINITY;
-    }
-    float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
-    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-    const float m_new = fmaxf(st.m, mx);
-    const float corr = (st.m == -INFINITY) ? 0.f : __expf(st.m - m_new);
-    s16x4 pb;
-    float psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float p = (sv[i] == -INFINITY) ? 0.f : __expf(sv[i] - m_new);
-        const bf16_t rb = f32_to_bf16(p);
-        pb[i] = (short)rb;
-        psum += bf16_to_f32(rb);              // the denominator sums what the product uses
-    }
-    psum += __shfl_xor(psum, 16, WAVE);
-    psum += __shfl_xor(psum, 32, WAVE);
-    st.l = st.l * corr + psum;
-    st.m = m_new;
-    // ---- weighted values
-#pragma unroll
-    for (int dt = 0; dt < ND; ++dt) {
-        s16x4 a = r.v[dt];
-        if (!full) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (kg + i < lo_all || kg + i > hi_all) a[i] = 0;   // stale or foreign memory: never multiplied
-        }
-        st.o[dt] = st.o[dt] * corr;
-        st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, st.o[dt], 0, 0, 0);
-    }
-}
-
 template <int ND>
 __device__ __forceinline__ void load_q(WaveState<ND>& st, const bf16_t* __restrict__ qrow, bool valid, int lane) {
     const int g = lane >> 4;
@@ -131,6 +49,133 @@ __device__ __forceinline__ void load_q(WaveState<ND>& st, const bf16_t* __restri
 }
 
 // ---------------------------------------------------------------- decode
+// The decode kernel walks the keys in tiles of 32 with the 16x16x32 product, so that every
+// lane loads 16 bytes at a time (half as many memory instructions as with tiles of 16):
+//   S^T: two products of 16 keys x 16 queries per 32 head dims. Which key an output row
+//        stands for is free to choose: row m of product t is key 8*(m/4) + 4*t + m%4, so
+//        that the 8 scores a lane ends up with (rows 4*(lane/16)+i of both products) are
+//        the 8 consecutive keys 8*(lane/16) .. +7,
+//   O^T: one product per 16 head dims over the 32 keys, whose B operand wants exactly
+//        those 8 consecutive keys per lane, and whose A operand is 16 bytes of a V^T row.
+// A head size that is no multiple of 32 pads the last product over head dims with zeros.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+union Frag8 {
+    uint4 u;
+    bf16x8 v;
+};
+
+template <int ND>
+struct DecodeState {
+    static constexpr int NK = (ND + 1) / 2;      // products of 32 over the head dims
+    f32x4 o[ND];        // O^T rows dt*16 + 4*(lane/16) + i of query lane%16
+    Frag8 q[NK];        // Q^T operand: dims dk*32 + 8*(lane/16) + j of query lane%16
+    float m, l;
+};
+
+template <int ND>
+struct DecodeTile {
+    Frag8 k[2][(ND + 1) / 2];
+    Frag8 v[ND];
+};
+
+__device__ __forceinline__ uint4 zero_unless(bool keep, uint4 v) {
+    return make_uint4(keep ? v.x : 0u, keep ? v.y : 0u, keep ? v.z : 0u, keep ? v.w : 0u);
+}
+
+// Issues the loads of the tile starting at key_base (a multiple of 32). [lo_all, hi_all] are
+// the live keys any query of the wave may read: addresses are clamped into it (what lies
+// outside is forced to zero before use). No load sits under a branch.
+template <int ND>
+__device__ __forceinline__ void decode_load(DecodeTile<ND>& r, const Paged& kv, int key_base, int lo_all, int hi_all,
+                                            int lane) {
+    constexpr int D = ND * 16, NK = (ND + 1) / 2;
+    const int c = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int key = min(max(key_base + 8 * (c >> 2) + 4 * t + (c & 3), lo_all), hi_all);
+        int page = kv.table[key / kv.page_size];
+        page = min(max(page, 0), kv.n_pages - 1);
+        const bf16_t* krow = kv.k + (((size_t)page * kv.kv_heads + kv.kvh) * kv.page_size + (key % kv.page_size)) * D;
+#pragma unroll
+        for (int dk = 0; dk < NK; ++dk)          // dims beyond D: read the row's last 8 again, zeroed in decode_tile
+            r.k[t][dk].u = *reinterpret_cast<const uint4*>(krow + min(dk * 32 + 8 * g, D - 8));
+    }
+    const int kgc = min(max(key_base + 8 * g, lo_all & ~7), hi_all & ~7);
+    int vpage = kv.table[kgc / kv.page_size];
+    vpage = min(max(vpage, 0), kv.n_pages - 1);
+    const bf16_t* vbase = kv.v + ((size_t)vpage * kv.kv_heads + kv.kvh) * kv.page_size * D + (kgc % kv.page_size);
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt)
+        r.v[dt].u = *reinterpret_cast<const uint4*>(vbase + (size_t)(dt * 16 + c) * kv.page_size);
+}
+
+// One softmax step over a loaded tile of 32 keys. [lo_q, hi_q] is the key range of this
+// lane's query. `full`: every key of the tile is inside every query's range.
+template <int ND>
+__device__ __forceinline__ void decode_tile(DecodeState<ND>& st, const DecodeTile<ND>& r, int key_base, int lo_q,
+                                            int hi_q, int lo_all, int hi_all, bool full, float scale, int lane) {
+    constexpr int D = ND * 16, NK = (ND + 1) / 2;
+    const int g = lane >> 4;
+    // ---- scores of keys kg .. kg+7: sv[4*t + i] from product t, row 4*g + i
+    f32x4 s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int dk = 0; dk < NK; ++dk) {
+            Frag8 a = r.k[t][dk];
+            if (dk * 32 + 32 > D) a.u = zero_unless(dk * 32 + 8 * g < D, a.u);
+            s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, st.q[dk].v, s[t], 0, 0, 0);
+        }
+    }
+    const int kg = key_base + 8 * g;
+    float sv[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const bool ok = full || (kg + j >= lo_q && kg + j <= hi_q);
+        sv[j] = ok ? s[j >> 2][j & 3] * scale : -INFINITY;
+        mx = fmaxf(mx, sv[j]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = fmaxf(st.m, mx);
+    const float corr = (st.m == -INFINITY) ? 0.f : __expf(st.m - m_new);
+    union {
+        uint4 u;
+        bf16x8 v;
+        bf16_t h[8];
+    } pb;
+    float psum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float p = (sv[j] == -INFINITY) ? 0.f : __expf(sv[j] - m_new);
+        pb.h[j] = f32_to_bf16(p);
+        psum += bf16_to_f32(pb.h[j]);             // the denominator sums what the product uses
+    }
+    psum += __shfl_xor(psum, 16, WAVE);
+    psum += __shfl_xor(psum, 32, WAVE);
+    st.l = st.l * corr + psum;
+    st.m = m_new;
+    // ---- weighted values
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) {
+        union {
+            uint4 u;
+            bf16x8 v;
+            bf16_t h[8];
+        } a;
+        a.u = r.v[dt].u;
+        if (!full) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (kg + j < lo_all || kg + j > hi_all) a.h[j] = 0;   // stale or foreign memory: never multiplied
+        }
+        st.o[dt] = st.o[dt] * corr;
+        st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb.v, st.o[dt], 0, 0, 0);
+    }
+}
+
 // grid (split, kv head x passes of 16 query heads, decode row). The four waves
 // of a block take the split's key tiles in turn, each with the loads of its
 // tiles in flight before the first product; their partial results meet in LDS
@@ -144,9 +189,8 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_decode(
     const int32_t* __restrict__ rows, const int32_t* __restrict__ seg_start, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int n_pages,
     float scale, int window, int n_splits) {
-    constexpr int D = ND * 16;
-    constexpr int TILES = DEC_SPLIT / (MFMA_WAVES * 16);   // tiles a wave takes at most
-    constexpr int DEPTH = ND <= 4 ? TILES : 2;             // of which this many are loaded ahead
+    constexpr int D = ND * 16, NK = (ND + 1) / 2;
+    constexpr int TILES = DEC_SPLIT / (MFMA_WAVES * 32);   // tiles a wave takes at most
     __shared__ float sm[MFMA_WAVES][16], sl[MFMA_WAVES][16];
     __shared__ float so[MFMA_WAVES][16][D + 1];
     const int split = blockIdx.x, ri = blockIdx.z;
@@ -156,7 +200,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_decode(
     const int t = seg_start[row];
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
-    const int k_begin = max(split * DEC_SPLIT, lo & ~15);
+    const int k_begin = max(split * DEC_SPLIT, lo & ~31);
     const int k_end = min((split + 1) * DEC_SPLIT, pos + 1);
     if (k_begin >= k_end) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -164,25 +208,31 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_decode(
     const int hq = pass * 16 + c;               // query head inside the group
     const bool qvalid = hq < G;
     const int head = kvh * G + min(hq, G - 1);
-    WaveState<ND> st;
-    load_q<ND>(st, q + ((size_t)t * heads + head) * D, qvalid, lane);
-    Paged kv{k_cache, v_cache, block_table + (size_t)row * table_stride, page_size, kv_heads, kvh, n_pages};
-    const int hi_q = qvalid ? pos : -1;
+    DecodeState<ND> st;
+    {
+        const bf16_t* qrow = q + ((size_t)t * heads + head) * D;
 #pragma unroll
-    for (int j0 = 0; j0 < TILES; j0 += DEPTH) {
-        TileRegs<ND> regs[DEPTH];
-#pragma unroll
-        for (int j = 0; j < DEPTH; ++j) {
-            const int kb = k_begin + (wave + (j0 + j) * MFMA_WAVES) * 16;
-            if (kb < k_end) load_tile<ND>(regs[j], kv, kb, lo, pos, lane);
+        for (int dk = 0; dk < NK; ++dk) {
+            const int d = dk * 32 + 8 * g;
+            st.q[dk].u = zero_unless(qvalid && d < D, *reinterpret_cast<const uint4*>(qrow + min(d, D - 8)));
         }
 #pragma unroll
-        for (int j = 0; j < DEPTH; ++j) {
-            const int kb = k_begin + (wave + (j0 + j) * MFMA_WAVES) * 16;
-            if (kb < k_end) {
-                const bool full = kb >= lo && kb + 15 <= pos;
-                attn_tile<ND>(st, regs[j], kb, lo, hi_q, lo, pos, full, scale, lane);
-            }
+        for (int dt = 0; dt < ND; ++dt) st.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        st.m = -INFINITY;
+        st.l = 0.f;
+    }
+    Paged kv{k_cache, v_cache, block_table + (size_t)row * table_stride, page_size, kv_heads, kvh, n_pages};
+    const int hi_q = qvalid ? pos : -1;
+    DecodeTile<ND> regs[TILES];
+#pragma unroll
+    for (int j = 0; j < TILES; ++j)             // past the split's end: clamped addresses, never used
+        decode_load<ND>(regs[j], kv, k_begin + (wave + j * MFMA_WAVES) * 32, lo, pos, lane);
+#pragma unroll
+    for (int j = 0; j < TILES; ++j) {
+        const int kb = k_begin + (wave + j * MFMA_WAVES) * 32;
+        if (kb < k_end) {
+            const bool full = kb >= lo && kb + 31 <= pos;
+            decode_tile<ND>(st, regs[j], kb, lo, hi_q, lo, pos, full, scale, lane);
         }
     }
     if (g == 0) {
