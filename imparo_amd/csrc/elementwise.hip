@@ -101,7 +101,11 @@ __global__ void k_rms_norm(float* __restrict__ x, const float* __restrict__ delt
 }
 
 // The same for rows whose width is a multiple of 4 and at most 4 * blockDim:
-// one float4 per thread, every load of the row issued before anything waits.
+// one float4 per thread. Every load of the row is issued before anything
+// waits, the slices of the delta four at a time from clamped addresses: what a
+// decode step hands this kernel was written a moment ago by another kernel and
+// is in no near cache, so a load that waits for the one before costs a trip to
+// memory each.
 template <typename TOut>
 __global__ void k_rms_norm_v4(float* __restrict__ x, const float* __restrict__ delta, int n_delta, size_t delta_stride,
                               const int32_t* __restrict__ rows, const float* __restrict__ weight,
@@ -110,29 +114,33 @@ __global__ void k_rms_norm_v4(float* __restrict__ x, const float* __restrict__ d
     const int i_out = blockIdx.x;
     const size_t src = (size_t)(rows ? rows[i_out] : i_out) * width;
     const size_t dst = (size_t)i_out * width;
-    const int i = threadIdx.x * 4;
-    const bool in = i < width;
-    float4 a = make_float4(0.f, 0.f, 0.f, 0.f), w = a;
-    if (in) {
-        a = *reinterpret_cast<const float4*>(x + src + i);
-        w = *reinterpret_cast<const float4*>(weight + i);
-        float4 d = make_float4(0.f, 0.f, 0.f, 0.f);   // the slices make up the delta first, then the delta joins x
-        for (int s = 0; s < n_delta; ++s) {
-            const float4 p = *reinterpret_cast<const float4*>(delta + s * delta_stride + src + i);
-            d.x += p.x;
-            d.y += p.y;
-            d.z += p.z;
-            d.w += p.w;
+    const bool in = (int)threadIdx.x * 4 < width;
+    const int i = min((int)threadIdx.x * 4, width - 4);      // threads past the row repeat its end and store nothing
+    float4 a = *reinterpret_cast<const float4*>(x + src + i);
+    const float4 w = *reinterpret_cast<const float4*>(weight + i);
+    float4 d = make_float4(0.f, 0.f, 0.f, 0.f);   // the slices make up the delta first, then the delta joins x
+    for (int s0 = 0; s0 < n_delta; s0 += 4) {
+        float4 p[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            p[j] = *reinterpret_cast<const float4*>(delta + (size_t)min(s0 + j, n_delta - 1) * delta_stride + src + i);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bool on = s0 + j < n_delta;
+            d.x += on ? p[j].x : 0.f;
+            d.y += on ? p[j].y : 0.f;
+            d.z += on ? p[j].z : 0.f;
+            d.w += on ? p[j].w : 0.f;
         }
-        a.x += d.x;
-        a.y += d.y;
-        a.z += d.z;
-        a.w += d.w;
-        if (write_back) *reinterpret_cast<float4*>(x + src + i) = a;
     }
+    a.x += d.x;
+    a.y += d.y;
+    a.z += d.z;
+    a.w += d.w;
+    if (write_back && in) *reinterpret_cast<float4*>(x + src + i) = a;
     // the same order of squares as the scalar kernel would not matter: each kernel is
     // used for a given width whatever the batch, so a row always sums the same way
-    const float ss = a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
+    const float ss = in ? a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w : 0.f;
     const float total = block_sum(ss, scratch);
     const float scale = 1.0f / sqrtf(total / (float)width + eps);
     if (in) {
@@ -293,29 +301,65 @@ extern "C" int imparo_short_conv(const float* bcx, const float* weight, const fl
 
 // Single-token rows: one thread per (row, channel) reads the history, writes
 // the output and the shifted history. It owns its channel, so nothing races.
-template <typename TOut>
+// HIST > 0: the history length is known at compile time and everything the
+// thread needs is loaded before the first value is used (one trip to memory
+// instead of one per tap; what a decode step hands this kernel is in no near
+// cache). HIST == 0: any length, tap by tap.
+template <typename TOut, int HIST>
 __global__ void k_short_conv_decode(const float* __restrict__ bcx, const float* __restrict__ weight,
                                     const float* __restrict__ bias, float* __restrict__ state,
                                     const int32_t* __restrict__ slot, TOut* __restrict__ out, int width, int taps) {
     const int ch = blockIdx.x * blockDim.x + threadIdx.x;
     const int r = blockIdx.y;
     if (ch >= width) return;
-    const int history = taps - 1;
+    const int history = HIST > 0 ? HIST : taps - 1;
     float* st = state + (size_t)slot[r] * history * width;
     const size_t row = (size_t)r * 3 * width;
-    const float u = bcx[row + ch] * bcx[row + 2 * width + ch];
+    const float b_in = bcx[row + ch], c_in = bcx[row + width + ch], x_in = bcx[row + 2 * width + ch];
+    const float bias_v = bias ? bias[ch] : 0.f;
     // the taps are summed oldest first, exactly as the general kernel sums them
     float acc = 0.f;
-    float prev = st[ch];                                  // oldest
-    for (int k = 0; k < history; ++k) {
-        acc = fmaf(weight[(size_t)ch * taps + k], prev, acc);
-        const float next = (k + 1 < history) ? st[(size_t)(k + 1) * width + ch] : u;
-        st[(size_t)k * width + ch] = next;
-        prev = next;
+    if (HIST > 0) {
+        float h[HIST > 0 ? HIST : 1], w[(HIST > 0 ? HIST : 1) + 1];
+#pragma unroll
+        for (int k = 0; k < HIST; ++k) h[k] = st[(size_t)k * width + ch];
+#pragma unroll
+        for (int k = 0; k <= HIST; ++k) w[k] = weight[(size_t)ch * (HIST + 1) + k];
+        const float u = b_in * x_in;
+#pragma unroll
+        for (int k = 0; k < HIST; ++k) {
+            acc = fmaf(w[k], h[k], acc);
+            st[(size_t)k * width + ch] = k + 1 < HIST ? h[k + 1] : u;
+        }
+        acc = fmaf(w[HIST], u, acc);
+    } else {
+        const float u = b_in * x_in;
+        float prev = st[ch];                                  // oldest
+        for (int k = 0; k < history; ++k) {
+            acc = fmaf(weight[(size_t)ch * taps + k], prev, acc);
+            const float next = (k + 1 < history) ? st[(size_t)(k + 1) * width + ch] : u;
+            st[(size_t)k * width + ch] = next;
+            prev = next;
+        }
+        acc = fmaf(weight[(size_t)ch * taps + history], u, acc);
     }
-    acc = fmaf(weight[(size_t)ch * taps + history], u, acc);
-    if (bias) acc += bias[ch];
-    store_f32<TOut>(out, (size_t)r * width + ch, bcx[row + width + ch] * acc);
+    acc += bias_v;
+    store_f32<TOut>(out, (size_t)r * width + ch, c_in * acc);
+}
+
+template <typename TOut>
+static void launch_conv_decode(dim3 grid, int threads, hipStream_t s, const float* bcx, const float* weight,
+                               const float* bias, float* state, const int32_t* slot, TOut* out, int width, int taps) {
+    switch (taps - 1) {
+        case 1: k_short_conv_decode<TOut, 1><<<grid, threads, 0, s>>>(bcx, weight, bias, state, slot, out, width, taps); break;
+        case 2: k_short_conv_decode<TOut, 2><<<grid, threads, 0, s>>>(bcx, weight, bias, state, slot, out, width, taps); break;
+        case 3: k_short_conv_decode<TOut, 3><<<grid, threads, 0, s>>>(bcx, weight, bias, state, slot, out, width, taps); break;
+        case 4: k_short_conv_decode<TOut, 4><<<grid, threads, 0, s>>>(bcx, weight, bias, state, slot, out, width, taps); break;
+        case 5: k_short_conv_decode<TOut, 5><<<grid, threads, 0, s>>>(bcx, weight, bias, state, slot, out, width, taps); break;
+        case 6: k_short_conv_decode<TOut, 6><<<grid, threads, 0, s>>>(bcx, weight, bias, state, slot, out, width, taps); break;
+        case 7: k_short_conv_decode<TOut, 7><<<grid, threads, 0, s>>>(bcx, weight, bias, state, slot, out, width, taps); break;
+        default: k_short_conv_decode<TOut, 0><<<grid, threads, 0, s>>>(bcx, weight, bias, state, slot, out, width, taps);
+    }
 }
 
 extern "C" int imparo_short_conv_decode(const float* bcx, const float* weight, const float* bias, float* state,
@@ -329,9 +373,9 @@ extern "C" int imparo_short_conv_decode(const float* bcx, const float* weight, c
     const int threads = width >= 256 ? 256 : 64;
     dim3 grid((width + threads - 1) / threads, n_rows);
     if (out_dtype == IMPARO_F32)
-        k_short_conv_decode<float><<<grid, threads, 0, s>>>(bcx, weight, bias, state, slot, (float*)out, width, taps);
+        launch_conv_decode<float>(grid, threads, s, bcx, weight, bias, state, slot, (float*)out, width, taps);
     else if (out_dtype == IMPARO_BF16)
-        k_short_conv_decode<bf16_t><<<grid, threads, 0, s>>>(bcx, weight, bias, state, slot, (bf16_t*)out, width, taps);
+        launch_conv_decode<bf16_t>(grid, threads, s, bcx, weight, bias, state, slot, (bf16_t*)out, width, taps);
     else
         return IMPARO_BAD_ARGUMENT;
     return launch_status();

@@ -33,30 +33,56 @@ __global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float*
     const bool is_v = u >= heads + kv_heads;
     const float* weight = is_q ? q_weight : k_weight;
 
-    float ss = 0.f;
-    for (int i = lane; i < head_dim; i += WAVE) {
-        const float a = src[i];
-        row[i] = a;
-        ss += a * a;
+    // Everything the wave needs is asked for before the first value is used: what a decode
+    // step hands this kernel is in no near cache, and each load that waits for the one
+    // before costs a trip to memory.
+    constexpr int PER_LANE = ROPE_MAX_HEAD_DIM / WAVE;
+    const int pos = positions[t];
+    int page = -1;
+    if (!is_q && write_kv) page = block_table[(size_t)row_of_token[t] * table_stride + pos / page_size];
+    float a[PER_LANE], w[PER_LANE], freq[PER_LANE];
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+        const int i = lane + j * WAVE;
+        a[j] = i < head_dim ? src[i] : 0.f;
+        w[j] = (i < head_dim && weight && !is_v) ? weight[i] : 1.f;
+        freq[j] = (i < n_freq && !is_v) ? inv_freq[i] : 0.f;
     }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) ss += a[j] * a[j];     // in the order i = lane, lane + 64, ...
     if (!is_v) {
+        float scale = 1.f;
         if (weight) {
             ss = wave_sum(ss);
-            const float scale = 1.0f / sqrtf(ss / (float)head_dim + eps);
-            for (int i = lane; i < head_dim; i += WAVE) row[i] = row[i] * scale * weight[i];
+            scale = 1.0f / sqrtf(ss / (float)head_dim + eps);
+        }
+#pragma unroll
+        for (int j = 0; j < PER_LANE; ++j) {
+            const int i = lane + j * WAVE;
+            if (i < head_dim) row[i] = weight ? a[j] * scale * w[j] : a[j];
         }
         wave_lds_sync();   // a pair's second element may have been written by another lane
         if (n_freq > 0) {
-            const int pos = positions[t];
             // each lane owns pair (i, i + n_freq): reads both, then writes both
-            for (int i = lane; i < n_freq; i += WAVE) {
-                const float theta = (float)((double)pos * (double)inv_freq[i]);
-                float sn, cs;
-                sincosf(theta, &sn, &cs);
-                const float x0 = row[i], x1 = row[i + n_freq];
-                row[i] = x0 * cs - x1 * sn;
-                row[i + n_freq] = x0 * sn + x1 * cs;
+#pragma unroll
+            for (int j = 0; j < PER_LANE; ++j) {
+                const int i = lane + j * WAVE;
+                if (i < n_freq) {
+                    const float theta = (float)((double)pos * (double)freq[j]);
+                    float sn, cs;
+                    sincosf(theta, &sn, &cs);
+                    const float x0 = row[i], x1 = row[i + n_freq];
+                    row[i] = x0 * cs - x1 * sn;
+                    row[i + n_freq] = x0 * sn + x1 * cs;
+                }
             }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < PER_LANE; ++j) {
+            const int i = lane + j * WAVE;
+            if (i < head_dim) row[i] = a[j];
         }
     }
     wave_lds_sync();
@@ -68,8 +94,6 @@ __global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float*
     }
     if (!write_kv) return;
     const int kvh = is_v ? u - heads - kv_heads : u - heads;
-    const int pos = positions[t];
-    const int page = block_table[(size_t)row_of_token[t] * table_stride + pos / page_size];
     if (page < 0 || page >= n_pages) return;   // never write outside the pool
     if (is_v && v_transposed) {
         // [page, kv head, dim, slot]: the keys of one dimension lie side by side
