@@ -365,6 +365,8 @@ __global__ __launch_bounds__(WM * WN * 64) void k_gemm_bf16_big(const bf16_t* __
     const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
     const int a_base = (wm * TM * 32 + frag_row) * BG_LD + frag_k;
     const int b_base = (wn * TN * 32 + frag_row) * BG_LD + frag_k;
+    // (reading the fragments of sub-step ks+1 by hand before the products of ks, as the 128x128
+    // kernel does, costs registers this tile does not have: it spills and runs slower)
     auto compute = [&](int buf) {
 #pragma unroll
         for (int ks = 0; ks < BG_BK / 16; ++ks) {
