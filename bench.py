@@ -108,6 +108,108 @@ def prefill_run(engine, tokens, vocab, reps, seed):
     return best
 
 
+def shape(hidden, heads, block_ff_dim):
+    """The layer sizes of the smaller LFM2 checkpoints: same layout as the 1.2B, other widths."""
+    cfg = dict(LFM2_1_2B)
+    cfg.update(hidden_size=hidden, num_attention_heads=heads, block_ff_dim=block_ff_dim)
+    return cfg
+
+
+def serving_workload(dtype):
+    """Continuous batching: 32 requests, prompts of 64..3072 tokens, replies of 32..512 tokens, in 4
+    waves of 8 (a wave every 48 steps), 512-token portions beside decoded tokens. LFM2-700M shape."""
+    import numpy as np
+    import torch
+    from imparo_amd import write_random_model
+    from imparo_amd.engine import Engine
+    from imparo_amd.engine.scheduler import Scheduler
+    from imparo_amd.sampling import Sampler, SamplingParams
+    cfg = shape(1536, 24, 10240)
+    tmp = tempfile.mkdtemp(prefix="imparo_bench_")
+    write_random_model(cfg, 3, tmp)
+    engine = Engine(tmp, dtype=dtype, max_tokens=32 * (3072 + 512 + 64), page_size=64, max_requests=32)
+    sampler = Sampler(engine.device)
+    rng = np.random.default_rng(3)
+    jobs = [(i, rng.integers(0, cfg["vocab_size"], size=int(rng.integers(64, 3073))).tolist(), int(rng.integers(32, 513)))
+            for i in range(32)]
+    sched = Scheduler(engine, sampler.pick, max_batch_tokens=2048, max_running=32, portion=512,
+                      pick_async=sampler.pick_async)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    steps = 0
+    while jobs or sched.has_work():
+        if jobs and steps % 48 == 0:
+            for i, prompt, n in jobs[:8]:
+                sched.add(i, prompt, SamplingParams(max_tokens=n, stop_token_ids=()))
+            jobs = jobs[8:]
+        sched.step()
+        steps += 1
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    done = sched.finished
+    n_prompt = sum(len(r.prompt) for r in done.values())
+    n_out = sum(len(r.generated) for r in done.values())
+    assert len(done) == 32 and all(r.finish_reason == "length" for r in done.values())
+    print(json.dumps({
+        "metric": "continuous batching, LFM2-700M shape: generated tok/s over the whole run", "value": round(n_out / dt, 1),
+        "unit": "tok/s", "n_gpus": 1, "seconds": round(dt, 3), "steps": steps, "prompt_tokens": n_prompt,
+        "generated_tokens": n_out, "all_tokens_per_s": round((n_prompt + n_out) / dt, 1),
+        "preemptions": sum(r.preemptions for r in done.values()), "dtype": "bf16" if dtype == "bfloat16" else "fp32",
+        "data": "synthetic token ids, random weights (seed 3)",
+        "config": {"model": "LFM2-700M shape", "requests": 32, "waves": 4, "portion": 512, "max_batch_tokens": 2048,
+                   "hidden_size": 1536, "heads": 24, "kv_heads": 8, "ff_dim": 6912, "layers": 16}}), flush=True)
+    return 0
+
+
+def long_workload(dtype, requests, prompt_len):
+    """Long contexts: `requests` concurrent requests, each a prompt of `prompt_len` tokens fed in
+    2,048-token portions, then 128 decoded tokens each. LFM2-350M shape."""
+    import torch
+    from imparo_amd import write_random_model
+    from imparo_amd.engine import DeviceToken, Engine, StepEntry
+    from imparo_amd.sampling import Sampler
+    cfg = shape(1024, 16, 6656)
+    tmp = tempfile.mkdtemp(prefix="imparo_bench_")
+    write_random_model(cfg, 4, tmp)
+    engine = Engine(tmp, dtype=dtype, max_tokens=requests * (prompt_len + 128 + 64), page_size=64, max_requests=requests)
+    sampler = Sampler(engine.device)
+    g = torch.Generator().manual_seed(4)
+    ids = list(range(requests))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    last = []
+    for rid in ids:
+        prompt = torch.randint(0, cfg["vocab_size"], (prompt_len,), generator=g).tolist()
+        for lo in range(0, prompt_len, 2048):
+            hi = min(prompt_len, lo + 2048)
+            out = engine.step([StepEntry(rid, prompt[lo:hi], [hi - lo - 1] if hi == prompt_len else [])])
+        last.append(out)
+        if rid % 8 == 7:
+            print(f"[bench] {rid + 1} of {requests} prompts are in the cache", file=sys.stderr, flush=True)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    zeros = [0.0] * requests
+    picked = sampler.pick_async(torch.cat(last), zeros, zeros)
+    for _ in range(128 - 1):
+        logits = engine.step([StepEntry(rid, [DeviceToken(picked.on_device, i)], [0]) for i, rid in enumerate(ids)])
+        following = sampler.pick_async(logits, zeros, zeros)
+        picked.tokens()
+        picked = following
+    picked.tokens()
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    print(json.dumps({
+        "metric": "long contexts, LFM2-350M shape: decode tok/s with every request at its full context",
+        "value": round(requests * 127 / (t2 - t1), 1), "unit": "tok/s", "n_gpus": 1,
+        "prefill_tok_s": round(requests * prompt_len / (t1 - t0), 1), "prefill_seconds": round(t1 - t0, 3),
+        "decode_ms_per_step": round((t2 - t1) / 127 * 1e3, 3), "dtype": "bf16" if dtype == "bfloat16" else "fp32",
+        "data": "synthetic token ids, random weights (seed 4)",
+        "config": {"model": "LFM2-350M shape", "requests": requests, "prompt_len": prompt_len, "portion": 2048,
+                   "decode_tokens": 128, "hidden_size": 1024, "heads": 16, "kv_heads": 8, "ff_dim": 4608, "layers": 16,
+                   "cache_pages_used": engine.cache.groups[0].pool.n_pages - engine.free_pages()[0]}}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -119,10 +221,20 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="run only the 2,048-token prefill (for profiling)")
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "long"],
+                    help="decode: the headline line (default). serving: continuous batching of 32 requests in 4 "
+                         "waves (LFM2-700M shape). long: 64 requests of 32,768-token prompts, then 128 tokens "
+                         "each (LFM2-350M shape). The last two print a line of their own")
+    ap.add_argument("--requests", type=int, default=64, help="--workload long: concurrent requests")
+    ap.add_argument("--prompt-len", type=int, default=32768, help="--workload long: tokens per prompt")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.workload == "serving":
+        return serving_workload(args.dtype)
+    if args.workload == "long":
+        return long_workload(args.dtype, args.requests, args.prompt_len)
 
     import torch
     from imparo_amd import write_random_model

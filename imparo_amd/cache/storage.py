@@ -8,12 +8,12 @@ page_size]. Per site with a fixed spec: [n_slots, *shape] float32.
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Dict, Tuple
 
 import torch
 
 from ..kernels import ops
-from .pages import CacheManager, FixedSpec, PagedSpec, StateSpec
+from .pages import CacheManager, FixedSpec, PagedSpec
 
 
 class CacheStorage:

@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import math
 from dataclasses import dataclass, field, asdict
-from typing import Any, Dict, List, Optional, Tuple
+from typing import Any, Dict, List, Optional
 
 from .errors import MissingKey, BadValue, Inconsistent
 from .plan import PartSpec, LayerPlan, LayerCall, ModelPlan

@@ -12,13 +12,13 @@ one batch.
 from __future__ import annotations
 
 import math
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
-from ..cache.pages import CacheError, CacheManager, OutOfPages
+from ..cache.pages import CacheError, CacheManager
 from ..cache.storage import CacheStorage
 from ..config import plan_from_config, read_config_json
 from ..kernels import library, ops

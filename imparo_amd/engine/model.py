@@ -8,15 +8,14 @@ reads another call's cache is bound to that call's site.
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional, Tuple
+from typing import Dict, List, Optional
 
 import torch
 
 from ..cache.pages import StateSpec
-from ..config.plan import LayerPlan, ModelPlan, PartSpec
+from ..config.plan import ModelPlan, PartSpec
 from ..parts import part_class
 from ..parts.base import Declared, Residual, StepContext
-from ..weights.loader import TensorDecl
 
 
 def _declare(role: str, spec: PartSpec) -> Declared:

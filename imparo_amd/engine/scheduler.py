@@ -17,11 +17,9 @@ from __future__ import annotations
 
 import ctypes
 import os
-from collections import deque
 from dataclasses import dataclass, field
-from typing import Callable, Deque, Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Callable, Dict, Hashable, List, Optional, Sequence, Tuple
 
-from ..cache.pages import OutOfPages
 from ..sampling.sampler import SamplingParams, uniform_for
 
 DEFAULT_PORTION = 512   # the reference's prefill chunk (crates/imparo-model/src/lib.rs:1000)

@@ -6,7 +6,6 @@ delta is left pending on the residual stream so that the next norm, whichever
 block it belongs to, adds it while reading the row."""
 from __future__ import annotations
 
-import torch
 
 from .base import Residual, StepContext
 from .registry import register_part

@@ -7,7 +7,6 @@ from typing import Dict
 import torch
 
 from ..config.plan import PartSpec
-from ..kernels import ops
 from ..weights.loader import TensorDecl
 from .base import Declared, StepContext
 from .linear import Linear, place_matrix

@@ -4,7 +4,7 @@ precedes a norm is fused into it (the reference's add_rms_norm,
 /root/reference/crates/imparo-backend/src/lib.rs:2603-2609)."""
 from __future__ import annotations
 
-from typing import Dict, Optional
+from typing import Dict
 
 import torch
 

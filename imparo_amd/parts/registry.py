@@ -4,7 +4,7 @@ registered here, by the framework or by a user, can appear in a plan.
 """
 from __future__ import annotations
 
-from typing import Dict, Type
+from typing import Dict
 
 ROLES = ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head")
 _PARTS: Dict[str, Dict[str, type]] = {role: {} for role in ROLES}

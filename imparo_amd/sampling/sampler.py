@@ -11,10 +11,9 @@ request's draws do not depend on what it was batched with.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import List, Optional, Sequence, Tuple
 
-import numpy as np
 
 _MASK = (1 << 64) - 1
 

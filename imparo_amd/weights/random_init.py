@@ -10,7 +10,7 @@ from __future__ import annotations
 import hashlib
 import json
 import os
-from typing import Any, Dict, Iterable, Optional
+from typing import Any, Dict, Iterable
 
 import torch
 
