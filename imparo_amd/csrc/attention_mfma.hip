@@ -360,7 +360,11 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
     constexpr int LDK = PF_LD_K(D);
     __shared__ __attribute__((aligned(16))) bf16_t ks[2][PF_KEYS * LDK];
     __shared__ __attribute__((aligned(16))) bf16_t vs[2][D * PF_LD_V];
+    // Later tiles of a prompt have more keys to walk. Blocks whose numbers differ by the number
+    // of CUs tend to share a CU: every other group of 256 blocks takes the tiles in reverse, so
+    // that a long walk sits beside a short one.
     int tile = blockIdx.x, row = -1;
+    if (((blockIdx.y * gridDim.x + blockIdx.x) / 256) & 1) tile = (int)gridDim.x - 1 - tile;
     for (int i = 0; i < n_rows; ++i) {
         const int r = rows[i];
         const int nt = (seg_len[r] + 63) >> 6;
@@ -400,6 +404,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
     const int lo_max = window > 0 ? max(0, pos_last + 1 - window) : 0;
     WaveState<ND> st;
     load_q<ND>(st, q + ((size_t)(t0 + min(qi, len - 1)) * heads + head) * D, qvalid && wave_on, lane);
+    const float scale_log2 = scale * 1.44269504088896340736f;
 
     // staging: K tile = 64 keys x D/8 pieces of 16 bytes; V^T tile = D rows x 8 pieces of 8 keys
     constexpr int K_PIECES = PF_KEYS * (D / 8), V_PIECES = D * (PF_KEYS / 8);
@@ -475,7 +480,8 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
                     sc[kt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, st.q[dk], sc[kt], 0, 0, 0);
                 }
             }
-            // sc[kt][i] = score of key kb + 16 kt + 4 g + i for query lane%16
+            // sc[kt][i] = score of key kb + 16 kt + 4 g + i for query lane%16. The running maximum
+            // st.m is kept in units of log2(e), so that every weight is one exp2 of a difference.
             float mx = -INFINITY;
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
@@ -483,24 +489,31 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
                 for (int i = 0; i < 4; ++i) {
                     const int kp = kb + kt * 16 + 4 * g + i;
                     const bool ok = full || (kp >= lo_q && kp <= hi_q);
-                    sc[kt][i] = ok ? sc[kt][i] * scale : -INFINITY;
+                    sc[kt][i] = ok ? sc[kt][i] * scale_log2 : -INFINITY;
                     mx = fmaxf(mx, sc[kt][i]);
                 }
             mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
             mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
             const float m_new = fmaxf(st.m, mx);
-            const float corr = (st.m == -INFINITY) ? 0.f : __expf(st.m - m_new);
+            const float corr = (st.m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(st.m - m_new);
+            const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;        // exp2(-inf - 0) = 0: masked keys
             s16x4 pb[4];
             float psum = 0.f;
 #pragma unroll
-            for (int kt = 0; kt < 4; ++kt)
+            for (int kt = 0; kt < 4; ++kt) {
+                union {
+                    uint32_t u[2];
+                    s16x4 v;
+                } pk;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float p = (sc[kt][i] == -INFINITY) ? 0.f : __expf(sc[kt][i] - m_new);
-                    const bf16_t r = f32_to_bf16(p);
-                    pb[kt][i] = (short)r;
-                    psum += bf16_to_f32(r);
+                for (int i = 0; i < 4; i += 2) {
+                    const float p0 = __builtin_amdgcn_exp2f(sc[kt][i] - m_sub), p1 = __builtin_amdgcn_exp2f(sc[kt][i + 1] - m_sub);
+                    pk.u[i >> 1] = f32x2_to_bf16x2(p0, p1);
+                    // the denominator sums what the product uses
+                    psum += __uint_as_float(pk.u[i >> 1] << 16) + __uint_as_float(pk.u[i >> 1] & 0xffff0000u);
                 }
+                pb[kt] = pk.v;
+            }
             psum += __shfl_xor(psum, 16, WAVE);
             psum += __shfl_xor(psum, 32, WAVE);
             st.l = st.l * corr + psum;

@@ -20,12 +20,17 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
     return __uint_as_float(((uint32_t)v) << 16);
 }
 
-// round to nearest even; NaN stays NaN
+// round to nearest even; NaN stays NaN (gfx950 converts in hardware, two values per instruction)
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
+    const __bf16 b = (__bf16)f;
+    return *reinterpret_cast<const bf16_t*>(&b);
+}
+
+// two values in one register, `lo` in the low half
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const bf16x2_t b = {(__bf16)lo, (__bf16)hi};
+    return *reinterpret_cast<const uint32_t*>(&b);
 }
 
 template <typename T> __device__ __forceinline__ float load_f32(const T* p, size_t i);
