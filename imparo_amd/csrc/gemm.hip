@@ -285,11 +285,15 @@ __global__ __launch_bounds__(256, 2) void k_gemm_bf16_tile(const bf16_t* __restr
 }
 
 // ------------------------------------------------------------------ bfloat16, many rows, large tiles
-// The 128x128 kernel moves (128 + 128) rows of K per 128 x 128 outputs through L2: 64 flops a byte,
-// which at this chip's L2 bandwidth caps it near 650 TFLOP/s whatever the matrix cores could do.
-// This kernel takes a WM x WN grid of waves, each TM x TN MFMA tiles of 32x32, so that a block's
-// tile is (WM TM 32) x (WN TN 32): 256 x 256 moves half the bytes per flop. One block per CU
+// What bounds these tile kernels is LDS: a CU reads about 60 bytes a clock from it (measured with
+// this kernel's fragment pattern, no bank conflicts), and the 128x128 kernel's waves (2x2 MFMA
+// tiles each) read one 1 KB fragment per product. This kernel takes a WM x WN grid of waves, each
+// TM x TN MFMA tiles of 32x32, so that a block's tile is (WM TM 32) x (WN TN 32): with 4x2 tiles
+// a wave reads three fragments per four products, and throughput goes up by that ratio. One block per CU
 // (its LDS holds two K-steps of both operands), global loads two K-steps ahead in registers.
+// (Four waves of 128x128 each would halve the LDS reads per product again, and LDS reads, at about
+// 60 bytes a clock per CU, are what bounds this kernel; the compiler spills that variant's 256
+// accumulator registers inside the loop and it runs five times slower, so it is not built.)
 template <typename TOut, int WM, int WN, int TM, int TN>
 __global__ __launch_bounds__(WM * WN * 64) void k_gemm_bf16_big(const bf16_t* __restrict__ X,
                                                                 const bf16_t* __restrict__ W,
@@ -396,12 +400,10 @@ __global__ __launch_bounds__(WM * WN * 64) void k_gemm_bf16_big(const bf16_t* __
     stash(0, 0, a0, b0);
     fetch(2, a0, b0);
     __syncthreads();
-    int kt = 0;
-    for (; kt + 2 <= nk; kt += 2) {                // whole rounds of the two sets, free of branches
-        step(kt, a1, b1);
+    for (int kt = 0; kt < nk; kt += 2) {           // rounds of the two sets, free of branches: with an odd
+        step(kt, a1, b1);                          // number of K-steps the last round multiplies a step of zeros
         step(kt + 1, a0, b0);
     }
-    if (kt < nk) step(kt, a1, b1);
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
