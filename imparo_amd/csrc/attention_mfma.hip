@@ -32,6 +32,7 @@ struct Paged {
     const bf16_t* __restrict__ v;
     const int32_t* __restrict__ table;
     int page_size, kv_heads, kvh, n_pages;
+    int page_shift;     // page_size is a power of two: divisions by it are shifts
 };
 
 __device__ __forceinline__ short pack_bf16(float f) { return (short)f32_to_bf16(f); }
@@ -93,17 +94,17 @@ __device__ __forceinline__ void decode_load(DecodeTile<ND>& r, const Paged& kv, 
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         const int key = min(max(key_base + 8 * (c >> 2) + 4 * t + (c & 3), lo_all), hi_all);
-        int page = kv.table[key / kv.page_size];
+        int page = kv.table[key >> kv.page_shift];
         page = min(max(page, 0), kv.n_pages - 1);
-        const bf16_t* krow = kv.k + (((size_t)page * kv.kv_heads + kv.kvh) * kv.page_size + (key % kv.page_size)) * D;
+        const bf16_t* krow = kv.k + (((size_t)page * kv.kv_heads + kv.kvh) * kv.page_size + (key & (kv.page_size - 1))) * D;
 #pragma unroll
         for (int dk = 0; dk < NK; ++dk)          // dims beyond D: read the row's last 8 again, zeroed in decode_tile
             r.k[t][dk].u = *reinterpret_cast<const uint4*>(krow + min(dk * 32 + 8 * g, D - 8));
     }
     const int kgc = min(max(key_base + 8 * g, lo_all & ~7), hi_all & ~7);
-    int vpage = kv.table[kgc / kv.page_size];
+    int vpage = kv.table[kgc >> kv.page_shift];
     vpage = min(max(vpage, 0), kv.n_pages - 1);
-    const bf16_t* vbase = kv.v + ((size_t)vpage * kv.kv_heads + kv.kvh) * kv.page_size * D + (kgc % kv.page_size);
+    const bf16_t* vbase = kv.v + ((size_t)vpage * kv.kv_heads + kv.kvh) * kv.page_size * D + (kgc & (kv.page_size - 1));
 #pragma unroll
     for (int dt = 0; dt < ND; ++dt)
         r.v[dt].u = *reinterpret_cast<const uint4*>(vbase + (size_t)(dt * 16 + c) * kv.page_size);
@@ -221,7 +222,8 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_decode(
         st.m = -INFINITY;
         st.l = 0.f;
     }
-    Paged kv{k_cache, v_cache, block_table + (size_t)row * table_stride, page_size, kv_heads, kvh, n_pages};
+    Paged kv{k_cache, v_cache, block_table + (size_t)row * table_stride, page_size, kv_heads, kvh, n_pages,
+             __ffs(page_size) - 1};
     const int hi_q = qvalid ? pos : -1;
     DecodeTile<ND> regs[TILES];
 #pragma unroll
@@ -358,6 +360,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
     float scale, int window) {
     constexpr int D = ND * 16;
     constexpr int LDK = PF_LD_K(D);
+    const int page_shift = __ffs(page_size) - 1;          // a power of two: divisions by it are shifts
     __shared__ __attribute__((aligned(16))) bf16_t ks[2][PF_KEYS * LDK];
     __shared__ __attribute__((aligned(16))) bf16_t vs[2][D * PF_LD_V];
     // Later tiles of a prompt have more keys to walk. Blocks whose numbers differ by the number
@@ -415,11 +418,11 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
         for (int j = 0; j < K_PER; ++j) {
             const int p = tid + j * 256;
             const int key = min(max(kb + p / (D / 8), blk_lo), blk_last);      // a live key: address always valid
-            int page = table[key / page_size];
+            int page = table[key >> page_shift];
             page = min(max(page, 0), n_pages - 1);
             kr[j] = (p < K_PIECES)
                         ? *reinterpret_cast<const uint4*>(k_cache + (((size_t)page * kv_heads + kvh) * page_size +
-                                                                     (key % page_size)) * D + (p % (D / 8)) * 8)
+                                                                     (key & (page_size - 1))) * D + (p % (D / 8)) * 8)
                         : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
@@ -427,12 +430,12 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
             const int p = tid + j * 256;
             const int d = p / (PF_KEYS / 8), kg = kb + (p % (PF_KEYS / 8)) * 8;   // 8 keys kg .. kg+7, one page
             const int kgc = min(max(kg, blk_lo & ~7), blk_last & ~7);
-            int page = table[kgc / page_size];
+            int page = table[kgc >> page_shift];
             page = min(max(page, 0), n_pages - 1);
             uint4 v = make_uint4(0, 0, 0, 0);
             if (p < V_PIECES)
                 v = *reinterpret_cast<const uint4*>(v_cache + (((size_t)page * kv_heads + kvh) * D + d) * page_size +
-                                                    (kgc % page_size));
+                                                    (kgc & (page_size - 1)));
             // values of keys outside the live range are zero, never stale memory
             if (kg < blk_lo || kg + 7 > blk_last) {
                 uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -483,15 +486,24 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
             // sc[kt][i] = score of key kb + 16 kt + 4 g + i for query lane%16. The running maximum
             // st.m is kept in units of log2(e), so that every weight is one exp2 of a difference.
             float mx = -INFINITY;
+            if (full) {                                   // most tiles: nothing to mask (the same for the whole wave)
 #pragma unroll
-            for (int kt = 0; kt < 4; ++kt)
+                for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int kp = kb + kt * 16 + 4 * g + i;
-                    const bool ok = full || (kp >= lo_q && kp <= hi_q);
-                    sc[kt][i] = ok ? sc[kt][i] * scale_log2 : -INFINITY;
-                    mx = fmaxf(mx, sc[kt][i]);
-                }
+                    for (int i = 0; i < 4; ++i) {
+                        sc[kt][i] *= scale_log2;
+                        mx = fmaxf(mx, sc[kt][i]);
+                    }
+            } else {
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int kp = kb + kt * 16 + 4 * g + i;
+                        sc[kt][i] = (kp >= lo_q && kp <= hi_q) ? sc[kt][i] * scale_log2 : -INFINITY;
+                        mx = fmaxf(mx, sc[kt][i]);
+                    }
+            }
             mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
             mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
             const float m_new = fmaxf(st.m, mx);
