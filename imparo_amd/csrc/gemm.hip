@@ -575,10 +575,33 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, const float* bias, T
         k_gemm_bf16_skinny<TOut, MT, 8><<<grid, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
 }
 
+// Which kernel takes a product of up to 64 rows: 0 for the K-split kernel, else the waves per
+// block of the shared-activation kernel. Measured with cold weights (they never stay in cache
+// between decode steps): from about 12k weight rows on the shared-activation kernel wins at
+// any number of rows; below that it wins when every wave would fetch its own copy of more
+// than 16 activation rows, or when K is long.
+static int stream_waves(int m, int n, int k) {
+    if (n >= 12288) return 4;
+    if (m > 16 || k >= 4096) return 2;
+    return 0;
+}
+
+// A slice's length is rounded up to the kernel's step along K; with a ragged K that can leave the
+// last slices empty. The consumer adds every slice it was promised: fewer slices then, all of
+// them non-empty.
+static int whole_slices(int slices, int k, int step) {
+    while (slices > 1) {
+        const int k_per = ((k + slices - 1) / slices + step - 1) / step * step;
+        if ((k + k_per - 1) / k_per == slices) break;
+        slices /= 2;
+    }
+    return slices;
+}
+
 // Into how many slices of K a product may be cut when its consumer adds the slices. A weight
 // with few rows gives too few blocks to keep the memory system busy otherwise (one CU draws
 // about 50 GB/s at best, so it takes all of them): the measured optimum, with cold weights,
-// is about 256 blocks.
+// is about 256 blocks, with at least 512 of K per slice and at most 8 slices.
 extern "C" int imparo_gemm_slices(int m, int n, int k, int dtype) {
     if (dtype != IMPARO_BF16) return 1;
     if (m > 64) {
@@ -587,14 +610,14 @@ extern "C" int imparo_gemm_slices(int m, int n, int k, int dtype) {
         const long long tiles = (long long)((m + BG_BM - 1) / BG_BM) * ((n + BG_BN - 1) / BG_BN);
         int slices = 1;
         while (slices < 4 && tiles * slices * 2 <= 512 && k / (slices * 2) >= 1024) slices *= 2;
-        return slices;
+        return whole_slices(slices, k, BG_BK);
     }
-    if (n > 4096) return 1;
-    if (m <= 16) {            // one block per 16 weight rows
-        if (k >= 4096) return (k + 2047) / 2048;
-        return k >= 2048 ? 2 : 1;
-    }
-    return k >= 2048 ? 4 : (k >= 1024 ? 2 : 1);   // one block per 32 weight rows
+    const int nw = stream_waves(m, n, k);
+    const int rows_per_block = nw ? nw * 16 : 16;
+    const int blocks = (n + rows_per_block - 1) / rows_per_block;
+    int slices = 1;
+    while (slices < 8 && blocks * slices * 2 <= 256 && k / (slices * 2) >= 512) slices *= 2;
+    return whole_slices(slices, k, 128);
 }
 
 // ------------------------------------------------------------------ bfloat16, some rows (17..64)
@@ -749,17 +772,6 @@ __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
         for (int i = 0; i < 4; ++i)
             if (nq + i < N) store_f32<TOut>(Y, (size_t)m * N + nq + i, v[i]);
     }
-}
-
-// Which kernel takes a product of up to 64 rows: 0 for the K-split kernel, else the waves per
-// block of the shared-activation kernel. Measured with cold weights (they never stay in cache
-// between decode steps): from about 12k weight rows on the shared-activation kernel wins at
-// any number of rows; below that it wins when every wave would fetch its own copy of more
-// than 16 activation rows, or when K is long.
-static int stream_waves(int m, int n, int k) {
-    if (n >= 12288) return 4;
-    if (m > 16 || k >= 4096) return 2;
-    return 0;
 }
 
 template <typename TOut, int MT>

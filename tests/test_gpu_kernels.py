@@ -83,8 +83,11 @@ def test_gemm_in_slices_of_k_and_the_norm_that_adds_them(m):
     n, k = 200, 4096 + 264
     x, w, b = rnd(m, k, seed=1).to(torch.bfloat16), rnd(n, k, seed=2, scale=0.1).to(torch.bfloat16), rnd(n, seed=3)
     slices = ops().gemm_slices(m, n, k, torch.bfloat16)
-    # up to 16 rows: one slice per 2048 of K; 17..64 rows: four
-    assert slices == (3 if m <= 16 else 4) and ops().gemm_slices(m, n, 2048, torch.bfloat16) == (2 if m <= 16 else 4)
+    # few weight rows: as many slices as it takes towards 256 blocks, at least 512 of K each, at most 8;
+    # 8 slices of this ragged K, rounded up to chunks of 128, would leave the eighth empty: 4 then
+    assert slices == 4 and ops().gemm_slices(m, n, 2048, torch.bfloat16) == 4
+    assert ops().gemm_slices(m, 1024, 4608, torch.bfloat16) == 8
+    assert ops().gemm_slices(m, 2048, 2048, torch.bfloat16) == (2 if m <= 16 else 4)    # 128 or 64 blocks
     assert ops().gemm_slices(m, 8192, k, torch.bfloat16) == 1       # a weight with many rows fills the chip by itself
     assert ops().gemm_slices(m, n, k, torch.float32) == 1
     # many rows and few tiles: the 128x128 kernel takes slices too (at least 1024 of K each, at most 4)
