@@ -6,7 +6,7 @@ from __future__ import annotations
 import ctypes
 import os
 import threading
-from ctypes import POINTER, c_int, c_int32, c_int64, c_uint64, c_void_p
+from ctypes import POINTER, c_float, c_int, c_int32, c_int64, c_uint64, c_void_p
 
 from ..csrc import build as _build
 
@@ -39,6 +39,13 @@ _SIGNATURES = {
     "imparo_sched_drop_waiting_head": ([P, P], I), "imparo_sched_retract": ([P, c_int64], I),
     "imparo_sched_n_waiting": ([P], I), "imparo_sched_n_running": ([P], I),
     "imparo_sched_waiting": ([P, P, I], I), "imparo_sched_running": ([P, P, I], I),
+    # plain float32 statements of the kernels, for tests (imparo_amd/kernels/reference.py)
+    "imparo_ref_embed": ([P, P, P, I, I], None), "imparo_ref_rms_norm": ([P, P, c_float, P, I, I], None),
+    "imparo_ref_gemm": ([P, P, P, P, I, I, I], None), "imparo_ref_swiglu": ([P, P, P, c_int64], None),
+    "imparo_ref_head_norm_rope": ([P, P, c_float, P, P, I, P, I, I, I], None),
+    "imparo_ref_attention": ([P, P, P, P, P, I, I, I, I, c_float, I], None),
+    "imparo_ref_short_conv": ([P, P, P, P, P, I, I, I], None),
+    "imparo_ref_argmax": ([P, P, I, I], None), "imparo_ref_sample": ([P, P, P, P, I, I], None),
 }
 EV_ADMIT, EV_WAIT, EV_PREEMPT, EV_FAIL = 1, 2, 3, 4
 
@@ -58,8 +65,17 @@ def host_library() -> ctypes.CDLL:
         if not os.path.isfile(path):
             path = _build.build_host(verbose=True)
         lib = ctypes.CDLL(path)
+        if not all(hasattr(lib, name) for name in _SIGNATURES):
+            # a library from an older build: the host runtime needs no GPU and builds in seconds
+            import _ctypes
+            _ctypes.dlclose(lib._handle)
+            lib = ctypes.CDLL(_build.build_host(verbose=True))
         for name, (argtypes, restype) in _SIGNATURES.items():
-            fn = getattr(lib, name)
+            try:
+                fn = getattr(lib, name)
+            except AttributeError:
+                raise RuntimeError(f"{path} lacks the entry point {name}; rebuild it "
+                                   f"(python -m imparo_amd.csrc.build)") from None
             fn.argtypes = argtypes
             fn.restype = restype
         _lib = lib

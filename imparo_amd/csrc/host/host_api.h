@@ -128,6 +128,22 @@ int imparo_sched_n_running(const ImparoSched* s);
 int imparo_sched_waiting(const ImparoSched* s, int64_t* out, int capacity);
 int imparo_sched_running(const ImparoSched* s, int64_t* out, int capacity);
 
+// ---- plain float32 statements of what the GPU kernels compute (reference_ops.cpp), for tests.
+// Arrays are dense and row-major; nothing here is used by the engine.
+void imparo_ref_embed(const float* table, const int32_t* ids, float* x, int n_tokens, int width);
+void imparo_ref_rms_norm(const float* x, const float* w, float eps, float* y, int rows, int width);
+void imparo_ref_gemm(const float* x, const float* w, const float* bias, float* y, int m, int n, int k);
+void imparo_ref_swiglu(const float* gate, const float* up, float* out, int64_t count);
+void imparo_ref_head_norm_rope(const float* x, const float* w, float eps, const int32_t* positions,
+                               const float* inv_freq, int n_freq, float* y, int n_tokens, int heads, int head_dim);
+void imparo_ref_attention(const float* q, const float* k, const float* v, const int32_t* q_positions, float* out,
+                          int n_queries, int heads, int kv_heads, int head_dim, float scale, int window);
+void imparo_ref_short_conv(const float* bcx, const float* w, const float* bias, float* state, float* y, int n_tokens,
+                           int width, int taps);
+void imparo_ref_argmax(const float* logits, int32_t* out, int rows, int vocab);
+void imparo_ref_sample(const float* logits, const float* temperature, const float* uniform, int32_t* out, int rows,
+                       int vocab);
+
 #ifdef __cplusplus
 }
 #endif

@@ -244,7 +244,7 @@ def test_qk_norm_rope_store(H, Hk, D, rot, page_size, vt):
 
 # ---------------------------------------------------------------- attention
 def _attention_case(H, Hk, D, page_size, window, dtype, sharpen=None, seed=0, kernel="wave", v_transposed=None,
-                    ctx_lens=(70, 1, 200, 33), q_lens=(5, 1, 1, 33)):
+                    ctx_lens=(70, 1, 200, 33), q_lens=(5, 1, 1, 33), attend=P.attend):
     """Rows at different depths of their contexts; the cache is filled by hand
     from whole-sequence k, v; the reference attends over the whole sequences."""
     # the last q_len positions of each context are queried
@@ -279,7 +279,7 @@ def _attention_case(H, Hk, D, page_size, window, dtype, sharpen=None, seed=0, ke
                 v_cache[page, :, :, p % page_size] = v[p].to(dtype).to(DEV)
             else:
                 v_cache[page, :, p % page_size] = v[p].to(dtype).to(DEV)
-        ref = P.attend(q, k, v, range(c), 1.0 / math.sqrt(D), window)
+        ref = torch.as_tensor(attend(q, k, v, range(c), 1.0 / math.sqrt(D), window))
         qs.append(q[c - ql:])
         refs.append(ref[c - ql:])
     q_all = torch.cat(qs).to(dtype).to(DEV)
