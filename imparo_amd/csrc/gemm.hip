@@ -22,6 +22,11 @@ union Frag8 {
 #define EPI_SWIGLU 1   // weight rows interleaved gate, up, gate, up...: out[m, j] = silu(y[m, 2j]) * y[m, 2j+1]
 
 __device__ __forceinline__ float silu_mul_f(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+// The same with the hardware's exp2 and reciprocal (an ulp each) for the bfloat16 kernels: the exact
+// division and exponential cost some thirty instructions per output, ten microseconds per 256x256 tile
+__device__ __forceinline__ float silu_mul_fast(float g, float u) {
+    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504f * g)) * u;
+}
 
 __device__ __forceinline__ uint4 zero_if(bool out, uint4 v) {
     return make_uint4(out ? 0u : v.x, out ? 0u : v.y, out ? 0u : v.z, out ? 0u : v.w);
@@ -271,7 +276,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_bf16_tile(const bf16_t* __restr
                     const float other = __shfl_xor(mine, 1, WAVE);
                     const int m = m0 + wm * 64 + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
                     if (!(lane & 1) && n + 1 < N && m < M)
-                        store_f32<TOut>(Y, (size_t)m * (N / 2) + n / 2, silu_mul_f(mine, other));
+                        store_f32<TOut>(Y, (size_t)m * (N / 2) + n / 2, silu_mul_fast(mine, other));
                 }
                 continue;
             }
@@ -292,9 +297,9 @@ __global__ __launch_bounds__(256, 2) void k_gemm_bf16_tile(const bf16_t* __restr
 // reads three fragments per four products) reaches 830-900. Counters say the matrix pipes are
 // busy a third of the time and LDS a quarter: what is exposed is the wait for fragments, with
 // two waves per SIMD to hide it. One block per CU (its LDS holds two K-steps of both operands),
-// global loads two K-steps ahead in registers. (Four waves of 128x128 each would halve the reads
-// per product again; the compiler spills that variant's 256 accumulator registers inside the
-// loop and it runs five times slower, so it is not built.)
+// global loads two K-steps ahead in registers. (Four waves of 128x128 each halve the reads per
+// product again, but only fit the register file when the operands bypass it: the kernel after
+// this one, which takes K in multiples of 128; this one takes the rest.)
 template <typename TOut, int WM, int WN, int TM, int TN>
 __global__ __launch_bounds__(WM * WN * 64) void k_gemm_bf16_big(const bf16_t* __restrict__ X,
                                                                 const bf16_t* __restrict__ W,
@@ -418,7 +423,7 @@ __global__ __launch_bounds__(WM * WN * 64) void k_gemm_bf16_big(const bf16_t* __
                     const float other = __shfl_xor(mine, 1, WAVE);
                     const int m = m0 + (wm * TM + i) * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
                     if (!(lane & 1) && n + 1 < N && m < M)
-                        store_f32<TOut>(Y, (size_t)m * (N / 2) + n / 2, silu_mul_f(mine, other));
+                        store_f32<TOut>(Y, (size_t)m * (N / 2) + n / 2, silu_mul_fast(mine, other));
                 }
                 continue;
             }
@@ -448,6 +453,218 @@ static int launch_big(const bf16_t* x, const bf16_t* w, const float* bias, TOut*
     const unsigned blocks = (unsigned)(((total + N_XCD - 1) / N_XCD) * N_XCD);
     k_gemm_bf16_big<TOut, WM, WN, TM, TN><<<blocks, WM * WN * 64, lds_bytes, s>>>(x, w, bias, y, m, n, k, tiles_m,
                                                                                  tiles_n, epilogue);
+    return launch_status();
+}
+
+// ------------------------------------------------------------------ bfloat16, many rows, loads straight into LDS
+// A 256x256 tile on four waves, one per SIMD, each with 128x128 of it (4x4 MFMA tiles of
+// 32x32, 256 accumulator registers): two fragments read from LDS per four products, half of
+// what the eight-wave kernel above reads. That only fits the register file because the
+// operands never pass through registers on their way in: global_load_lds writes 16 bytes per
+// lane straight into LDS, a wave's 64 lanes to 1 KB in a row. LDS rows are the 128 bytes of
+// a K-step without padding, so the eight 16-byte pieces of row r are stored in the order
+// piece ^ swz(r), swz(r) = (r & 7) ^ ((r >> 3) & 1): the loading lane picks its global piece
+// accordingly, and the 16 rows that a quarter of a wave reads for one fragment fall on
+// distinct banks. Two stages of 64 KB are two separate arrays: the compiler can then tell
+// that reads of one stage need not wait for loads in flight to the other. A wave keeps the
+// fragments of the next K-sub-step in flight while it multiplies (two register sets), and the
+// barrier of a K-step sits before the last sub-step's products, so the matrix pipe has
+// work queued while the waves meet. Needs K a multiple of 128 (two K-steps).
+#define DM_T 256       // tile rows of each operand
+#define DM_BK 64
+
+// Two (`pair`) or four outputs of one row in one store; the address is aligned to the store
+template <typename T> __device__ __forceinline__ void store_vector(T* dst, const float (&o)[4], bool pair);
+template <> __device__ __forceinline__ void store_vector<float>(float* dst, const float (&o)[4], bool pair) {
+    if (pair)
+        *reinterpret_cast<float2*>(dst) = make_float2(o[0], o[1]);
+    else
+        *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+}
+template <> __device__ __forceinline__ void store_vector<bf16_t>(bf16_t* dst, const float (&o)[4], bool pair) {
+    const unsigned lo = f32x2_to_bf16x2(o[0], o[1]);
+    if (pair)
+        *reinterpret_cast<unsigned*>(dst) = lo;
+    else
+        *reinterpret_cast<uint2*>(dst) = make_uint2(lo, f32x2_to_bf16x2(o[2], o[3]));
+}
+
+__device__ __forceinline__ void load_to_lds(const bf16_t* src, bf16_t* dst_wave_uniform) {
+    __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
+                                     (void __attribute__((address_space(3)))*)dst_wave_uniform, 16, 0, 0);
+}
+
+template <typename TOut>
+__global__ __launch_bounds__(256) void k_gemm_bf16_dma(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+                                                       const float* __restrict__ bias, TOut* __restrict__ Y,
+                                                       int M, int N, int K, int tiles_m, int tiles_n, int epilogue) {
+    __shared__ __attribute__((aligned(1024))) bf16_t stage0[2 * DM_T * DM_BK];   // X rows, then W rows
+    __shared__ __attribute__((aligned(1024))) bf16_t stage1[2 * DM_T * DM_BK];
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + N_XCD - 1) / N_XCD;
+    const int logical = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;
+    if (logical >= total) return;
+    const int per_group = BG_GROUP_M * tiles_n;
+    const int first_m = (logical / per_group) * BG_GROUP_M;
+    const int gsize = min(tiles_m - first_m, BG_GROUP_M);
+    const int tile_m = first_m + (logical % per_group) % gsize;
+    const int tile_n = (logical % per_group) / gsize;
+    const int m0 = tile_m * DM_T, n0 = tile_n * DM_T;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    // loading: instruction j of a wave fills rows j*32 + wave*8 .. +7; lane -> row lane/8, slot lane%8
+    const int load_row = wave * 8 + (lane >> 3);
+    const int load_piece = (lane & 7) ^ (lane >> 3) ^ (wave & 1);          // lane%8 ^ swz(row)
+    unsigned off_x[8], off_w[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        off_x[j] = (unsigned)min(m0 + j * 32 + load_row, M - 1) * (unsigned)K + load_piece * 8;
+        off_w[j] = (unsigned)min(n0 + j * 32 + load_row, N - 1) * (unsigned)K + load_piece * 8;
+    }
+    auto load_step = [&](bf16_t* stage, int kt) __attribute__((always_inline)) {
+        const bf16_t* xk = X + (size_t)kt * DM_BK;
+        const bf16_t* wk = W + (size_t)kt * DM_BK;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) load_to_lds(xk + off_x[j], stage + (j * 32 + wave * 8) * DM_BK);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) load_to_lds(wk + off_w[j], stage + (DM_T + j * 32 + wave * 8) * DM_BK);
+    };
+    // fragments: lane holds row lane%32, K-half lane/32 of a 32x16 piece; sub-step ks is pieces 2ks, 2ks+1
+    const int frag_row = lane & 31;
+    const int swz = (frag_row & 7) ^ ((frag_row >> 3) & 1);
+    const int a_base = (wm * 128 + frag_row) * DM_BK + (((lane >> 5) ^ swz) << 3);
+    const int b_base = (DM_T + wn * 128 + frag_row) * DM_BK + (((lane >> 5) ^ swz) << 3);
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    auto read = [&](const bf16_t* stage, int ks, Frag8 (&fa)[4], Frag8 (&fb)[4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            fa[i].u = *reinterpret_cast<const uint4*>(&stage[(a_base ^ (ks << 4)) + i * 32 * DM_BK]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            fb[j].u = *reinterpret_cast<const uint4*>(&stage[(b_base ^ (ks << 4)) + j * 32 * DM_BK]);
+    };
+    auto multiply = [&](const Frag8 (&fa)[4], const Frag8 (&fb)[4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i].v, fb[j].v, acc[i][j], 0, 0, 0);
+    };
+    const int nk = K / DM_BK;
+    Frag8 fa0[4], fb0[4], fa1[4], fb1[4];
+    // K-step kt from `cur`: on entry set 0 holds its first sub-step and the loads of step kt+1
+    // into `next` are in flight; on exit set 0 holds the first sub-step of kt+1 and the loads
+    // of kt+2 into `cur` are in flight
+    auto k_step = [&](bf16_t* cur, bf16_t* next, int kt) __attribute__((always_inline)) {
+        // (the scheduling barriers keep each sub-step's reads and products where they are written:
+        // left alone, the compiler sinks the loads of the next step to just before the wait for them)
+        read(cur, 1, fa1, fb1);
+        multiply(fa0, fb0);
+        __builtin_amdgcn_sched_barrier(0);
+        read(cur, 2, fa0, fb0);
+        multiply(fa1, fb1);
+        __builtin_amdgcn_sched_barrier(0);
+        read(cur, 3, fa1, fb1);
+        multiply(fa0, fb0);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();               // this wave's part of `next` has landed and `cur` is read; so for every wave
+        read(next, 0, fa0, fb0);
+        load_step(cur, min(kt + 2, nk - 1));      // past the end: the last step again, into a stage nobody reads any more
+        multiply(fa1, fb1);
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {            // one product, one load, (one fragment read)
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (q < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    load_step(stage0, 0);
+    __syncthreads();
+    load_step(stage1, 1);
+    read(stage0, 0, fa0, fb0);
+    for (int kt = 0; kt < nk; kt += 2) {               // an even number of K-steps: one loop, one way round it
+        k_step(stage0, stage1, kt);
+        k_step(stage1, stage0, kt + 1);
+    }
+    // The tile leaves through LDS, a wave's 32 rows x 128 columns at a time (one row of its MFMA
+    // tiles): the wave writes the accumulators as the matrix pipe left them, reads whole rows
+    // back, four columns per lane, and stores 16 (or 8, or 4) bytes per lane, half a wave to a row.
+    // That keeps the 256 accumulators out of the vector registers (where the compiler would
+    // otherwise gather them all at once, spilling what the K loop needs) and gives row-long
+    // stores. A staged row is 136 floats: the two rows a store instruction touches, 4 apart,
+    // fall on disjoint banks. Each wave has a region of its own, so no barrier between passes.
+    __syncthreads();                                   // every wave is done with the operands in LDS
+    constexpr int EP_LD = 136;
+    float* staged = reinterpret_cast<float*>((wave & 2) ? stage1 : stage0) + (wave & 1) * (32 * EP_LD);
+    const int out_col = (lane & 31) * 4;               // of the wave's 128 columns
+    const int n = n0 + wn * 128 + out_col;
+    float bn[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            if (n + c < N) bn[c] = bias[n + c];
+    }
+    const bool swiglu = epilogue == EPI_SWIGLU;
+    const int out_n = swiglu ? N / 2 : N;              // columns of Y
+    const int per_lane = swiglu ? 2 : 4;               // outputs a lane holds of a row
+    // whole vectors: every row of this tile inside, the lane's columns inside, rows of Y aligned
+    const bool vectors = m0 + DM_T <= M && n0 + DM_T <= N && out_n % per_lane == 0 &&
+                         ((uintptr_t)Y % (per_lane * sizeof(TOut))) == 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                staged[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * EP_LD + j * 32 + (lane & 31)] = acc[i][j][r];
+#pragma unroll 2
+        for (int it = 0; it < 16; ++it) {
+            const int row = it * 2 + (lane >> 5);
+            const float4 v = *reinterpret_cast<const float4*>(&staged[row * EP_LD + out_col]);
+            const int m = m0 + wm * 128 + i * 32 + row;
+            float o[4] = {v.x + bn[0], v.y + bn[1], v.z + bn[2], v.w + bn[3]};
+            if (swiglu) {
+                o[0] = silu_mul_fast(o[0], o[1]);
+                o[1] = silu_mul_fast(o[2], o[3]);
+            }
+            TOut* dst = Y + (size_t)m * out_n + (swiglu ? n / 2 : n);
+            if (vectors) {
+                store_vector<TOut>(dst, o, swiglu);
+            } else if (m < M) {
+                if (swiglu) {
+                    if (n + 1 < N) store_f32<TOut>(dst, 0, o[0]);
+                    if (n + 3 < N) store_f32<TOut>(dst, 1, o[1]);
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        if (n + c < N) store_f32<TOut>(dst, c, o[c]);
+                }
+            }
+        }
+    }
+}
+
+static bool dma_tile_takes(int m, int n, int k) {
+    // the operands' offsets are kept in 32 bits
+    return k % (2 * DM_BK) == 0 && (long long)m * k < (1LL << 31) && (long long)n * k < (1LL << 31);
+}
+
+template <typename TOut>
+static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
+                      hipStream_t s) {
+    const int tiles_m = (m + DM_T - 1) / DM_T, tiles_n = (n + DM_T - 1) / DM_T;
+    const long long total = (long long)tiles_m * tiles_n;
+    const unsigned blocks = (unsigned)(((total + N_XCD - 1) / N_XCD) * N_XCD);
+    k_gemm_bf16_dma<TOut><<<blocks, 256, 0, s>>>(x, w, bias, y, m, n, k, tiles_m, tiles_n, epilogue);
     return launch_status();
 }
 
@@ -547,7 +764,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_bf16_skinny(const bf16_t* __re
 #pragma unroll
             for (int i = 0; i < 4; i += 2) {
                 const int n = n0 + g * 4 + i;
-                if (n + 1 < N) store_f32<TOut>(Y, (size_t)m * (N / 2) + n / 2, silu_mul_f(v[i], v[i + 1]));
+                if (n + 1 < N) store_f32<TOut>(Y, (size_t)m * (N / 2) + n / 2, silu_mul_fast(v[i], v[i + 1]));
             }
             continue;
         }
@@ -765,7 +982,7 @@ __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
         if (epilogue == EPI_SWIGLU) {
 #pragma unroll
             for (int i = 0; i < 4; i += 2)
-                if (nq + i + 1 < N) store_f32<TOut>(Y, (size_t)m * (N / 2) + (nq + i) / 2, silu_mul_f(v[i], v[i + 1]));
+                if (nq + i + 1 < N) store_f32<TOut>(Y, (size_t)m * (N / 2) + (nq + i) / 2, silu_mul_fast(v[i], v[i + 1]));
             continue;
         }
 #pragma unroll
@@ -818,11 +1035,16 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
         else
             launch_skinny<TOut, 4>(x, w, bias, y, m, n, k, epilogue, slices, s);
     } else {
-        // `force` 256: the 256x256 tile; 257: 256x128 (for measurements); otherwise by shape
+        // `force` 256: the 256x256 tile on eight waves; 257: 256x128; 258: 256x256 on four waves with loads
+        // straight into LDS (for measurements); otherwise by shape
+        if (slices == 1 && force == 0 && big_tile_pays(m, n, k) && dma_tile_takes(m, n, k))
+            return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, s);
         if (slices == 1 && (force == 256 || (force == 0 && big_tile_pays(m, n, k))))
             return launch_big<TOut, 2, 4, 4, 2>(x, w, bias, y, m, n, k, epilogue, s);
         if (slices == 1 && force == 257)
             return launch_big<TOut, 4, 2, 2, 2>(x, w, bias, y, m, n, k, epilogue, s);
+        if (slices == 1 && force == 258 && dma_tile_takes(m, n, k))
+            return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, s);
         const int tiles_m = (m + BG_BM - 1) / BG_BM, tiles_n = (n + BG_BN - 1) / BG_BN;
         const long long total = (long long)tiles_m * tiles_n;
         if (total > 0x7fffff00LL) return IMPARO_BAD_ARGUMENT;

@@ -140,6 +140,30 @@ def test_gemm_with_many_weight_rows(m, k):
     assert (act.cpu().double() - ref).abs().max() <= 1e-6 * math.sqrt(k) * y.abs().max() * max(1.0, y.abs().max().item())
 
 
+@pytest.mark.parametrize("k", [256, 200, 1152])
+def test_gemm_with_large_tiles(k):
+    """Enough 256x256 tiles (160 or more) for the large-tile kernels: K a multiple of 128 goes to
+    the four-wave kernel that loads straight into LDS, another K to the eight-wave one. Edges in
+    both directions, an odd number of column pairs, a bias, both epilogues and output types."""
+    m, n = 2600, 3900 + 2 * (k % 3)
+    x, w, b = rnd(m, k, seed=1, scale=0.5).to(torch.bfloat16), rnd(n, k, seed=2, scale=0.3).to(torch.bfloat16), rnd(n, seed=3)
+    y = x.float() @ w.float().t() + b                       # float32 on the CPU: products exact, sums to 1e-6 sqrt(k)
+    bound = 1e-6 * math.sqrt(k) * float(y.abs().max())
+    out = torch.full((m, n), float("nan"), device=DEV)
+    ops().gemm(x.to(DEV), w.to(DEV), out, bias=b.to(DEV))
+    assert (out.cpu() - y).abs().max() <= 4 * bound
+    outb = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().gemm(x.to(DEV), w.to(DEV), outb, bias=b.to(DEV))
+    assert torch.equal(outb.cpu(), out.cpu().to(torch.bfloat16))
+    ref = torch.nn.functional.silu(y[:, 0::2].double()) * y[:, 1::2].double()
+    out = torch.full((m, n // 2), float("nan"), device=DEV)
+    ops().gemm(x.to(DEV), w.to(DEV), out, bias=b.to(DEV), swiglu=True)
+    torch.testing.assert_close(out.cpu().double(), ref, rtol=1e-5, atol=8 * bound)
+    outb = torch.full((m, n // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().gemm(x.to(DEV), w.to(DEV), outb, bias=b.to(DEV), swiglu=True)
+    assert torch.equal(outb.cpu(), out.cpu().to(torch.bfloat16))
+
+
 def test_gemm_refuses_what_it_cannot_take():
     from imparo_amd.kernels import KernelArgumentError
     x, w = rnd(4, 12).to(torch.bfloat16).to(DEV), rnd(8, 12).to(torch.bfloat16).to(DEV)
