@@ -164,6 +164,21 @@ def test_gemm_with_large_tiles(k):
     assert torch.equal(outb.cpu(), out.cpu().to(torch.bfloat16))
 
 
+def test_gemm_with_large_tiles_in_slices_of_k():
+    """Few 256x256 tiles and a long K: four slices of K on the large tiles, one block per CU."""
+    m, n, k = 1900, 2000, 8192
+    assert ops().gemm_slices(m, n, k, torch.bfloat16) == 4
+    assert ops().gemm_slices(m, n, 4096, torch.bfloat16) == 2          # shorter K: the 128x128 tiles' rule
+    x, w, b = rnd(m, k, seed=1, scale=0.5).to(torch.bfloat16), rnd(n, k, seed=2, scale=0.3).to(torch.bfloat16), rnd(n, seed=3)
+    y = x.float() @ w.float().t() + b
+    out = torch.full((4, m, n), float("nan"), device=DEV)
+    ops().gemm(x.to(DEV), w.to(DEV), out, bias=b.to(DEV))
+    assert (out.cpu().sum(0) - y).abs().max() <= 4e-6 * math.sqrt(k) * float(y.abs().max())
+    # each slice is its own range of K; the bias rides on the first
+    part = x[:, 2048:4096].float() @ w[:, 2048:4096].float().t()
+    assert (out[1].cpu() - part).abs().max() <= 4e-6 * math.sqrt(2048) * float(part.abs().max())
+
+
 def test_gemm_refuses_what_it_cannot_take():
     from imparo_amd.kernels import KernelArgumentError
     x, w = rnd(4, 12).to(torch.bfloat16).to(DEV), rnd(8, 12).to(torch.bfloat16).to(DEV)
@@ -264,6 +279,54 @@ def test_qk_norm_rope_store(H, Hk, D, rot, page_size, vt):
         untouched = ~written
         assert k_cache.cpu().float().permute(0, 2, 1, 3)[untouched].abs().sum() == 0
         assert v_cache.cpu().float().permute(0, 2, 1, 3)[untouched].abs().sum() == 0
+
+
+@pytest.mark.parametrize("H,Hk,D,rot", [(4, 2, 16, 16), (5, 1, 64, 64), (6, 3, 96, 32), (3, 1, 144, 144), (2, 2, 272, 0)])
+@pytest.mark.parametrize("vt", [False, True])
+def test_qk_norm_rope_store_many_tokens(H, Hk, D, rot, vt):
+    """From 32 tokens on a launch takes the kernel with a block per token. A token's results are the
+    same bits whichever kernel it met (the same tokens again, a few at a time), and right."""
+    segments, page_size, n_pages = [(0, 70), (5, 41)], 16, 12
+    tables = [[3, 1, 7, 9, 11], [0, 2, 4]]
+    for dtype in (torch.float32, torch.bfloat16):
+        qkv = rnd(111, (H + 2 * Hk) * D, seed=D).to(DEV)
+        qw, kw = (1 + 0.1 * rnd(D, seed=1)).to(DEV), (1 + 0.1 * rnd(D, seed=2)).to(DEV)
+        inv = None
+        if rot:
+            i = np.arange(rot // 2, dtype=np.float32)
+            inv = torch.from_numpy(np.power(np.float32(1e6), (np.float32(-2.0) * i / np.float32(rot))).astype(np.float32)).to(DEV)
+        results = []
+        for step in (111, 7):
+            ctx = hand_context(segments, page_size, n_pages, dtype, DEV, kv_sites={0: (Hk, D)}, tables=tables,
+                               v_transposed=vt)
+            k_cache, v_cache, table = ctx.kv(0)
+            q_out = torch.empty(111, H, D, dtype=dtype, device=DEV)
+            for t0 in range(0, 111, step):
+                t1 = min(111, t0 + step)
+                ops().qk_norm_rope_store(qkv[t0:t1], qw, kw, 1e-6, inv, ctx.positions[t0:t1], ctx.row_of_token[t0:t1],
+                                         table, page_size, q_out[t0:t1], k_cache, v_cache, H, Hk, D, v_transposed=vt)
+            results.append((q_out.cpu(), k_cache.cpu().clone(), v_cache.cpu().clone()))
+        for a, b in zip(*results):
+            assert torch.equal(a, b)
+        positions = ctx.positions.cpu().tolist()
+        q = qkv.cpu()[:, :H * D].reshape(111, H, D)
+        q_ref = P.rms_norm(q, qw.cpu(), 1e-6)
+        if rot:
+            q_ref = P.rope_neox(q_ref, positions, 1e6, rot)
+        tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -7)
+        torch.testing.assert_close(results[0][0].float(), q_ref, **tol)
+        k = qkv.cpu()[:, H * D:(H + Hk) * D].reshape(111, Hk, D)
+        k_ref = P.rms_norm(k, kw.cpu(), 1e-6)
+        if rot:
+            k_ref = P.rope_neox(k_ref, positions, 1e6, rot)
+        v = qkv.cpu()[:, (H + Hk) * D:].reshape(111, Hk, D)
+        kc, vc = results[0][1].float(), results[0][2].float()
+        if vt:
+            vc = vc.transpose(2, 3)
+        for t, (pos, r) in enumerate(zip(positions, ctx.row_of_token.cpu().tolist())):
+            page = tables[r][pos // page_size]
+            torch.testing.assert_close(kc[page, :, pos % page_size], k_ref[t], **tol)
+            torch.testing.assert_close(vc[page, :, pos % page_size], v[t], **tol)
 
 
 # ---------------------------------------------------------------- attention
