@@ -277,6 +277,57 @@ __global__ void k_short_conv(const float* __restrict__ bcx, const float* __restr
     store_f32<TOut>(out, (size_t)t * width + ch, c * acc);
 }
 
+__device__ __forceinline__ void store_four(float* dst, float a, float b, float c, float d) {
+    *reinterpret_cast<float4*>(dst) = make_float4(a, b, c, d);
+}
+__device__ __forceinline__ void store_four(bf16_t* dst, float a, float b, float c, float d) {
+    *reinterpret_cast<uint2*>(dst) = make_uint2(f32x2_to_bf16x2(a, b), f32x2_to_bf16x2(c, d));
+}
+
+// The same, four channels to a thread with 16-byte loads (width a multiple of 4, rows 16-byte
+// aligned): a prompt's portion is bound by how many bytes a memory instruction moves. Each
+// channel's taps are summed exactly as above.
+template <typename TOut>
+__global__ void k_short_conv_v4(const float* __restrict__ bcx, const float* __restrict__ weight,
+                                const float* __restrict__ bias, const float* __restrict__ state,
+                                const int32_t* __restrict__ row_of_token, const int32_t* __restrict__ seg_start,
+                                const int32_t* __restrict__ slot, TOut* __restrict__ out,
+                                int n_tokens, int width, int taps) {
+    const int ch = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    const int t = blockIdx.y;
+    if (ch >= width) return;
+    const int r = row_of_token[t];
+    const int local = t - seg_start[r];
+    const int history = taps - 1;
+    const float* st = state + (size_t)slot[r] * history * width;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < taps; ++k) {
+        const int e = local + k;            // index into state ++ values
+        float4 v;
+        if (e < history) {
+            v = *reinterpret_cast<const float4*>(st + (size_t)e * width + ch);
+        } else {
+            const size_t row = (size_t)(t - (history - k)) * 3 * width;
+            const float4 b = *reinterpret_cast<const float4*>(bcx + row + ch);
+            const float4 x = *reinterpret_cast<const float4*>(bcx + row + 2 * width + ch);
+            v = make_float4(b.x * x.x, b.y * x.y, b.z * x.z, b.w * x.w);
+        }
+        acc[0] = fmaf(weight[(size_t)ch * taps + k], v.x, acc[0]);
+        acc[1] = fmaf(weight[(size_t)(ch + 1) * taps + k], v.y, acc[1]);
+        acc[2] = fmaf(weight[(size_t)(ch + 2) * taps + k], v.z, acc[2]);
+        acc[3] = fmaf(weight[(size_t)(ch + 3) * taps + k], v.w, acc[3]);
+    }
+    if (bias) {
+        const float4 bv = *reinterpret_cast<const float4*>(bias + ch);
+        acc[0] += bv.x;
+        acc[1] += bv.y;
+        acc[2] += bv.z;
+        acc[3] += bv.w;
+    }
+    const float4 c = *reinterpret_cast<const float4*>(bcx + (size_t)t * 3 * width + width + ch);
+    store_four(out + (size_t)t * width + ch, c.x * acc[0], c.y * acc[1], c.z * acc[2], c.w * acc[3]);
+}
+
 extern "C" int imparo_short_conv(const float* bcx, const float* weight, const float* bias, const float* state,
                                  const int32_t* row_of_token, const int32_t* seg_start, const int32_t* slot,
                                  void* out, int out_dtype, int n_tokens, int width, int taps, int n_slots,
@@ -286,6 +337,19 @@ extern "C" int imparo_short_conv(const float* bcx, const float* weight, const fl
     if (n_tokens == 0) return IMPARO_OK;
     if (n_tokens > 65535) return IMPARO_BAD_ARGUMENT;
     hipStream_t s = (hipStream_t)stream;
+    if (width % 4 == 0 && n_tokens >= 32 && ((uintptr_t)bcx % 16) == 0 && ((uintptr_t)state % 16) == 0 &&
+        ((uintptr_t)out % 16) == 0 && (!bias || ((uintptr_t)bias % 16) == 0) &&
+        (out_dtype == IMPARO_F32 || out_dtype == IMPARO_BF16)) {
+        const int threads4 = width >= 1024 ? 256 : 64;
+        dim3 grid4((width / 4 + threads4 - 1) / threads4, n_tokens);
+        if (out_dtype == IMPARO_F32)
+            k_short_conv_v4<float><<<grid4, threads4, 0, s>>>(bcx, weight, bias, state, row_of_token, seg_start, slot,
+                                                              (float*)out, n_tokens, width, taps);
+        else
+            k_short_conv_v4<bf16_t><<<grid4, threads4, 0, s>>>(bcx, weight, bias, state, row_of_token, seg_start,
+                                                               slot, (bf16_t*)out, n_tokens, width, taps);
+        return launch_status();
+    }
     const int threads = width >= 256 ? 256 : 64;
     dim3 grid((width + threads - 1) / threads, n_tokens);
     if (out_dtype == IMPARO_F32)

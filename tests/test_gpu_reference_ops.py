@@ -86,15 +86,17 @@ def test_attention_over_pages(H, Hk, D, page_size, window):
 
 
 @pytest.mark.parametrize("width,taps", [(100, 3), (300, 4), (64, 9)])
-def test_short_conv_is_the_statement_bit_for_bit(width, taps):
-    segments, slots = [(0, 1), (0, 9), (0, 2)], [3, 0, 5]
+@pytest.mark.parametrize("segments", [[(0, 1), (0, 9), (0, 2)], [(0, 40), (0, 3), (0, 1)]])
+def test_short_conv_is_the_statement_bit_for_bit(width, taps, segments):
+    """Few tokens take the kernel with a channel per thread, 32 or more the one with four: the same bits."""
+    slots, n_tok = [3, 0, 5], sum(n for _, n in segments)
     w, bias = rnd(width, taps, seed=1, scale=0.3), rnd(width, seed=2, scale=0.1)
     state0 = rnd(8, taps - 1, width, seed=3)
-    bcx = rnd(12, 3 * width, seed=4)
+    bcx = rnd(n_tok, 3 * width, seed=4)
     ctx = hand_context(segments, 16, 16, torch.float32, DEV, fixed_sites={0: (taps - 1, width)}, slots=slots)
     state = ctx.fixed_state(0)
     state.copy_(state0)
-    out = torch.empty(12, width, device=DEV)
+    out = torch.empty(n_tok, width, device=DEV)
     ops().short_conv(bcx.to(DEV), w.to(DEV), bias.to(DEV), state, ctx.row_of_token, ctx.seg_start, ctx.seg_len,
                      ctx.slot, out)
     at = 0
