@@ -42,11 +42,20 @@ class SwiGlu:
         gate, up = tensors[n["gate"] + ".weight"], tensors[n["up"] + ".weight"]
         if gate.dtype != up.dtype:
             gate, up = gate.to(torch.float32), up.to(torch.float32)
+        down = tensors[n["down"] + ".weight"]
+        # The bfloat16 kernels walk K in steps of 8. A hidden width that is no multiple of 8 is
+        # filled up with hidden units whose weights are zero: silu(0) * 0 = 0 goes through zero
+        # columns of the way back, so every sum is the one it was.
+        fill = (-self.hidden) % 8
+        if fill and engine_dtype != torch.float32 and down.dtype != torch.float32:
+            gate = torch.cat([gate, gate.new_zeros(fill, self.width)])
+            up = torch.cat([up, up.new_zeros(fill, self.width)])
+            down = torch.cat([down, down.new_zeros(self.width, fill)], dim=1)
         # gate and up as one projection with alternating rows (g0, u0, g1, u1, ...): the same dot
         # products, one launch, and the GEMM's epilogue applies silu(gate) * up before it stores
-        fused = torch.stack([gate, up], dim=1).reshape(2 * self.hidden, self.width)
+        fused = torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], self.width)
         self.gate_up = Linear(place_matrix(fused, engine_dtype, device))
-        self.down = Linear(place_matrix(tensors[n["down"] + ".weight"], engine_dtype, device))
+        self.down = Linear(place_matrix(down, engine_dtype, device))
 
     @property
     def in_dtype(self) -> torch.dtype:

@@ -82,7 +82,7 @@ def test_plan_is_chosen_layer_by_layer():
     kinds = [l.mixer.kind for l in plan.layers]
     assert kinds == ["attention", "short_conv", "attention", "attention", "short_conv"]
     assert [l.mixer.get("window") for l in plan.layers] == [24, None, None, 24, None]
-    assert all(l.ffn.kind == "swiglu" and l.ffn["hidden"] == 176 for l in plan.layers)
+    assert all(l.ffn.kind == "swiglu" and l.ffn["hidden"] == 172 for l in plan.layers)
     assert [c.layer for c in plan.order] == [0, 1, 2, 3, 4] and all(c.cache_of is None for c in plan.order)
     assert plan.layers[0].mixer["position"]["base"] == 50000.0
     assert plan.layers[0].mixer_norm["eps"] == 1e-4

@@ -27,7 +27,7 @@ TINY_C = dict(
     vocab_size=200, hidden_size=160, num_hidden_layers=5,
     layer_types=["sliding_attention", "conv", "full_attention", "sliding_attention", "conv"],
     num_attention_heads=10, num_key_value_heads=5,
-    block_auto_adjust_ff_dim=False, block_ff_dim=176,
+    block_auto_adjust_ff_dim=False, block_ff_dim=172,
     conv_L_cache=2, conv_bias=False, rope_theta=50000.0, tie_embedding=True,
     norm_eps=1e-4, max_position_embeddings=1024, sliding_window=24,
 )
