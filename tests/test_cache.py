@@ -8,8 +8,8 @@ from imparo_amd.cache import (PagePool, CacheManager, PagedSpec, FixedSpec, OutO
 
 
 def test_lowest_free_page_always():
-    # the reference's sequence (/root/reference/crates/imparo-kv/src/alloc.rs:147-276 as the survey
-    # records it): 0,1,2,3; free 2 and 0; next 0, 2, 4
+    # the reference's sequence (/root/reference/crates/imparo-kv/src/alloc.rs:147-276):
+    # 0,1,2,3; free 2 and 0; next 0, 2, 4
     p = PagePool(8)
     assert [p.alloc() for _ in range(4)] == [0, 1, 2, 3]
     p.free(2)

@@ -62,7 +62,7 @@ def test_rotation_and_head_norm():
 
 
 def test_attention():
-    # /root/reference/crates/imparo-model/src/cpu_support.rs tests as the survey records them:
+    # /root/reference/crates/imparo-model/src/cpu_support.rs:485-512:
     # q = [1,0] twice, k = [[0,1],[1,0]], v = I: row 0 sees only key 0 -> [1,0]; row 1's weights sum to 1
     q = np.array([[[1.0, 0.0]], [[1.0, 0.0]]], dtype=np.float32)
     k = np.array([[[0.0, 1.0]], [[1.0, 0.0]]], dtype=np.float32)
