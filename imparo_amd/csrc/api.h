@@ -108,6 +108,13 @@ int imparo_short_conv_decode(const float* bcx, const float* weight, const float*
                              const int32_t* slot, void* out, int out_dtype, int n_rows, int width, int taps,
                              int n_slots, imparo_stream stream);
 
+// The conv mixer's input projection and imparo_short_conv_decode in one launch, for at most 16
+// single-token rows: x [m, k] and w [3 e, k] bfloat16, in_bias [3 e] or null, conv_w [e, taps],
+// conv_b [e] or null, slot [m] (distinct). out [m, e]; the state is shifted in place.
+int imparo_in_proj_conv_decode(const void* x, const void* w, const float* in_bias, const float* conv_w,
+                               const float* conv_b, float* state, const int32_t* slot, void* out, int out_dtype,
+                               int m, int e, int k, int taps, int n_slots, imparo_stream stream);
+
 // state' = the last taps-1 rows of (state ++ B*x) for every request; runs after
 // imparo_short_conv on the same stream.
 int imparo_short_conv_state(const float* bcx, float* state, const int32_t* seg_start, const int32_t* seg_len,

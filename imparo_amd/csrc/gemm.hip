@@ -802,6 +802,183 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, const float* bias, T
         k_gemm_bf16_skinny<TOut, MT, 8><<<grid, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
 }
 
+// ------------------------------------------------------------------ conv input projection + gated conv, single tokens
+// For a decode step's rows (one token each, at most 16): the projection to [B | C | x] and the
+// gated short convolution that consumes it in one launch. A block takes 8 channels: its first
+// MFMA tile holds the B rows of those channels (tile rows 0..7) and their x rows (8..15), its
+// second the C rows (0..7, and again in 8..15: the same cache lines, nothing more to fetch).
+// K is split over the waves as in the kernel above and the partial sums meet in LDS in wave
+// order; then 32 lanes of wave 0 each own one token and four channels: u = B * x, the taps
+// oldest first exactly as the conv kernels sum them, the C gate, and the shift of the state
+// (a lane owns its channels' history, so nothing races). With HIST > 0 the history, the taps
+// and the biases are asked for before the walk along K, so they are there when it ends.
+template <typename TOut, int NW, int HIST>
+__global__ __launch_bounds__(NW * 64) void k_in_proj_conv_decode(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, const float* __restrict__ in_bias,
+    const float* __restrict__ conv_w, const float* __restrict__ conv_b, float* __restrict__ state,
+    const int32_t* __restrict__ slot, TOut* __restrict__ out, int M, int E, int K, int taps) {
+    __shared__ float red[NW][2][64][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int c0 = blockIdx.x * 8;
+    const bf16_t* wrow0 = W + (size_t)(r16 < 8 ? c0 + r16 : 2 * E + c0 + (r16 - 8)) * K + g * 8;
+    const bf16_t* wrow1 = W + (size_t)(E + c0 + (r16 & 7)) * K + g * 8;
+    const bf16_t* xrow = X + (size_t)min(r16, M - 1) * K + g * 8;
+    const int history = HIST > 0 ? HIST : taps - 1;
+    // the lanes that finish the block: token r16, channels cb .. cb+3
+    const bool finisher = wave == 0 && g < 2 && r16 < M;
+    const int cb = c0 + 4 * (g & 1);
+    float* st = state + (size_t)(finisher ? slot[r16] : 0) * history * E;
+    constexpr int HN = HIST > 0 ? HIST : 1;
+    float hist[HN][4], tap[HN + 1][4], bias_b[4], bias_c[4], bias_x[4], bias_conv[4];
+    if (HIST > 0 && finisher) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int k = 0; k < HIST; ++k) hist[k][i] = st[(size_t)k * E + cb + i];
+#pragma unroll
+            for (int k = 0; k <= HIST; ++k) tap[k][i] = conv_w[(size_t)(cb + i) * (HIST + 1) + k];
+            bias_b[i] = in_bias ? in_bias[cb + i] : 0.f;
+            bias_c[i] = in_bias ? in_bias[E + cb + i] : 0.f;
+            bias_x[i] = in_bias ? in_bias[2 * E + cb + i] : 0.f;
+            bias_conv[i] = conv_b ? conv_b[cb + i] : 0.f;
+        }
+    }
+    struct Frags {
+        Frag8 w0[4], w1[4], x[4];
+    };
+    f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+    auto load = [&](int k0, Frags& f) {
+#pragma unroll
+        for (int s2 = 0; s2 < 4; ++s2) {
+            const int k = k0 + s2 * 32;
+            const bool in = k + g * 8 < K;
+            f.w0[s2].u = in ? *reinterpret_cast<const uint4*>(wrow0 + k) : make_uint4(0, 0, 0, 0);
+            f.w1[s2].u = in ? *reinterpret_cast<const uint4*>(wrow1 + k) : make_uint4(0, 0, 0, 0);
+            f.x[s2].u = in ? *reinterpret_cast<const uint4*>(xrow + k) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto multiply = [&](const Frags& f) {
+#pragma unroll
+        for (int s2 = 0; s2 < 4; ++s2) {
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.w0[s2].v, f.x[s2].v, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.w1[s2].v, f.x[s2].v, acc1, 0, 0, 0);
+        }
+    };
+    Frags cur, nxt;
+    int k0 = wave * 128;
+    if (k0 < K) load(k0, cur);
+    while (k0 < K) {
+        const int k1 = k0 + NW * 128;
+        if (k1 < K) load(k1, nxt);
+        multiply(cur);
+        cur = nxt;
+        k0 = k1;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        red[wave][0][lane][i] = acc0[i];
+        red[wave][1][lane][i] = acc1[i];
+    }
+    __syncthreads();
+    if (!finisher) return;
+    // D layout: lane holds column lane%16 (a token), tile rows 4*(lane/16) + i: B and C of channel
+    // cb + i sit in this lane's entries, x of the same channel 8 tile rows further: lane + 32
+    float b[4], c[4], x[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        b[i] = red[0][0][lane][i];
+        x[i] = red[0][0][lane + 32][i];
+        c[i] = red[0][1][lane][i];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) {
+            b[i] += red[w][0][lane][i];
+            x[i] += red[w][0][lane + 32][i];
+            c[i] += red[w][1][lane][i];
+        }
+    }
+    float y[4];
+    if (HIST > 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float u = (b[i] + bias_b[i]) * (x[i] + bias_x[i]);
+            float a = 0.f;
+#pragma unroll
+            for (int k = 0; k < HIST; ++k) {
+                a = fmaf(tap[k][i], hist[k][i], a);
+                st[(size_t)k * E + cb + i] = k + 1 < HIST ? hist[k + 1][i] : u;
+            }
+            a = fmaf(tap[HIST][i], u, a);
+            a += bias_conv[i];
+            y[i] = (c[i] + bias_c[i]) * a;
+        }
+    } else {
+        for (int i = 0; i < 4; ++i) {
+            const int ch = cb + i;
+            const float bv = b[i] + (in_bias ? in_bias[ch] : 0.f);
+            const float cv = c[i] + (in_bias ? in_bias[E + ch] : 0.f);
+            const float xv = x[i] + (in_bias ? in_bias[2 * E + ch] : 0.f);
+            const float u = bv * xv;
+            float a = 0.f;
+            float prev = st[ch];                                  // oldest
+            for (int k = 0; k < history; ++k) {
+                a = fmaf(conv_w[(size_t)ch * taps + k], prev, a);
+                const float next = (k + 1 < history) ? st[(size_t)(k + 1) * E + ch] : u;
+                st[(size_t)k * E + ch] = next;
+                prev = next;
+            }
+            a = fmaf(conv_w[(size_t)ch * taps + history], u, a);
+            a += conv_b ? conv_b[ch] : 0.f;
+            y[i] = cv * a;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) store_f32<TOut>(out, (size_t)r16 * E + cb + i, y[i]);
+}
+
+template <typename TOut, int NW>
+static void launch_in_proj_conv(const bf16_t* x, const bf16_t* w, const float* in_bias, const float* conv_w,
+                                const float* conv_b, float* state, const int32_t* slot, TOut* out, int m, int e, int k,
+                                int taps, hipStream_t s) {
+    const unsigned blocks = (unsigned)(e / 8);
+    switch (taps - 1) {
+        case 1: k_in_proj_conv_decode<TOut, NW, 1><<<blocks, NW * 64, 0, s>>>(x, w, in_bias, conv_w, conv_b, state, slot, out, m, e, k, taps); break;
+        case 2: k_in_proj_conv_decode<TOut, NW, 2><<<blocks, NW * 64, 0, s>>>(x, w, in_bias, conv_w, conv_b, state, slot, out, m, e, k, taps); break;
+        case 3: k_in_proj_conv_decode<TOut, NW, 3><<<blocks, NW * 64, 0, s>>>(x, w, in_bias, conv_w, conv_b, state, slot, out, m, e, k, taps); break;
+        default: k_in_proj_conv_decode<TOut, NW, 0><<<blocks, NW * 64, 0, s>>>(x, w, in_bias, conv_w, conv_b, state, slot, out, m, e, k, taps);
+    }
+}
+
+// x [m, k] bfloat16 (m <= 16 single tokens), w [3 e, k] bfloat16, conv_w [e, taps], state
+// [n_slots, taps-1, e], slot [m] (distinct): out [m, e] = the gated conv's output, state shifted.
+extern "C" int imparo_in_proj_conv_decode(const void* x, const void* w, const float* in_bias, const float* conv_w,
+                                          const float* conv_b, float* state, const int32_t* slot, void* out,
+                                          int out_dtype, int m, int e, int k, int taps, int n_slots,
+                                          imparo_stream stream) {
+    if (!x || !w || !conv_w || !state || !slot || !out) return IMPARO_BAD_ARGUMENT;
+    if (m < 0 || m > 16 || e <= 0 || e % 8 != 0 || k <= 0 || k % 8 != 0 || taps < 2 || taps > 64 || n_slots <= 0)
+        return IMPARO_BAD_ARGUMENT;
+    if (((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return IMPARO_BAD_ARGUMENT;
+    if (out_dtype != IMPARO_F32 && out_dtype != IMPARO_BF16) return IMPARO_BAD_ARGUMENT;
+    if (m == 0) return IMPARO_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const bf16_t* xb = (const bf16_t*)x;
+    const bf16_t* wb = (const bf16_t*)w;
+    // waves over K as the K-split kernel has them: chunks of 128, few per wave
+    if (out_dtype == IMPARO_F32) {
+        if (k <= 512)
+            launch_in_proj_conv<float, 4>(xb, wb, in_bias, conv_w, conv_b, state, slot, (float*)out, m, e, k, taps, s);
+        else
+            launch_in_proj_conv<float, 8>(xb, wb, in_bias, conv_w, conv_b, state, slot, (float*)out, m, e, k, taps, s);
+    } else {
+        if (k <= 512)
+            launch_in_proj_conv<bf16_t, 4>(xb, wb, in_bias, conv_w, conv_b, state, slot, (bf16_t*)out, m, e, k, taps, s);
+        else
+            launch_in_proj_conv<bf16_t, 8>(xb, wb, in_bias, conv_w, conv_b, state, slot, (bf16_t*)out, m, e, k, taps, s);
+    }
+    return launch_status();
+}
+
 // Which kernel takes a product of up to 64 rows: 0 for the K-split kernel, else the waves per
 // block of the shared-activation kernel. Measured with cold weights (they never stay in cache
 // between decode steps): from about 12k weight rows on the shared-activation kernel wins at

@@ -29,6 +29,7 @@ _SIGNATURES = {
     "imparo_gemm": [P, P, P, P, I, I, I, I, I, I, I, P],
     "imparo_gemm_slices": [I, I, I, I],
     "imparo_short_conv_decode": [P, P, P, P, P, P, I, I, I, I, I, P],
+    "imparo_in_proj_conv_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
     "imparo_qk_norm_rope_store": [P, P, P, F, P, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, P],
     "imparo_attention": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
     "imparo_attention_decode": [P, P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],

@@ -308,6 +308,36 @@ def short_conv(bcx: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     return out
 
 
+def in_proj_conv_decode_supported(x_rows: int, weight: torch.Tensor) -> bool:
+    """The fused launch takes a bfloat16 projection and at most 16 rows."""
+    return weight.dtype == torch.bfloat16 and 0 < x_rows <= 16 and weight.shape[0] % 24 == 0 and weight.shape[1] % 8 == 0
+
+
+def in_proj_conv_decode(x: torch.Tensor, in_weight: torch.Tensor, in_bias: Optional[torch.Tensor],
+                        conv_weight: torch.Tensor, conv_bias: Optional[torch.Tensor], state: torch.Tensor,
+                        slot: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """For rows of one token each: [B | C | x] = x . in_weight^T (+ bias), then the gated short
+    convolution against each row's state, which is shifted; one launch."""
+    m, k = x.shape
+    three_e, kw = in_weight.shape
+    width, taps = conv_weight.shape
+    if three_e != 3 * width or kw != k:
+        raise KernelArgumentError(f"in_proj_conv_decode: a [{three_e}, {kw}] projection does not feed a conv of "
+                                  f"width {width} from rows of {k}")
+    if not in_proj_conv_decode_supported(m, in_weight) or x.dtype != torch.bfloat16:
+        raise KernelArgumentError("in_proj_conv_decode: takes 1 to 16 bfloat16 rows and a bfloat16 projection whose "
+                                  "width is a multiple of 8")
+    n_slots = state.shape[0]
+    _check(library().imparo_in_proj_conv_decode(
+        _dev(x, "x", torch.bfloat16), _dev(in_weight, "in_proj weight", torch.bfloat16),
+        _dev(in_bias, "in_proj bias", torch.float32, (three_e,)), _dev(conv_weight, "conv weight", torch.float32),
+        _dev(conv_bias, "conv bias", torch.float32, (width,)),
+        _dev(state, "conv state", torch.float32, (n_slots, taps - 1, width)),
+        _dev(slot, "slot", torch.int32, (m,)), _dev(out, "conv out", None, (m, width)), _code(out, "conv out"),
+        m, width, k, taps, n_slots, _stream()), "in_proj_conv_decode")
+    return out
+
+
 def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     n, vocab = logits.shape
     _check(library().imparo_argmax_rows(_dev(logits, "logits", torch.float32), _dev(out, "picks", torch.int32, (n,)),

@@ -508,6 +508,48 @@ def test_short_conv_exact_vectors_from_the_reference():
     assert out.flatten().tolist() == [5.0, 7.0] and state[0].flatten().tolist() == [1.0, 1.0]
 
 
+@pytest.mark.parametrize("m", [1, 5, 16])
+@pytest.mark.parametrize("width,k,taps", [(16, 264, 2), (200, 1024, 3), (64, 2048, 4), (40, 512, 6), (24, 4608, 3)])
+def test_in_proj_and_conv_in_one_launch(m, width, k, taps):
+    """A decode step's rows: the projection to [B | C | x] and the gated conv in one launch give what
+    the two launches give (the same bits where both split K over the same waves), and shift the state."""
+    x = rnd(m, k, seed=1).to(torch.bfloat16).to(DEV)
+    w_in = rnd(3 * width, k, seed=2, scale=0.05).to(torch.bfloat16).to(DEV)
+    b_in = rnd(3 * width, seed=3, scale=0.1).to(DEV)
+    w = rnd(width, taps, seed=4, scale=0.3).to(DEV)
+    b = rnd(width, seed=5, scale=0.1).to(DEV)
+    state0 = rnd(20, taps - 1, width, seed=6)
+    slots = torch.randperm(20, generator=torch.Generator().manual_seed(7))[:m].to(torch.int32)
+    for use_bias in (True, False):
+        for out_dtype in (torch.float32, torch.bfloat16):
+            ctx = hand_context([(3, 1)] * m, 16, 2 * m, torch.float32, DEV, fixed_sites={0: (taps - 1, width)},
+                               n_slots=20, slots=slots.tolist())
+            state = ctx.fixed_state(0)
+            state.copy_(state0)
+            bcx = torch.empty(m, 3 * width, device=DEV)
+            ops().gemm(x, w_in, bcx, bias=b_in if use_bias else None)
+            two = torch.empty(m, width, dtype=out_dtype, device=DEV)
+            ops().short_conv(bcx, w, b if use_bias else None, state, ctx.row_of_token, ctx.seg_start, ctx.seg_len,
+                             ctx.slot, two, single_tokens=True)
+            state_two = state.cpu().clone()
+            state.copy_(state0)
+            one = torch.full((m, width), float("nan"), dtype=out_dtype, device=DEV)
+            ops().in_proj_conv_decode(x, w_in, b_in if use_bias else None, w, b if use_bias else None, state,
+                                      ctx.slot, one)
+            if k <= 2048:
+                assert torch.equal(one.cpu(), two.cpu()) and torch.equal(state.cpu(), state_two)
+            else:
+                tol = dict(rtol=1e-5, atol=1e-5) if out_dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -7)
+                torch.testing.assert_close(one.cpu().float(), two.cpu().float(), **tol)
+                torch.testing.assert_close(state.cpu(), state_two, rtol=1e-5, atol=1e-5)
+            untouched = [s for s in range(20) if s not in slots.tolist()]
+            assert torch.equal(state.cpu()[untouched], state0[untouched])
+    from imparo_amd.kernels import KernelArgumentError
+    with pytest.raises(KernelArgumentError, match="16"):
+        ops().in_proj_conv_decode(torch.zeros(17, k, dtype=torch.bfloat16, device=DEV), w_in, None, w, None, state,
+                                  torch.zeros(17, dtype=torch.int32, device=DEV), torch.empty(17, width, device=DEV))
+
+
 # ---------------------------------------------------------------- sampling
 @pytest.mark.parametrize("vocab", [7, 200, 1000, 65536, 70001])
 def test_argmax_rows(vocab):
