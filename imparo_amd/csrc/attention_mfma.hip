@@ -16,6 +16,7 @@
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 #define DEC_SPLIT 256     // keys per decode split, aligned at absolute multiples
 #define MFMA_WAVES 4
@@ -557,6 +558,280 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
     }
 }
 
+// ---------------------------------------------------------------- prompt portions, head sizes in steps of 32
+// The same walk with the 16x16x32 product and more work per staged tile. A wave takes 32
+// queries of one head as two halves of 16 that share every K and V^T fragment it reads from
+// LDS; a block's four waves are four heads that share a kv head (or two heads x two runs of
+// 32 queries, or one head x four runs, as the group size allows), so a tile of 64 keys is
+// fetched and staged once for all of them. Per 32 head dims, S^T of 16 keys x 16 queries is
+// one product; a lane's scores of the two products over keys 16t .. 16t+15 (t = 0, 1) of a
+// group of 32 keys are keys 16t + 4*(lane/16) + i, and those eight are the lane's eight
+// K-slots of the second product's B operand as they are. Its A operand, 16 bytes of a V^T
+// row, must hold the same eight keys: the V^T tile is staged with its keys in that order
+// (key k of a group of 32 at 8*((k%16)/4) + 4*(k/16) + k%4).
+#define PX_KEYS 64
+
+template <int ND>
+__global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill_x32(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    bf16_t* __restrict__ out, const int32_t* __restrict__ rows, int n_rows,
+    const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int n_pages,
+    float scale, int window, int heads_per_block) {
+    constexpr int D = ND * 16, NK = ND / 2;
+    constexpr int LDK = D + 8, LDV = PX_KEYS + 8;
+    static_assert(ND % 2 == 0, "head sizes in steps of 32");
+    const int page_shift = __ffs(page_size) - 1;
+    __shared__ __attribute__((aligned(16))) bf16_t ks[2][PX_KEYS * LDK];
+    __shared__ __attribute__((aligned(16))) bf16_t vs[2][D * LDV];
+    const int runs = MFMA_WAVES / heads_per_block;        // runs of 32 queries per block
+    const int qt = 32 * runs;                             // queries per block and head
+    int tile = blockIdx.x, row = -1;
+    if (((blockIdx.y * gridDim.x + blockIdx.x) / 256) & 1) tile = (int)gridDim.x - 1 - tile;
+    for (int i = 0; i < n_rows; ++i) {
+        const int r = rows[i];
+        const int nt = (seg_len[r] + qt - 1) / qt;
+        if (tile < nt) {
+            row = r;
+            break;
+        }
+        tile -= nt;
+    }
+    if (row < 0) return;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int c = lane & 15, g = lane >> 4;
+    const int len = seg_len[row];
+    const int head = blockIdx.y * heads_per_block + wave % heads_per_block;
+    const int kvh = (blockIdx.y * heads_per_block) / (heads / kv_heads);
+    const int t0 = seg_start[row];
+    const int pos0 = positions[t0];
+    const int32_t* table = block_table + (size_t)row * table_stride;
+
+    // the block's key range: from the lowest key its first query may read to its last query's position
+    const int blk_first = pos0 + tile * qt;
+    const int blk_last = pos0 + min(len, tile * qt + qt) - 1;
+    const int blk_lo = window > 0 ? max(0, blk_first + 1 - window) : 0;
+
+    // this wave's queries: q_first + 16 h + c for the halves h = 0, 1
+    const int q_first = tile * qt + (wave / heads_per_block) * 32;
+    const bool wave_on = q_first < len;
+    const int pos_first = pos0 + q_first;
+    const int pos_last = pos0 + min(len, q_first + 32) - 1;
+    const int lo_all = window > 0 ? max(0, pos_first + 1 - window) : 0;
+    const int lo_max = window > 0 ? max(0, pos_last + 1 - window) : 0;
+    int lo_q[2], hi_q[2];
+    bool qvalid[2];
+    Frag8 qf[2][NK];
+    f32x4 o[2][ND];
+    float m_run[2], l_run[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int qi = q_first + 16 * h + c;
+        qvalid[h] = qi < len;
+        const int pos_q = pos0 + qi;
+        lo_q[h] = window > 0 ? max(0, pos_q + 1 - window) : 0;
+        hi_q[h] = qvalid[h] ? pos_q : -1;
+        const bf16_t* qrow = q + ((size_t)(t0 + min(qi, len - 1)) * heads + head) * D + 8 * g;
+#pragma unroll
+        for (int dk = 0; dk < NK; ++dk)
+            qf[h][dk].u = zero_unless(qvalid[h] && wave_on, *reinterpret_cast<const uint4*>(qrow + 32 * dk));
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) o[h][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        m_run[h] = -INFINITY;
+        l_run[h] = 0.f;
+    }
+    const float scale_log2 = scale * 1.44269504088896340736f;
+
+    // Staging: K tile = 64 keys x D/8 pieces of 16 bytes; V^T tile = D rows x 8 pieces of 8 keys; with
+    // head sizes in steps of 32 the 256 threads take a whole number of pieces each. A piece's
+    // page comes out of the block table first and its data from that page: two trips to memory
+    // in a row. So the pages of a tile are asked for a tile ahead of its data, the data a tile
+    // ahead of its use, and no load sits under a branch (past the last tile they read the
+    // last tile again): the waits then fall where the values are needed and nowhere else.
+    constexpr int K_PER = PX_KEYS * (D / 8) / 256, V_PER = D * (PX_KEYS / 8) / 256;
+    static_assert(K_PER * 256 == PX_KEYS * (D / 8) && V_PER * 256 == D * (PX_KEYS / 8), "whole pieces per thread");
+    u32x4 kr[K_PER], vr[V_PER];           // (the compiler's own vector type: an array of HIP's uint4 stays in memory)
+    int kpage[K_PER], vpage[V_PER];
+    const int kb_last = blk_last & ~(PX_KEYS - 1);
+    auto load_pages = [&](int kb) __attribute__((always_inline)) {
+        kb = min(kb, kb_last);
+#pragma unroll
+        for (int j = 0; j < K_PER; ++j) {
+            const int pc = tid + j * 256;
+            const int key = min(max(kb + pc / (D / 8), blk_lo), blk_last);     // a live key: address always valid
+            kpage[j] = table[key >> page_shift];
+        }
+#pragma unroll
+        for (int j = 0; j < V_PER; ++j) {
+            const int pc = tid + j * 256;
+            const int kgc = min(max(kb + (pc % (PX_KEYS / 8)) * 8, blk_lo & ~7), blk_last & ~7);
+            vpage[j] = table[kgc >> page_shift];
+        }
+    };
+    auto load_data = [&](int kb) __attribute__((always_inline)) {
+        kb = min(kb, kb_last);
+#pragma unroll
+        for (int j = 0; j < K_PER; ++j) {
+            const int pc = tid + j * 256;
+            const int key = min(max(kb + pc / (D / 8), blk_lo), blk_last);
+            const int page = min(max(kpage[j], 0), n_pages - 1);
+            kr[j] = *reinterpret_cast<const u32x4*>(k_cache + (((size_t)page * kv_heads + kvh) * page_size +
+                                                               (key & (page_size - 1))) * D + (pc % (D / 8)) * 8);
+        }
+#pragma unroll
+        for (int j = 0; j < V_PER; ++j) {
+            const int pc = tid + j * 256;
+            const int d = pc / (PX_KEYS / 8);
+            const int kgc = min(max(kb + (pc % (PX_KEYS / 8)) * 8, blk_lo & ~7), blk_last & ~7);   // 8 keys, one page
+            const int page = min(max(vpage[j], 0), n_pages - 1);
+            vr[j] = *reinterpret_cast<const u32x4*>(v_cache + (((size_t)page * kv_heads + kvh) * D + d) * page_size +
+                                                    (kgc & (page_size - 1)));
+        }
+    };
+    // the tile whose data is in kr/vr goes to LDS: kb is its first key
+    auto stage_store = [&](int kb, int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < K_PER; ++j) {
+            const int pc = tid + j * 256;
+            *reinterpret_cast<u32x4*>(&ks[buf][(pc / (D / 8)) * LDK + (pc % (D / 8)) * 8]) = kr[j];
+        }
+#pragma unroll
+        for (int j = 0; j < V_PER; ++j) {
+            const int pc = tid + j * 256;
+            const int q8 = pc % (PX_KEYS / 8);
+            const int kg = kb + q8 * 8;
+            // values of keys outside the live range are zero, never stale memory
+            uint32_t w[4] = {vr[j].x, vr[j].y, vr[j].z, vr[j].w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const bool dead = kg + e < blk_lo || kg + e > blk_last;
+                w[e >> 1] = dead ? (w[e >> 1] & ((e & 1) ? 0x0000ffffu : 0xffff0000u)) : w[e >> 1];
+            }
+            // keys 8 q8 .. +7 of the tile: the first four go to 32 G + 16 (q8 % 2) + 4 t, the next four 8 further
+            bf16_t* dst = &vs[buf][(pc / (PX_KEYS / 8)) * LDV + 32 * (q8 >> 2) + 16 * (q8 & 1) + 4 * ((q8 >> 1) & 1)];
+            *reinterpret_cast<uint2*>(dst) = make_uint2(w[0], w[1]);
+            *reinterpret_cast<uint2*>(dst + 8) = make_uint2(w[2], w[3]);
+        }
+    };
+
+    const int kb_first = blk_lo & ~(PX_KEYS - 1);
+    load_pages(kb_first);
+    load_data(kb_first);
+    load_pages(kb_first + PX_KEYS);
+    stage_store(kb_first, 0);
+    __syncthreads();
+    int buf = 0;
+    for (int kb = kb_first; kb <= blk_last; kb += PX_KEYS) {
+        const int kn = kb + PX_KEYS;
+        load_data(kn);                    // with the pages asked for a tile ago
+        load_pages(kn + PX_KEYS);
+        // this wave's part of the tile: keys lo_all .. pos_last
+        if (wave_on && kb <= pos_last && kb + PX_KEYS - 1 >= lo_all) {
+            const bool full = kb >= lo_max && kb + PX_KEYS - 1 <= pos_first;
+            f32x4 sc[2][4];
+#pragma unroll
+            for (int s16 = 0; s16 < 4; ++s16) {
+                sc[0][s16] = f32x4{0.f, 0.f, 0.f, 0.f};
+                sc[1][s16] = f32x4{0.f, 0.f, 0.f, 0.f};
+                const bf16_t* krow = &ks[buf][(s16 * 16 + c) * LDK + 8 * g];
+#pragma unroll
+                for (int dk = 0; dk < NK; ++dk) {
+                    Frag8 kf;
+                    kf.u = *reinterpret_cast<const uint4*>(krow + dk * 32);
+                    sc[0][s16] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[0][dk].v, sc[0][s16], 0, 0, 0);
+                    sc[1][s16] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[1][dk].v, sc[1][s16], 0, 0, 0);
+                }
+            }
+            // sc[h][s16][i] = score of key kb + 16 s16 + 4 g + i for query (h, lane%16). The running
+            // maximum is kept in units of log2(e), so that every weight is one exp2 of a difference.
+            Frag8 pb[2][2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                float mx = -INFINITY;
+                if (full) {                               // most tiles: nothing to mask (the same for the whole wave)
+#pragma unroll
+                    for (int s16 = 0; s16 < 4; ++s16)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            sc[h][s16][i] *= scale_log2;
+                            mx = fmaxf(mx, sc[h][s16][i]);
+                        }
+                } else {
+#pragma unroll
+                    for (int s16 = 0; s16 < 4; ++s16)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int kp = kb + s16 * 16 + 4 * g + i;
+                            sc[h][s16][i] = (kp >= lo_q[h] && kp <= hi_q[h]) ? sc[h][s16][i] * scale_log2 : -INFINITY;
+                            mx = fmaxf(mx, sc[h][s16][i]);
+                        }
+                }
+                mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+                const float m_new = fmaxf(m_run[h], mx);
+                const float corr = (m_run[h] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run[h] - m_new);
+                const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;      // exp2(-inf - 0) = 0: masked keys
+                float psum = 0.f;
+#pragma unroll
+                for (int s16 = 0; s16 < 4; ++s16) {
+                    uint32_t pk[2];
+#pragma unroll
+                    for (int i = 0; i < 4; i += 2) {
+                        const float p0 = __builtin_amdgcn_exp2f(sc[h][s16][i] - m_sub);
+                        const float p1 = __builtin_amdgcn_exp2f(sc[h][s16][i + 1] - m_sub);
+                        pk[i >> 1] = f32x2_to_bf16x2(p0, p1);
+                        // the denominator sums what the product uses
+                        psum += __uint_as_float(pk[i >> 1] << 16) + __uint_as_float(pk[i >> 1] & 0xffff0000u);
+                    }
+                    // K-slots 4 t + i of group G, s16 = 2 G + t
+                    if (s16 & 1) {
+                        pb[h][s16 >> 1].u.z = pk[0];
+                        pb[h][s16 >> 1].u.w = pk[1];
+                    } else {
+                        pb[h][s16 >> 1].u.x = pk[0];
+                        pb[h][s16 >> 1].u.y = pk[1];
+                    }
+                }
+                psum += __shfl_xor(psum, 16, WAVE);
+                psum += __shfl_xor(psum, 32, WAVE);
+                l_run[h] = l_run[h] * corr + psum;
+                m_run[h] = m_new;
+#pragma unroll
+                for (int dt = 0; dt < ND; ++dt) o[h][dt] = o[h][dt] * corr;
+            }
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) {
+                const bf16_t* vrow = &vs[buf][(dt * 16 + c) * LDV + 8 * g];
+#pragma unroll
+                for (int G = 0; G < 2; ++G) {
+                    Frag8 vf;
+                    vf.u = *reinterpret_cast<const uint4*>(vrow + 32 * G);
+                    o[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pb[0][G].v, o[0][dt], 0, 0, 0);
+                    o[1][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pb[1][G].v, o[1][dt], 0, 0, 0);
+                }
+            }
+        }
+        stage_store(min(kn, kb_last), buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+    if (!wave_on) return;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        if (!qvalid[h]) continue;
+        const float inv = l_run[h] > 0.f ? 1.0f / l_run[h] : 0.f;
+        bf16_t* dst = out + ((size_t)(t0 + q_first + 16 * h + c) * heads + head) * D + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) {
+            s16x4 v;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = pack_bf16(o[h][dt][i] * inv);
+            *reinterpret_cast<s16x4*>(dst + dt * 16) = v;
+        }
+    }
+}
+
 // ---------------------------------------------------------------- entry points
 static int check_common(const void* q, const void* k_cache, const void* v_cache, const void* out, const int32_t* rows,
                         const int32_t* seg_start, const int32_t* positions, const int32_t* block_table,
@@ -620,6 +895,25 @@ extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, cons
     if (!seg_len || n_rows < 0 || n_tiles < 0 || heads > 65535) return IMPARO_BAD_ARGUMENT;
     if (n_rows == 0 || n_tiles == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;
+    if (head_dim % 32 == 0) {
+        // four heads of a kv head to a block where the group allows it, else more runs of 32 queries;
+        // n_tiles counts tiles of 64 queries per row: twice as many tiles of 32 at most, no more of 128
+        const int group = heads / kv_heads;
+        const int hpb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+        dim3 grid32(hpb == 4 ? 2 * n_tiles : n_tiles, heads / hpb);
+#define PREFILL_X32(ND)                                                                                              \
+    k_attn_prefill_x32<ND><<<grid32, MFMA_WAVES * 64, 0, s>>>(                                                       \
+        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, rows, n_rows, seg_start,    \
+        seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, hpb)
+        switch (head_dim / 32) {
+            case 1: PREFILL_X32(2); break;
+            case 2: PREFILL_X32(4); break;
+            case 3: PREFILL_X32(6); break;
+            default: PREFILL_X32(8);
+        }
+#undef PREFILL_X32
+        return launch_status();
+    }
     dim3 grid(n_tiles, heads);
     DISPATCH_ND(head_dim / 16, (k_attn_prefill<ND><<<grid, MFMA_WAVES * 64, 0, s>>>(
         (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, rows, n_rows, seg_start,

@@ -395,7 +395,8 @@ def test_attention(H, Hk, D, page_size, window):
     torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)      # one rounding of the output, P in float32
 
 
-@pytest.mark.parametrize("H,Hk,D", [(1, 1, 16), (6, 2, 48), (5, 5, 64), (8, 1, 128), (4, 2, 80), (40, 2, 32)])
+@pytest.mark.parametrize("H,Hk,D", [(1, 1, 16), (6, 2, 48), (5, 5, 64), (8, 1, 128), (4, 2, 80), (40, 2, 32),
+                                    (6, 3, 64), (12, 3, 96)])
 @pytest.mark.parametrize("page_size,window", [(16, None), (64, None), (32, 19), (16, 64), (16, 1), (128, 300)])
 def test_matrix_core_attention(H, Hk, D, page_size, window):
     """The split-KV decode kernel and the tiled prefill kernel: contexts that
