@@ -571,8 +571,10 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
 // (key k of a group of 32 at 8*((k%16)/4) + 4*(k/16) + k%4).
 #define PX_KEYS 64
 
+// (Two blocks per CU for head sizes up to 64: within 256 registers a wave the compiler keeps the
+// products' results in vector registers, where the softmax wants them, not in the accumulator file.)
 template <int ND>
-__global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill_x32(
+__global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefill_x32(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int32_t* __restrict__ rows, int n_rows,
     const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len, const int32_t* __restrict__ positions,
@@ -651,6 +653,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill_x32(
     // last tile again): the waits then fall where the values are needed and nowhere else.
     constexpr int K_PER = PX_KEYS * (D / 8) / 256, V_PER = D * (PX_KEYS / 8) / 256;
     static_assert(K_PER * 256 == PX_KEYS * (D / 8) && V_PER * 256 == D * (PX_KEYS / 8), "whole pieces per thread");
+    const size_t page_elems = (size_t)kv_heads * page_size * D;      // of one page of K (or V) over all kv heads
     u32x4 kr[K_PER], vr[V_PER];           // (the compiler's own vector type: an array of HIP's uint4 stays in memory)
     int kpage[K_PER], vpage[V_PER];
     const int kb_last = blk_last & ~(PX_KEYS - 1);
@@ -676,8 +679,8 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill_x32(
             const int pc = tid + j * 256;
             const int key = min(max(kb + pc / (D / 8), blk_lo), blk_last);
             const int page = min(max(kpage[j], 0), n_pages - 1);
-            kr[j] = *reinterpret_cast<const u32x4*>(k_cache + (((size_t)page * kv_heads + kvh) * page_size +
-                                                               (key & (page_size - 1))) * D + (pc % (D / 8)) * 8);
+            const unsigned in_page = (unsigned)(kvh * page_size + (key & (page_size - 1))) * D + (pc % (D / 8)) * 8;
+            kr[j] = *reinterpret_cast<const u32x4*>(k_cache + (size_t)page * page_elems + in_page);
         }
 #pragma unroll
         for (int j = 0; j < V_PER; ++j) {
@@ -685,8 +688,8 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill_x32(
             const int d = pc / (PX_KEYS / 8);
             const int kgc = min(max(kb + (pc % (PX_KEYS / 8)) * 8, blk_lo & ~7), blk_last & ~7);   // 8 keys, one page
             const int page = min(max(vpage[j], 0), n_pages - 1);
-            vr[j] = *reinterpret_cast<const u32x4*>(v_cache + (((size_t)page * kv_heads + kvh) * D + d) * page_size +
-                                                    (kgc & (page_size - 1)));
+            const unsigned in_page = (unsigned)(kvh * D + d) * page_size + (kgc & (page_size - 1));
+            vr[j] = *reinterpret_cast<const u32x4*>(v_cache + (size_t)page * page_elems + in_page);
         }
     };
     // the tile whose data is in kr/vr goes to LDS: kb is its first key
@@ -701,12 +704,15 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill_x32(
             const int pc = tid + j * 256;
             const int q8 = pc % (PX_KEYS / 8);
             const int kg = kb + q8 * 8;
-            // values of keys outside the live range are zero, never stale memory
+            // values of keys outside the live range are zero, never stale memory (a tile at either
+            // end of the block's range only: the same for every thread)
             uint32_t w[4] = {vr[j].x, vr[j].y, vr[j].z, vr[j].w};
+            if (kb < blk_lo || kb + PX_KEYS - 1 > blk_last) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const bool dead = kg + e < blk_lo || kg + e > blk_last;
-                w[e >> 1] = dead ? (w[e >> 1] & ((e & 1) ? 0x0000ffffu : 0xffff0000u)) : w[e >> 1];
+                for (int e = 0; e < 8; ++e) {
+                    const bool dead = kg + e < blk_lo || kg + e > blk_last;
+                    w[e >> 1] = dead ? (w[e >> 1] & ((e & 1) ? 0x0000ffffu : 0xffff0000u)) : w[e >> 1];
+                }
             }
             // keys 8 q8 .. +7 of the tile: the first four go to 32 G + 16 (q8 % 2) + 4 t, the next four 8 further
             bf16_t* dst = &vs[buf][(pc / (PX_KEYS / 8)) * LDV + 32 * (q8 >> 2) + 16 * (q8 & 1) + 4 * ((q8 >> 1) & 1)];
@@ -743,8 +749,9 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill_x32(
                     sc[1][s16] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[1][dk].v, sc[1][s16], 0, 0, 0);
                 }
             }
-            // sc[h][s16][i] = score of key kb + 16 s16 + 4 g + i for query (h, lane%16). The running
-            // maximum is kept in units of log2(e), so that every weight is one exp2 of a difference.
+            // sc[h][s16][i] = score of key kb + 16 s16 + 4 g + i for query (h, lane%16), unscaled. The
+            // running maximum is kept unscaled too: a weight is one fused multiply-add and one exp2,
+            // exp2((score - max) * scale * log2 e). The vector ALUs are what this kernel is bound by.
             Frag8 pb[2][2];
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
@@ -753,36 +760,31 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill_x32(
 #pragma unroll
                     for (int s16 = 0; s16 < 4; ++s16)
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            sc[h][s16][i] *= scale_log2;
-                            mx = fmaxf(mx, sc[h][s16][i]);
-                        }
+                        for (int i = 0; i < 4; ++i) mx = fmaxf(mx, sc[h][s16][i]);
                 } else {
 #pragma unroll
                     for (int s16 = 0; s16 < 4; ++s16)
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
                             const int kp = kb + s16 * 16 + 4 * g + i;
-                            sc[h][s16][i] = (kp >= lo_q[h] && kp <= hi_q[h]) ? sc[h][s16][i] * scale_log2 : -INFINITY;
+                            sc[h][s16][i] = (kp >= lo_q[h] && kp <= hi_q[h]) ? sc[h][s16][i] : -INFINITY;
                             mx = fmaxf(mx, sc[h][s16][i]);
                         }
                 }
                 mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
                 mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
                 const float m_new = fmaxf(m_run[h], mx);
-                const float corr = (m_run[h] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run[h] - m_new);
-                const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;      // exp2(-inf - 0) = 0: masked keys
+                const float m_sub = (m_new == -INFINITY) ? 0.f : m_new * scale_log2;   // exp2(-inf - 0) = 0: masked keys
                 float psum = 0.f;
 #pragma unroll
                 for (int s16 = 0; s16 < 4; ++s16) {
                     uint32_t pk[2];
 #pragma unroll
                     for (int i = 0; i < 4; i += 2) {
-                        const float p0 = __builtin_amdgcn_exp2f(sc[h][s16][i] - m_sub);
-                        const float p1 = __builtin_amdgcn_exp2f(sc[h][s16][i + 1] - m_sub);
+                        const float p0 = __builtin_amdgcn_exp2f(fmaf(sc[h][s16][i], scale_log2, -m_sub));
+                        const float p1 = __builtin_amdgcn_exp2f(fmaf(sc[h][s16][i + 1], scale_log2, -m_sub));
                         pk[i >> 1] = f32x2_to_bf16x2(p0, p1);
-                        // the denominator sums what the product uses
-                        psum += __uint_as_float(pk[i >> 1] << 16) + __uint_as_float(pk[i >> 1] & 0xffff0000u);
+                        psum += p0 + p1;
                     }
                     // K-slots 4 t + i of group G, s16 = 2 G + t
                     if (s16 & 1) {
@@ -795,10 +797,16 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill_x32(
                 }
                 psum += __shfl_xor(psum, 16, WAVE);
                 psum += __shfl_xor(psum, 32, WAVE);
-                l_run[h] = l_run[h] * corr + psum;
-                m_run[h] = m_new;
+                // the old sums shrink by exp2((old max - new max) * scale): by 1, and nothing to do, for
+                // every query whose maximum stood (the whole wave mostly, once the walk is under way)
+                if (__any(m_new != m_run[h])) {
+                    const float corr = (m_run[h] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_run[h] - m_new) * scale_log2);
+                    l_run[h] *= corr;
 #pragma unroll
-                for (int dt = 0; dt < ND; ++dt) o[h][dt] = o[h][dt] * corr;
+                    for (int dt = 0; dt < ND; ++dt) o[h][dt] = o[h][dt] * corr;
+                }
+                l_run[h] += psum;
+                m_run[h] = m_new;
             }
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt) {
