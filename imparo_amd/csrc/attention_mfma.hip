@@ -573,7 +573,8 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
 
 // (Two blocks per CU for head sizes up to 64: within 256 registers a wave the compiler keeps the
 // products' results in vector registers, where the softmax wants them, not in the accumulator file.)
-template <int ND>
+// HALVES: 2 for 32 queries a wave; 1 for 16, twice the waves, when a launch has too few to fill the SIMDs twice.
+template <int ND, int HALVES>
 __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefill_x32(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int32_t* __restrict__ rows, int n_rows,
@@ -586,8 +587,9 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     const int page_shift = __ffs(page_size) - 1;
     __shared__ __attribute__((aligned(16))) bf16_t ks[2][PX_KEYS * LDK];
     __shared__ __attribute__((aligned(16))) bf16_t vs[2][D * LDV];
-    const int runs = MFMA_WAVES / heads_per_block;        // runs of 32 queries per block
-    const int qt = 32 * runs;                             // queries per block and head
+    constexpr int QW = 16 * HALVES;                       // queries of a wave
+    const int runs = MFMA_WAVES / heads_per_block;        // runs of QW queries per block
+    const int qt = QW * runs;                             // queries per block and head
     int tile = blockIdx.x, row = -1;
     if (((blockIdx.y * gridDim.x + blockIdx.x) / 256) & 1) tile = (int)gridDim.x - 1 - tile;
     for (int i = 0; i < n_rows; ++i) {
@@ -615,20 +617,20 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     const int blk_last = pos0 + min(len, tile * qt + qt) - 1;
     const int blk_lo = window > 0 ? max(0, blk_first + 1 - window) : 0;
 
-    // this wave's queries: q_first + 16 h + c for the halves h = 0, 1
-    const int q_first = tile * qt + (wave / heads_per_block) * 32;
+    // this wave's queries: q_first + 16 h + c for the halves h
+    const int q_first = tile * qt + (wave / heads_per_block) * QW;
     const bool wave_on = q_first < len;
     const int pos_first = pos0 + q_first;
-    const int pos_last = pos0 + min(len, q_first + 32) - 1;
+    const int pos_last = pos0 + min(len, q_first + QW) - 1;
     const int lo_all = window > 0 ? max(0, pos_first + 1 - window) : 0;
     const int lo_max = window > 0 ? max(0, pos_last + 1 - window) : 0;
-    int lo_q[2], hi_q[2];
-    bool qvalid[2];
-    Frag8 qf[2][NK];
-    f32x4 o[2][ND];
-    float m_run[2], l_run[2];
+    int lo_q[HALVES], hi_q[HALVES];
+    bool qvalid[HALVES];
+    Frag8 qf[HALVES][NK];
+    f32x4 o[HALVES][ND];
+    float m_run[HALVES], l_run[HALVES];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int h = 0; h < HALVES; ++h) {
         const int qi = q_first + 16 * h + c;
         qvalid[h] = qi < len;
         const int pos_q = pos0 + qi;
@@ -735,26 +737,27 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
         // this wave's part of the tile: keys lo_all .. pos_last
         if (wave_on && kb <= pos_last && kb + PX_KEYS - 1 >= lo_all) {
             const bool full = kb >= lo_max && kb + PX_KEYS - 1 <= pos_first;
-            f32x4 sc[2][4];
+            f32x4 sc[HALVES][4];
 #pragma unroll
             for (int s16 = 0; s16 < 4; ++s16) {
-                sc[0][s16] = f32x4{0.f, 0.f, 0.f, 0.f};
-                sc[1][s16] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int h = 0; h < HALVES; ++h) sc[h][s16] = f32x4{0.f, 0.f, 0.f, 0.f};
                 const bf16_t* krow = &ks[buf][(s16 * 16 + c) * LDK + 8 * g];
 #pragma unroll
                 for (int dk = 0; dk < NK; ++dk) {
                     Frag8 kf;
                     kf.u = *reinterpret_cast<const uint4*>(krow + dk * 32);
-                    sc[0][s16] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[0][dk].v, sc[0][s16], 0, 0, 0);
-                    sc[1][s16] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[1][dk].v, sc[1][s16], 0, 0, 0);
+#pragma unroll
+                    for (int h = 0; h < HALVES; ++h)
+                        sc[h][s16] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[h][dk].v, sc[h][s16], 0, 0, 0);
                 }
             }
             // sc[h][s16][i] = score of key kb + 16 s16 + 4 g + i for query (h, lane%16), unscaled. The
             // running maximum is kept unscaled too: a weight is one fused multiply-add and one exp2,
             // exp2((score - max) * scale * log2 e). The vector ALUs are what this kernel is bound by.
-            Frag8 pb[2][2];
+            Frag8 pb[HALVES][2];
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
+            for (int h = 0; h < HALVES; ++h) {
                 float mx = -INFINITY;
                 if (full) {                               // most tiles: nothing to mask (the same for the whole wave)
 #pragma unroll
@@ -815,8 +818,9 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
                 for (int G = 0; G < 2; ++G) {
                     Frag8 vf;
                     vf.u = *reinterpret_cast<const uint4*>(vrow + 32 * G);
-                    o[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pb[0][G].v, o[0][dt], 0, 0, 0);
-                    o[1][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pb[1][G].v, o[1][dt], 0, 0, 0);
+#pragma unroll
+                    for (int h = 0; h < HALVES; ++h)
+                        o[h][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pb[h][G].v, o[h][dt], 0, 0, 0);
                 }
             }
         }
@@ -826,7 +830,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     }
     if (!wave_on) return;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int h = 0; h < HALVES; ++h) {
         if (!qvalid[h]) continue;
         const float inv = l_run[h] > 0.f ? 1.0f / l_run[h] : 0.f;
         bf16_t* dst = out + ((size_t)(t0 + q_first + 16 * h + c) * heads + head) * D + 4 * g;
@@ -904,15 +908,24 @@ extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, cons
     if (n_rows == 0 || n_tiles == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;
     if (head_dim % 32 == 0) {
-        // four heads of a kv head to a block where the group allows it, else more runs of 32 queries;
-        // n_tiles counts tiles of 64 queries per row: twice as many tiles of 32 at most, no more of 128
+        // four heads of a kv head to a block where the group allows it, else more runs of queries
         const int group = heads / kv_heads;
         const int hpb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
-        dim3 grid32(hpb == 4 ? 2 * n_tiles : n_tiles, heads / hpb);
+        // 32 queries a wave unless that leaves fewer waves than twice the SIMDs (n_tiles x 64 queries x heads at most)
+        const bool wide = (long long)n_tiles * 2 * heads >= 2048;
+        // n_tiles counts tiles of 64 queries per row: a row has at most that many blocks of 64 queries or more,
+        // and 64 / qt times as many of fewer (blocks past a row's last find no tile and leave)
+        const int qt = (wide ? 32 : 16) * (MFMA_WAVES / hpb);
+        dim3 grid32((unsigned)(n_tiles * (qt < 64 ? 64 / qt : 1)), heads / hpb);
 #define PREFILL_X32(ND)                                                                                              \
-    k_attn_prefill_x32<ND><<<grid32, MFMA_WAVES * 64, 0, s>>>(                                                       \
-        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, rows, n_rows, seg_start,    \
-        seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, hpb)
+    if (wide)                                                                                                        \
+        k_attn_prefill_x32<ND, 2><<<grid32, MFMA_WAVES * 64, 0, s>>>(                                                \
+            (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, rows, n_rows, seg_start, \
+            seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, hpb); \
+    else                                                                                                             \
+        k_attn_prefill_x32<ND, 1><<<grid32, MFMA_WAVES * 64, 0, s>>>(                                                \
+            (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, rows, n_rows, seg_start, \
+            seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, hpb)
         switch (head_dim / 32) {
             case 1: PREFILL_X32(2); break;
             case 2: PREFILL_X32(4); break;

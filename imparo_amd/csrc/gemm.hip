@@ -1233,7 +1233,7 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
         else
             launch_skinny<TOut, 4>(x, w, bias, y, m, n, k, epilogue, slices, s);
     } else {
-        // `force` 256: the 256x256 tile on eight waves; 257: 256x128; 258: 256x256 on four waves with loads
+        // `force` 256: the 256x256 tile on eight waves; 258: 256x256 on four waves with loads
         // straight into LDS (for measurements); otherwise by shape
         if (slices == 1 && force == 0 && big_tile_pays(m, n, k) && dma_tile_takes(m, n, k))
             return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, 1, s);
@@ -1241,8 +1241,6 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
             return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, slices, s);
         if (slices == 1 && (force == 256 || (force == 0 && big_tile_pays(m, n, k))))
             return launch_big<TOut, 2, 4, 4, 2>(x, w, bias, y, m, n, k, epilogue, s);
-        if (slices == 1 && force == 257)
-            return launch_big<TOut, 4, 2, 2, 2>(x, w, bias, y, m, n, k, epilogue, s);
         if (force == 258 && k % slices == 0 && dma_tile_takes(m, n, k / slices) && dma_tile_takes(m, n, k))
             return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, slices, s);
         const int tiles_m = (m + BG_BM - 1) / BG_BM, tiles_n = (n + BG_BN - 1) / BG_BN;
@@ -1260,7 +1258,7 @@ static int g_force_few_row_kernel = 0;
 static int g_force_slices = 0;
 
 // For measurements only: 0 lets the library choose the kernel, 1 forces the K-split kernel,
-// 2, 4 or 8 the shared-activation kernel with that many waves, 256/257 the large tiles;
+// 2, 4 or 8 the shared-activation kernel with that many waves, 256/258 the large tiles;
 // plus 1000 times a number of K slices that imparo_gemm then accepts whatever the shape.
 extern "C" void imparo_gemm_force_kernel(int which) {
     g_force_slices = which / 1000;
