@@ -652,11 +652,14 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     // page comes out of the block table first and its data from that page: two trips to memory
     // in a row. So the pages of a tile are asked for a tile ahead of its data, the data a tile
     // ahead of its use, and no load sits under a branch (past the last tile they read the
-    // last tile again): the waits then fall where the values are needed and nowhere else.
+    // last tile again): the waits then fall where the values are needed and nowhere else. With long
+    // contexts the keys come from HBM and take longer than a tile's arithmetic: two register sets,
+    // so that a tile's data is asked for two tiles before it goes to LDS.
     constexpr int K_PER = PX_KEYS * (D / 8) / 256, V_PER = D * (PX_KEYS / 8) / 256;
     static_assert(K_PER * 256 == PX_KEYS * (D / 8) && V_PER * 256 == D * (PX_KEYS / 8), "whole pieces per thread");
     const size_t page_elems = (size_t)kv_heads * page_size * D;      // of one page of K (or V) over all kv heads
-    u32x4 kr[K_PER], vr[V_PER];           // (the compiler's own vector type: an array of HIP's uint4 stays in memory)
+    // (the compiler's own vector type: an array of HIP's uint4 stays in memory)
+    u32x4 kr_a[K_PER], vr_a[V_PER], kr_b[K_PER], vr_b[V_PER];
     int kpage[K_PER], vpage[V_PER];
     const int kb_last = blk_last & ~(PX_KEYS - 1);
     auto load_pages = [&](int kb) __attribute__((always_inline)) {
@@ -674,7 +677,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
             vpage[j] = table[kgc >> page_shift];
         }
     };
-    auto load_data = [&](int kb) __attribute__((always_inline)) {
+    auto load_data = [&](int kb, u32x4 (&kr)[K_PER], u32x4 (&vr)[V_PER]) __attribute__((always_inline)) {
         kb = min(kb, kb_last);
 #pragma unroll
         for (int j = 0; j < K_PER; ++j) {
@@ -695,7 +698,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
         }
     };
     // the tile whose data is in kr/vr goes to LDS: kb is its first key
-    auto stage_store = [&](int kb, int buf) __attribute__((always_inline)) {
+    auto stage_store = [&](int kb, int buf, const u32x4 (&kr)[K_PER], const u32x4 (&vr)[V_PER]) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < K_PER; ++j) {
             const int pc = tid + j * 256;
@@ -723,17 +726,12 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
         }
     };
 
-    const int kb_first = blk_lo & ~(PX_KEYS - 1);
-    load_pages(kb_first);
-    load_data(kb_first);
-    load_pages(kb_first + PX_KEYS);
-    stage_store(kb_first, 0);
-    __syncthreads();
-    int buf = 0;
-    for (int kb = kb_first; kb <= blk_last; kb += PX_KEYS) {
-        const int kn = kb + PX_KEYS;
-        load_data(kn);                    // with the pages asked for a tile ago
-        load_pages(kn + PX_KEYS);
+    // One tile: LDS buffer `buf` holds it, `have` the next tile's data (asked for a tile ago), `fill`
+    // takes the loads of the tile after that; then `have` goes to the other LDS buffer.
+    auto tile_step = [&](int kb, int buf, u32x4 (&kr_have)[K_PER], u32x4 (&vr_have)[V_PER], u32x4 (&kr_fill)[K_PER],
+                         u32x4 (&vr_fill)[V_PER]) __attribute__((always_inline)) {
+        load_data(kb + 2 * PX_KEYS, kr_fill, vr_fill);      // with the pages asked for a tile ago
+        load_pages(kb + 3 * PX_KEYS);
         // this wave's part of the tile: keys lo_all .. pos_last
         if (wave_on && kb <= pos_last && kb + PX_KEYS - 1 >= lo_all) {
             const bool full = kb >= lo_max && kb + PX_KEYS - 1 <= pos_first;
@@ -824,9 +822,21 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
                 }
             }
         }
-        stage_store(min(kn, kb_last), buf ^ 1);
+        stage_store(min(kb + PX_KEYS, kb_last), buf ^ 1, kr_have, vr_have);
         __syncthreads();
-        buf ^= 1;
+    };
+    const int kb_first = blk_lo & ~(PX_KEYS - 1);
+    load_pages(kb_first);
+    load_data(kb_first, kr_a, vr_a);
+    load_pages(kb_first + PX_KEYS);
+    load_data(kb_first + PX_KEYS, kr_b, vr_b);
+    load_pages(kb_first + 2 * PX_KEYS);
+    stage_store(kb_first, 0, kr_a, vr_a);
+    __syncthreads();
+    for (int kb = kb_first; kb <= blk_last; kb += 2 * PX_KEYS) {
+        tile_step(kb, 0, kr_b, vr_b, kr_a, vr_a);
+        if (kb + PX_KEYS > blk_last) break;
+        tile_step(kb + PX_KEYS, 1, kr_a, vr_a, kr_b, vr_b);
     }
     if (!wave_on) return;
 #pragma unroll
