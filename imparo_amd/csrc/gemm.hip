@@ -796,7 +796,7 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, const float* bias, T
         k_gemm_bf16_skinny<TOut, MT, 4><<<grid, 4 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
     else if (k_per <= 2048)
         k_gemm_bf16_skinny<TOut, MT, 8><<<grid, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
-    else if (MT <= 2)
+    else if constexpr (MT <= 2)
         k_gemm_bf16_skinny<TOut, MT, 16><<<grid, 16 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
     else   // 64 activation rows keep too many fragments in registers for 1024 threads
         k_gemm_bf16_skinny<TOut, MT, 8><<<grid, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
@@ -1106,11 +1106,13 @@ __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
 #pragma unroll
         for (int j = 0; j < XP; ++j) f.x[j] = *reinterpret_cast<const uint4*>(xsrc[j] + min(k0 + xkc[j], K - 8));
     };
-    auto stash = [&](int kt, int buf, const StreamSet<XP>& f) {
-        const int k0 = chunk_of(kt) * ST_BK;
+    // (What an activation chunk holds at or beyond K is real data read again from inside the row; only
+    // the weights there are zeroed, in `compute`: one select per weight value instead of one more per
+    // activation value, which with 64 rows were a third of the kernel's vector instructions.)
+    auto stash = [&](int buf, const StreamSet<XP>& f) {
 #pragma unroll
         for (int j = 0; j < XP; ++j)     // threads beyond the last piece repeat it: same value, same place
-            *reinterpret_cast<uint4*>(&xs[buf][xdst[j]]) = zero_if(k0 + xkc[j] >= K, f.x[j]);
+            *reinterpret_cast<uint4*>(&xs[buf][xdst[j]]) = f.x[j];
     };
     f32x4 acc[MT];
 #pragma unroll
@@ -1151,7 +1153,7 @@ __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
     // chunk i-1 used takes the loads of chunk i+3, then chunk i is multiplied
     auto step = [&](int i, const StreamSet<XP>& cur, const StreamSet<XP>& next, StreamSet<XP>& refill) {
         const int buf = i & 1;
-        stash(i + 1, buf ^ 1, next);
+        stash(buf ^ 1, next);
         fetch(i + 3, refill);
         compute(i, buf, cur);
         __syncthreads();
@@ -1160,7 +1162,7 @@ __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
     fetch(0, s0);
     fetch(1, s1);
     fetch(2, s2);
-    stash(0, 0, s0);
+    stash(0, s0);
     __syncthreads();
     for (int kt = 0; kt < nk; kt += 4) {
         step(kt, s0, s1, s3);
