@@ -328,6 +328,70 @@ __global__ void k_short_conv_v4(const float* __restrict__ bcx, const float* __re
     store_four(out + (size_t)t * width + ch, c.x * acc[0], c.y * acc[1], c.z * acc[2], c.w * acc[3]);
 }
 
+// For prompt portions and a short history (HIST = taps - 1 <= 3): four channels and TT
+// consecutive tokens to a thread. The thread reads B*x of its tokens and of the HIST tokens
+// before them once (the plain kernel reads each value taps times), every load issued before
+// the first use and none under a branch; only a token among the first HIST of its segment
+// takes its oldest values from the request's state instead. Each channel's taps are summed
+// exactly as above.
+template <typename TOut, int HIST, int TT>
+__global__ void k_short_conv_tile(const float* __restrict__ bcx, const float* __restrict__ weight,
+                                  const float* __restrict__ bias, const float* __restrict__ state,
+                                  const int32_t* __restrict__ row_of_token, const int32_t* __restrict__ seg_start,
+                                  const int32_t* __restrict__ slot, TOut* __restrict__ out, int n_tokens, int width) {
+    const int ch = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    const int t0 = blockIdx.y * TT;
+    if (ch >= width) return;
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    f4 u[TT + HIST], c[TT];
+#pragma unroll
+    for (int j = 0; j < TT + HIST; ++j) {
+        const int tj = min(max(t0 - HIST + j, 0), n_tokens - 1);
+        const float* row = bcx + (size_t)tj * 3 * width + ch;
+        u[j] = *reinterpret_cast<const f4*>(row) * *reinterpret_cast<const f4*>(row + 2 * width);
+    }
+#pragma unroll
+    for (int i = 0; i < TT; ++i)
+        c[i] = *reinterpret_cast<const f4*>(bcx + (size_t)min(t0 + i, n_tokens - 1) * 3 * width + width + ch);
+    float w[4][HIST + 1];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int k = 0; k <= HIST; ++k) w[q][k] = weight[(size_t)(ch + q) * (HIST + 1) + k];
+    f4 bv = {0.f, 0.f, 0.f, 0.f};
+    if (bias) bv = *reinterpret_cast<const f4*>(bias + ch);
+#pragma unroll
+    for (int i = 0; i < TT; ++i) {
+        const int t = t0 + i;
+        if (t >= n_tokens) break;
+        const int r = row_of_token[t];
+        const int local = t - seg_start[r];
+        f4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k <= HIST; ++k) {
+            f4 v = u[i + k];                                   // token t - (HIST - k)
+            if (local + k < HIST)                               // before the segment's first token: the state
+                v = *reinterpret_cast<const f4*>(state + ((size_t)slot[r] * HIST + local + k) * width + ch);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[q] = fmaf(w[q][k], v[q], acc[q]);
+        }
+        acc += bv;
+        const f4 y = c[i] * acc;
+        store_four(out + (size_t)t * width + ch, y.x, y.y, y.z, y.w);
+    }
+}
+
+template <typename TOut, int HIST>
+static void launch_conv_tile(const float* bcx, const float* weight, const float* bias, const float* state,
+                             const int32_t* row_of_token, const int32_t* seg_start, const int32_t* slot, TOut* out,
+                             int n_tokens, int width, hipStream_t s) {
+    constexpr int TT = 4;
+    const int threads = width >= 1024 ? 256 : 64;
+    dim3 grid((width / 4 + threads - 1) / threads, (n_tokens + TT - 1) / TT);
+    k_short_conv_tile<TOut, HIST, TT><<<grid, threads, 0, s>>>(bcx, weight, bias, state, row_of_token, seg_start, slot,
+                                                               out, n_tokens, width);
+}
+
 extern "C" int imparo_short_conv(const float* bcx, const float* weight, const float* bias, const float* state,
                                  const int32_t* row_of_token, const int32_t* seg_start, const int32_t* slot,
                                  void* out, int out_dtype, int n_tokens, int width, int taps, int n_slots,
@@ -340,6 +404,21 @@ extern "C" int imparo_short_conv(const float* bcx, const float* weight, const fl
     if (width % 4 == 0 && n_tokens >= 32 && ((uintptr_t)bcx % 16) == 0 && ((uintptr_t)state % 16) == 0 &&
         ((uintptr_t)out % 16) == 0 && (!bias || ((uintptr_t)bias % 16) == 0) &&
         (out_dtype == IMPARO_F32 || out_dtype == IMPARO_BF16)) {
+        if (taps <= 4 && (n_tokens + 3) / 4 <= 65535) {
+#define CONV_TILE(T)                                                                                                 \
+    switch (taps - 1) {                                                                                              \
+        case 1: launch_conv_tile<T, 1>(bcx, weight, bias, state, row_of_token, seg_start, slot, (T*)out, n_tokens, width, s); break; \
+        case 2: launch_conv_tile<T, 2>(bcx, weight, bias, state, row_of_token, seg_start, slot, (T*)out, n_tokens, width, s); break; \
+        default: launch_conv_tile<T, 3>(bcx, weight, bias, state, row_of_token, seg_start, slot, (T*)out, n_tokens, width, s);      \
+    }
+            if (out_dtype == IMPARO_F32) {
+                CONV_TILE(float)
+            } else {
+                CONV_TILE(bf16_t)
+            }
+#undef CONV_TILE
+            return launch_status();
+        }
         const int threads4 = width >= 1024 ? 256 : 64;
         dim3 grid4((width / 4 + threads4 - 1) / threads4, n_tokens);
         if (out_dtype == IMPARO_F32)
