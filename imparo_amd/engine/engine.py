@@ -131,6 +131,7 @@ class Engine:
         # HIP graph: the launches of a step cost more host time than the step's kernels take
         self.use_graphs = use_graphs
         self._graphs: Dict[Tuple[int, int], _DecodeGraph] = {}
+        self._decode_code_loaded = False
         self._graph_pool = None
         self.vocab_size = self.plan.vocab_size
         self.max_position = self.plan.max_position
@@ -189,7 +190,8 @@ class Engine:
                 logits = self._decode_step(entries, batch)       # one token each, wanted
             else:
                 ctx, token_ids, want_rows = self._pack(batch)
-                logits = self.model.forward(ctx, token_ids, want_rows)
+                with ops.on_current_stream():
+                    logits = self.model.forward(ctx, token_ids, want_rows)
         except BaseException:
             self.cache.abort_step(batch)
             raise
@@ -214,16 +216,19 @@ class Engine:
         return f"request {e.request!r}: the cache manager refused the step with code {code}"
 
     def _decode_step(self, entries: Sequence[StepEntry], batch) -> torch.Tensor:
-        """A step of single tokens. The first step of a batch shape runs
-        launch by launch (so that every kernel it needs has been loaded), the
-        second is captured, later ones replay the capture."""
+        """A step of single tokens. The engine's first such step runs launch by
+        launch (a capture cannot load code onto the device, and every module of
+        kernels a decode step uses is loaded once one has run); after that a
+        batch shape is captured when it first comes and replayed from then on."""
         width = -(-batch.widest // TABLE_BUCKET) * TABLE_BUCKET
         key = (len(entries), width)
         g = self._graphs.setdefault(key, _DecodeGraph())
         g.seen += 1
-        if g.seen == 1:
+        if not self._decode_code_loaded:
+            self._decode_code_loaded = True
             ctx, token_ids, want_rows = self._pack(batch)
-            return self.model.forward(ctx, token_ids, want_rows)
+            with ops.on_current_stream():
+                return self.model.forward(ctx, token_ids, want_rows)
         if g.graph is None:
             g.workspace = Workspace(self.device)
             # the capture fixes grid sizes: they are sized for the widest context the tables can hold
@@ -231,7 +236,7 @@ class Engine:
             if self._graph_pool is None:
                 self._graph_pool = torch.cuda.graph_pool_handle()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
+            with torch.cuda.graph(graph, pool=self._graph_pool), ops.on_current_stream():
                 g.logits = self.model.forward(ctx, token_ids, want_rows)
             g.graph = graph
         else:

@@ -44,7 +44,29 @@ def _dev(t: Optional[torch.Tensor], what: str, dtype=None, shape=None) -> int:
     return t.data_ptr()
 
 
+_launch_stream: Optional[int] = None
+
+
+class on_current_stream:
+    """For a run of launches that all go to the stream that is current now (a
+    step's hundred kernels, also under graph capture): looks the stream up once
+    instead of once per launch, which costs more host time than the launch."""
+
+    def __enter__(self):
+        global _launch_stream
+        self._before = _launch_stream
+        _launch_stream = torch.cuda.current_stream().cuda_stream
+        return self
+
+    def __exit__(self, *exc):
+        global _launch_stream
+        _launch_stream = self._before
+        return False
+
+
 def _stream() -> int:
+    if _launch_stream is not None:
+        return _launch_stream
     return torch.cuda.current_stream().cuda_stream
 
 
