@@ -494,13 +494,18 @@ __device__ __forceinline__ void load_to_lds(const bf16_t* src, bf16_t* dst_wave_
                                      (void __attribute__((address_space(3)))*)dst_wave_uniform, 16, 0, 0);
 }
 
-template <typename TOut>
+// TN: MFMA tiles across a wave's part of the weight rows: the block's tile is 256 activation rows
+// x 64 TN weight rows (256, 192 or 128), chosen by the launcher so that the blocks come out in
+// whole rounds of the CUs.
+template <typename TOut, int TN>
 __global__ __launch_bounds__(256) void k_gemm_bf16_dma(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                        const float* __restrict__ bias, TOut* __restrict__ Y,
                                                        int M, int N, int K_all, int k_per, int tiles_m, int tiles_n,
                                                        int epilogue) {
-    __shared__ __attribute__((aligned(1024))) bf16_t stage0[2 * DM_T * DM_BK];   // X rows, then W rows
-    __shared__ __attribute__((aligned(1024))) bf16_t stage1[2 * DM_T * DM_BK];
+    constexpr int BN = 64 * TN;                        // weight rows of the block's tile
+    constexpr int WN = 32 * TN;                        // of one wave's part
+    __shared__ __attribute__((aligned(1024))) bf16_t stage0[(DM_T + BN) * DM_BK];   // X rows, then W rows
+    __shared__ __attribute__((aligned(1024))) bf16_t stage1[(DM_T + BN) * DM_BK];
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + N_XCD - 1) / N_XCD;
     const int logical = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;
@@ -510,7 +515,7 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_dma(const bf16_t* __restrict_
     const int gsize = min(tiles_m - first_m, BG_GROUP_M);
     const int tile_m = first_m + (logical % per_group) % gsize;
     const int tile_n = (logical % per_group) / gsize;
-    const int m0 = tile_m * DM_T, n0 = tile_n * DM_T;
+    const int m0 = tile_m * DM_T, n0 = tile_n * BN;
     // slices of K (gridDim.y > 1): block (x, y) sums K range [y * k_per, (y+1) * k_per) into Y + y * M * N
     const int k_lo = blockIdx.y * k_per;
     const int K = min(K_all, k_lo + k_per) - k_lo;
@@ -525,49 +530,50 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_dma(const bf16_t* __restrict_
     // loading: instruction j of a wave fills rows j*32 + wave*8 .. +7; lane -> row lane/8, slot lane%8
     const int load_row = wave * 8 + (lane >> 3);
     const int load_piece = (lane & 7) ^ (lane >> 3) ^ (wave & 1);          // lane%8 ^ swz(row)
-    unsigned off_x[8], off_w[8];
+    unsigned off_x[8], off_w[2 * TN];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < 8; ++j)
         off_x[j] = (unsigned)min(m0 + j * 32 + load_row, M - 1) * (unsigned)K_all + load_piece * 8;
+#pragma unroll
+    for (int j = 0; j < 2 * TN; ++j)
         off_w[j] = (unsigned)min(n0 + j * 32 + load_row, N - 1) * (unsigned)K_all + load_piece * 8;
-    }
     auto load_step = [&](bf16_t* stage, int kt) __attribute__((always_inline)) {
         const bf16_t* xk = X + (size_t)kt * DM_BK;
         const bf16_t* wk = W + (size_t)kt * DM_BK;
 #pragma unroll
         for (int j = 0; j < 8; ++j) load_to_lds(xk + off_x[j], stage + (j * 32 + wave * 8) * DM_BK);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) load_to_lds(wk + off_w[j], stage + (DM_T + j * 32 + wave * 8) * DM_BK);
+        for (int j = 0; j < 2 * TN; ++j) load_to_lds(wk + off_w[j], stage + (DM_T + j * 32 + wave * 8) * DM_BK);
     };
     // fragments: lane holds row lane%32, K-half lane/32 of a 32x16 piece; sub-step ks is pieces 2ks, 2ks+1
     const int frag_row = lane & 31;
     const int swz = (frag_row & 7) ^ ((frag_row >> 3) & 1);
     const int a_base = (wm * 128 + frag_row) * DM_BK + (((lane >> 5) ^ swz) << 3);
-    const int b_base = (DM_T + wn * 128 + frag_row) * DM_BK + (((lane >> 5) ^ swz) << 3);
-    f32x16 acc[4][4];
+    const int b_base = (DM_T + wn * WN + frag_row) * DM_BK + (((lane >> 5) ^ swz) << 3);
+    f32x16 acc[4][TN];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    auto read = [&](const bf16_t* stage, int ks, Frag8 (&fa)[4], Frag8 (&fb)[4]) __attribute__((always_inline)) {
+    auto read = [&](const bf16_t* stage, int ks, Frag8 (&fa)[4], Frag8 (&fb)[TN]) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             fa[i].u = *reinterpret_cast<const uint4*>(&stage[(a_base ^ (ks << 4)) + i * 32 * DM_BK]);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
             fb[j].u = *reinterpret_cast<const uint4*>(&stage[(b_base ^ (ks << 4)) + j * 32 * DM_BK]);
     };
-    auto multiply = [&](const Frag8 (&fa)[4], const Frag8 (&fb)[4]) __attribute__((always_inline)) {
+    auto multiply = [&](const Frag8 (&fa)[4], const Frag8 (&fb)[TN]) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < TN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i].v, fb[j].v, acc[i][j], 0, 0, 0);
     };
     const int nk = K / DM_BK;
-    Frag8 fa0[4], fb0[4], fa1[4], fb1[4];
+    Frag8 fa0[4], fb0[TN], fa1[4], fb1[TN];
     // K-step kt from `cur`: on entry set 0 holds its first sub-step and the loads of step kt+1
     // into `next` are in flight; on exit set 0 holds the first sub-step of kt+1 and the loads
     // of kt+2 into `cur` are in flight
@@ -588,10 +594,13 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_dma(const bf16_t* __restrict_
         load_step(cur, min(kt + 2, nk - 1));      // past the end: the last step again, into a stage nobody reads any more
         multiply(fa1, fb1);
 #pragma unroll
-        for (int q = 0; q < 16; ++q) {            // one product, one load, (one fragment read)
+        for (int q = 0; q < 4 * TN; ++q) {        // one product, (one fragment read,) one load or two
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (q < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            if (q < 4 + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (q < 8 - 2 * TN)
+                __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+            else
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -613,10 +622,11 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_dma(const bf16_t* __restrict_
     __syncthreads();                                   // every wave is done with the operands in LDS
     constexpr int EP_LD = 136;
     float* staged = reinterpret_cast<float*>((wave & 2) ? stage1 : stage0) + (wave & 1) * (32 * EP_LD);
-    const int out_col = (lane & 31) * 4;               // of the wave's 128 columns
-    const int n = n0 + wn * 128 + out_col;
+    const int out_col = (lane & 31) * 4;               // of the wave's columns: lanes past them (narrow tiles) sit out
+    const bool lane_on = out_col < WN;
+    const int n = n0 + wn * WN + out_col;
     float bn[4] = {0.f, 0.f, 0.f, 0.f};
-    if (bias) {
+    if (bias && lane_on) {
 #pragma unroll
         for (int c = 0; c < 4; ++c)
             if (n + c < N) bn[c] = bias[n + c];
@@ -625,17 +635,18 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_dma(const bf16_t* __restrict_
     const int out_n = swiglu ? N / 2 : N;              // columns of Y
     const int per_lane = swiglu ? 2 : 4;               // outputs a lane holds of a row
     // whole vectors: every row of this tile inside, the lane's columns inside, rows of Y aligned
-    const bool vectors = m0 + DM_T <= M && n0 + DM_T <= N && out_n % per_lane == 0 &&
+    const bool vectors = m0 + DM_T <= M && n0 + BN <= N && out_n % per_lane == 0 &&
                          ((uintptr_t)Y % (per_lane * sizeof(TOut))) == 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 staged[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * EP_LD + j * 32 + (lane & 31)] = acc[i][j][r];
 #pragma unroll 2
         for (int it = 0; it < 16; ++it) {
+            if (!lane_on) continue;
             const int row = it * 2 + (lane >> 5);
             const float4 v = *reinterpret_cast<const float4*>(&staged[row * EP_LD + out_col]);
             const int m = m0 + wm * 128 + i * 32 + row;
@@ -666,15 +677,57 @@ static bool dma_tile_takes(int m, int n, int k) {
     return k % (2 * DM_BK) == 0 && (long long)m * k < (1LL << 31) && (long long)n * k < (1LL << 31);
 }
 
+// Which width of the four-wave tile (TN = 4, 3, 2: 256, 192, 128 weight rows) and how many slices
+// of K suit a product of many rows; tn = 0: none (too few blocks to keep the CUs busy, or a K the
+// kernel does not take). Blocks run in rounds of one per CU, so what counts is how many rounds a
+// choice needs and how long its blocks take: measured on this machine, a K-step of 64 takes a
+// block 0.25 + 0.18 TN us, and a block's beginning and end (first loads, the tile's way out)
+// 10 + 6 TN us; a slice beyond the first costs its consumer one more pass over rows x width of
+// float32. A narrower tile reads more operand bytes per product, which timing with warm caches
+// does not show: with operands beyond what the caches hold (48 MB here) a K-step was measured 30%
+// slower per 64 weight rows less than 256, inside the model, where weights come from HBM.
+// `fixed_slices` > 0: the caller has decided (1: its consumer cannot add slices).
+struct DmaPlan {
+    int tn, slices;
+};
+static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
+    DmaPlan best{0, fixed_slices > 0 ? fixed_slices : 1};
+    if (m <= 64 || !dma_tile_takes(m, n, k)) return best;
+    const long long tiles_m = (m + DM_T - 1) / DM_T;
+    double best_cost = 0.0;
+    const bool cold = ((double)m + n) * k * 2.0 > 48e6;
+    for (int slices = 1; slices <= 4; slices *= 2) {
+        if (fixed_slices > 0 && slices != fixed_slices) continue;
+        if (k % (128 * slices) != 0 || (slices > 1 && k / slices < 1024)) continue;
+        for (int tn = 4; tn >= 2; --tn) {
+            const long long blocks = tiles_m * ((n + 64 * tn - 1) / (64 * tn)) * slices;
+            if (blocks < 160) continue;
+            const long long rounds = (blocks + 255) / 256;
+            const double step = (0.25 + 0.18 * tn) * (cold ? 1.0 + 0.3 * (4 - tn) : 1.0);
+            const double cost = rounds * (k / slices / 64 * step + 10.0 + 6.0 * tn) +
+                                (slices - 1) * ((double)m * n * 8.0 / 5e6);
+            if (best.tn == 0 || cost < best_cost) {
+                best = DmaPlan{tn, slices};
+                best_cost = cost;
+            }
+        }
+    }
+    return best;
+}
+
 // `slices` must leave every slice a multiple of 128 of K (dma_tile_takes(m, n, k / slices) and k % slices == 0)
 template <typename TOut>
 static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
-                      int slices, hipStream_t s) {
-    const int tiles_m = (m + DM_T - 1) / DM_T, tiles_n = (n + DM_T - 1) / DM_T;
+                      int tn, int slices, hipStream_t s) {
+    const int tiles_m = (m + DM_T - 1) / DM_T, tiles_n = (n + 64 * tn - 1) / (64 * tn);
     const long long total = (long long)tiles_m * tiles_n;
-    const unsigned blocks = (unsigned)(((total + N_XCD - 1) / N_XCD) * N_XCD);
-    k_gemm_bf16_dma<TOut><<<dim3(blocks, (unsigned)slices), 256, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m,
-                                                                        tiles_n, epilogue);
+    const dim3 grid((unsigned)(((total + N_XCD - 1) / N_XCD) * N_XCD), (unsigned)slices);
+    if (tn == 4)
+        k_gemm_bf16_dma<TOut, 4><<<grid, 256, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
+    else if (tn == 3)
+        k_gemm_bf16_dma<TOut, 3><<<grid, 256, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
+    else
+        k_gemm_bf16_dma<TOut, 2><<<grid, 256, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
     return launch_status();
 }
 
@@ -990,16 +1043,6 @@ static int stream_waves(int m, int n, int k) {
     return 0;
 }
 
-// A product of many rows whose 256x256 tiles fill a quarter of the CUs or fewer, with a long K:
-// four slices of K (2048 or more each) on the four-wave tile kernel give every CU a block.
-// Measured at 2048 x 2048 x 8192: 75 us against 94 us for the 128x128 tiles in two slices.
-static int dma_slices(int m, int n, int k) {
-    const long long tiles = (long long)((m + 255) / 256) * ((n + 255) / 256);
-    if (m > 64 && tiles * 4 <= 256 && tiles * 4 >= 160 && k % (4 * 128) == 0 && k / 4 >= 2048 && dma_tile_takes(m, n, k))
-        return 4;
-    return 0;
-}
-
 // A slice's length is rounded up to the kernel's step along K; with a ragged K that can leave the
 // last slices empty. The consumer adds every slice it was promised: fewer slices then, all of
 // them non-empty.
@@ -1019,7 +1062,8 @@ static int whole_slices(int slices, int k, int step) {
 extern "C" int imparo_gemm_slices(int m, int n, int k, int dtype) {
     if (dtype != IMPARO_BF16) return 1;
     if (m > 64) {
-        if (dma_slices(m, n, k)) return dma_slices(m, n, k);
+        const DmaPlan plan = dma_plan(m, n, k, 0);
+        if (plan.tn) return plan.slices;
         // many rows: with about one tile of 128x128 per CU or fewer, a block has a CU to itself and
         // nothing hides its waits; slices of K (at least 1024 each, at most 4) multiply the blocks
         const long long tiles = (long long)((m + BG_BM - 1) / BG_BM) * ((n + BG_BN - 1) / BG_BN);
@@ -1237,14 +1281,16 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
     } else {
         // `force` 256: the 256x256 tile on eight waves; 258: 256x256 on four waves with loads
         // straight into LDS (for measurements); otherwise by shape
-        if (slices == 1 && force == 0 && big_tile_pays(m, n, k) && dma_tile_takes(m, n, k))
-            return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, 1, s);
-        if (slices > 1 && force == 0 && slices == dma_slices(m, n, k))
-            return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, slices, s);
+        if (force == 0) {
+            const DmaPlan plan = dma_plan(m, n, k, slices);
+            if (plan.tn) return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, plan.tn, slices, s);
+        }
         if (slices == 1 && (force == 256 || (force == 0 && big_tile_pays(m, n, k))))
             return launch_big<TOut, 2, 4, 4, 2>(x, w, bias, y, m, n, k, epilogue, s);
-        if (force == 258 && k % slices == 0 && dma_tile_takes(m, n, k / slices) && dma_tile_takes(m, n, k))
-            return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, slices, s);
+        // 258: the four-wave tile 256 wide; 262, 263: 128 and 192 wide
+        if ((force == 258 || force == 262 || force == 263) && k % slices == 0 && dma_tile_takes(m, n, k / slices) &&
+            dma_tile_takes(m, n, k))
+            return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, force == 258 ? 4 : force - 260, slices, s);
         const int tiles_m = (m + BG_BM - 1) / BG_BM, tiles_n = (n + BG_BN - 1) / BG_BN;
         const long long total = (long long)tiles_m * tiles_n;
         if (total > 0x7fffff00LL) return IMPARO_BAD_ARGUMENT;

@@ -140,12 +140,13 @@ def test_gemm_with_many_weight_rows(m, k):
     assert (act.cpu().double() - ref).abs().max() <= 1e-6 * math.sqrt(k) * y.abs().max() * max(1.0, y.abs().max().item())
 
 
-@pytest.mark.parametrize("k", [256, 200, 1152])
-def test_gemm_with_large_tiles(k):
-    """Enough 256x256 tiles (160 or more) for the large-tile kernels: K a multiple of 128 goes to
-    the four-wave kernel that loads straight into LDS, another K to the eight-wave one. Edges in
-    both directions, an odd number of column pairs, a bias, both epilogues and output types."""
-    m, n = 2600, 3900 + 2 * (k % 3)
+@pytest.mark.parametrize("m,n,k", [(2600, 3900, 256), (2600, 3904, 1152), (3900, 4002, 384), (1500, 3900, 640),
+                                   (2600, 3904, 200)])
+def test_gemm_with_large_tiles(m, n, k):
+    """Enough tiles (160 or more) for the large-tile kernels: K a multiple of 128 goes to the
+    four-wave kernel that loads straight into LDS, 256 rows by 192 (11 x 21 tiles), 256 (16 x 16)
+    or 128 (6 x 31) weight rows, whichever fills the CUs best; another K to the eight-wave one.
+    Edges in both directions, an odd number of column pairs, a bias, both epilogues and output types."""
     x, w, b = rnd(m, k, seed=1, scale=0.5).to(torch.bfloat16), rnd(n, k, seed=2, scale=0.3).to(torch.bfloat16), rnd(n, seed=3)
     y = x.float() @ w.float().t() + b                       # float32 on the CPU: products exact, sums to 1e-6 sqrt(k)
     bound = 1e-6 * math.sqrt(k) * float(y.abs().max())
@@ -164,19 +165,20 @@ def test_gemm_with_large_tiles(k):
     assert torch.equal(outb.cpu(), out.cpu().to(torch.bfloat16))
 
 
-def test_gemm_with_large_tiles_in_slices_of_k():
-    """Few 256x256 tiles and a long K: four slices of K on the large tiles, one block per CU."""
-    m, n, k = 1900, 2000, 8192
-    assert ops().gemm_slices(m, n, k, torch.bfloat16) == 4
-    assert ops().gemm_slices(m, n, 4096, torch.bfloat16) == 2          # shorter K: the 128x128 tiles' rule
+@pytest.mark.parametrize("m,n,k,slices", [(1900, 2000, 8192, 4), (1000, 2000, 8192, 4), (1900, 2100, 4096, 2),
+                                          (1900, 2000, 2048, 2)])
+def test_gemm_with_large_tiles_in_slices_of_k(m, n, k, slices):
+    """Few tiles and a long K: slices of K on the large tiles, as many as give one block per CU."""
+    assert ops().gemm_slices(m, n, k, torch.bfloat16) == slices
     x, w, b = rnd(m, k, seed=1, scale=0.5).to(torch.bfloat16), rnd(n, k, seed=2, scale=0.3).to(torch.bfloat16), rnd(n, seed=3)
     y = x.float() @ w.float().t() + b
-    out = torch.full((4, m, n), float("nan"), device=DEV)
+    out = torch.full((slices, m, n), float("nan"), device=DEV)
     ops().gemm(x.to(DEV), w.to(DEV), out, bias=b.to(DEV))
     assert (out.cpu().sum(0) - y).abs().max() <= 4e-6 * math.sqrt(k) * float(y.abs().max())
     # each slice is its own range of K; the bias rides on the first
-    part = x[:, 2048:4096].float() @ w[:, 2048:4096].float().t()
-    assert (out[1].cpu() - part).abs().max() <= 4e-6 * math.sqrt(2048) * float(part.abs().max())
+    per = k // slices
+    part = x[:, per:2 * per].float() @ w[:, per:2 * per].float().t()
+    assert (out[1].cpu() - part).abs().max() <= 4e-6 * math.sqrt(per) * float(part.abs().max())
 
 
 def test_gemm_refuses_what_it_cannot_take():
