@@ -234,8 +234,12 @@ static void launch_rope_token(const float* qkv, const float* q_weight, const flo
 #undef ROPE_TOKEN
 }
 
-// From this many tokens on a launch takes the kernel with a block per token
-#define ROPE_TOKEN_KERNEL_FROM 32
+// From this many tokens on a launch takes the kernel with a block per token: its table of sines
+// and cosines costs each block a fixed 10 us or so, which the kernel with a wave per head passes
+// at about 400 tokens (40 heads of 64: 8 us at 256 tokens, 13 at 512, 43 at 2,048 against 22)
+#ifndef ROPE_TOKEN_KERNEL_FROM
+#define ROPE_TOKEN_KERNEL_FROM 400
+#endif
 
 extern "C" int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight, const float* k_weight, float eps,
                                          const float* inv_freq, int n_freq,

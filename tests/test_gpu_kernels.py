@@ -286,42 +286,42 @@ def test_qk_norm_rope_store(H, Hk, D, rot, page_size, vt):
 @pytest.mark.parametrize("H,Hk,D,rot", [(4, 2, 16, 16), (5, 1, 64, 64), (6, 3, 96, 32), (3, 1, 144, 144), (2, 2, 272, 0)])
 @pytest.mark.parametrize("vt", [False, True])
 def test_qk_norm_rope_store_many_tokens(H, Hk, D, rot, vt):
-    """From 32 tokens on a launch takes the kernel with a block per token. A token's results are the
+    """From 400 tokens on a launch takes the kernel with a block per token. A token's results are the
     same bits whichever kernel it met (the same tokens again, a few at a time), and right."""
-    segments, page_size, n_pages = [(0, 70), (5, 41)], 16, 12
-    tables = [[3, 1, 7, 9, 11], [0, 2, 4]]
+    segments, page_size, n_pages = [(0, 270), (5, 141)], 16, 30
+    tables = [[3, 1, 7, 9, 11, 29, 28, 13, 15, 17, 19, 21, 23, 25, 27, 5, 6], [0, 2, 4, 8, 10, 12, 14, 16, 18, 20]]
     for dtype in (torch.float32, torch.bfloat16):
-        qkv = rnd(111, (H + 2 * Hk) * D, seed=D).to(DEV)
+        qkv = rnd(411, (H + 2 * Hk) * D, seed=D).to(DEV)
         qw, kw = (1 + 0.1 * rnd(D, seed=1)).to(DEV), (1 + 0.1 * rnd(D, seed=2)).to(DEV)
         inv = None
         if rot:
             i = np.arange(rot // 2, dtype=np.float32)
             inv = torch.from_numpy(np.power(np.float32(1e6), (np.float32(-2.0) * i / np.float32(rot))).astype(np.float32)).to(DEV)
         results = []
-        for step in (111, 7):
+        for step in (411, 7):
             ctx = hand_context(segments, page_size, n_pages, dtype, DEV, kv_sites={0: (Hk, D)}, tables=tables,
                                v_transposed=vt)
             k_cache, v_cache, table = ctx.kv(0)
-            q_out = torch.empty(111, H, D, dtype=dtype, device=DEV)
-            for t0 in range(0, 111, step):
-                t1 = min(111, t0 + step)
+            q_out = torch.empty(411, H, D, dtype=dtype, device=DEV)
+            for t0 in range(0, 411, step):
+                t1 = min(411, t0 + step)
                 ops().qk_norm_rope_store(qkv[t0:t1], qw, kw, 1e-6, inv, ctx.positions[t0:t1], ctx.row_of_token[t0:t1],
                                          table, page_size, q_out[t0:t1], k_cache, v_cache, H, Hk, D, v_transposed=vt)
             results.append((q_out.cpu(), k_cache.cpu().clone(), v_cache.cpu().clone()))
         for a, b in zip(*results):
             assert torch.equal(a, b)
         positions = ctx.positions.cpu().tolist()
-        q = qkv.cpu()[:, :H * D].reshape(111, H, D)
+        q = qkv.cpu()[:, :H * D].reshape(411, H, D)
         q_ref = P.rms_norm(q, qw.cpu(), 1e-6)
         if rot:
             q_ref = P.rope_neox(q_ref, positions, 1e6, rot)
         tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -7)
         torch.testing.assert_close(results[0][0].float(), q_ref, **tol)
-        k = qkv.cpu()[:, H * D:(H + Hk) * D].reshape(111, Hk, D)
+        k = qkv.cpu()[:, H * D:(H + Hk) * D].reshape(411, Hk, D)
         k_ref = P.rms_norm(k, kw.cpu(), 1e-6)
         if rot:
             k_ref = P.rope_neox(k_ref, positions, 1e6, rot)
-        v = qkv.cpu()[:, (H + Hk) * D:].reshape(111, Hk, D)
+        v = qkv.cpu()[:, (H + Hk) * D:].reshape(411, Hk, D)
         kc, vc = results[0][1].float(), results[0][2].float()
         if vt:
             vc = vc.transpose(2, 3)
