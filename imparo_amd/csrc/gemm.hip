@@ -1059,8 +1059,12 @@ static int whole_slices(int slices, int k, int step) {
 // with few rows gives too few blocks to keep the memory system busy otherwise (one CU draws
 // about 50 GB/s at best, so it takes all of them): the measured optimum, with cold weights,
 // is about 256 blocks, with at least 512 of K per slice and at most 8 slices.
+static int g_force_few_row_kernel = 0;
+static int g_force_slices = 0;      // set by imparo_gemm_force_kernel, for measurements
+
 extern "C" int imparo_gemm_slices(int m, int n, int k, int dtype) {
     if (dtype != IMPARO_BF16) return 1;
+    if (g_force_slices) return g_force_slices;
     if (m > 64) {
         const DmaPlan plan = dma_plan(m, n, k, 0);
         if (plan.tn) return plan.slices;
@@ -1302,8 +1306,6 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
     return launch_status();
 }
 
-static int g_force_few_row_kernel = 0;
-static int g_force_slices = 0;
 
 // For measurements only: 0 lets the library choose the kernel, 1 forces the K-split kernel,
 // 2, 4 or 8 the shared-activation kernel with that many waves, 256/258 the large tiles;
@@ -1318,7 +1320,7 @@ extern "C" int imparo_gemm(const void* x, const void* w, const float* bias, void
     if (!x || !w || !y || m < 0 || n <= 0 || k <= 0) return IMPARO_BAD_ARGUMENT;
     if (slices < 1) return IMPARO_BAD_ARGUMENT;
     // slices: only what imparo_gemm_slices allows, float32 out, no epilogue that is not linear
-    const int slices_ok = g_force_slices ? g_force_slices : imparo_gemm_slices(m, n, k, dtype);
+    const int slices_ok = imparo_gemm_slices(m, n, k, dtype);
     if (slices > 1 && (slices != slices_ok || out_dtype != IMPARO_F32 || epilogue != EPI_NONE))
         return IMPARO_BAD_ARGUMENT;
     if (epilogue != EPI_NONE && epilogue != EPI_SWIGLU) return IMPARO_BAD_ARGUMENT;

@@ -94,10 +94,11 @@ class _DecodeGraph:
         self.meta: Optional[torch.Tensor] = None
         self.workspace: Optional[Workspace] = None
         self.logits: Optional[torch.Tensor] = None
-        self.seen = 0
+        self.last_used = 0
 
 
 TABLE_BUCKET = 8     # captured steps round their block-table width up to this many pages
+MAX_GRAPHS = 96      # captured batch shapes kept; beyond that the one unused for longest goes
 
 
 class Engine:
@@ -156,7 +157,8 @@ class Engine:
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Runs one batch. Returns float32 logits [wanted, vocab] on the
         device, in the order of the entries and of each entry's `want`, or
-        None when nothing is wanted."""
+        None when nothing is wanted. The tensor is the engine's: a later step
+        may write its own logits there, so use it (or copy it) before the next."""
         entries = list(entries)
         if not entries:
             return None
@@ -222,13 +224,17 @@ class Engine:
         batch shape is captured when it first comes and replayed from then on."""
         width = -(-batch.widest // TABLE_BUCKET) * TABLE_BUCKET
         key = (len(entries), width)
-        g = self._graphs.setdefault(key, _DecodeGraph())
-        g.seen += 1
         if not self._decode_code_loaded:
             self._decode_code_loaded = True
             ctx, token_ids, want_rows = self._pack(batch)
             with ops.on_current_stream():
                 return self.model.forward(ctx, token_ids, want_rows)
+        g = self._graphs.get(key)
+        if g is None:
+            if len(self._graphs) >= MAX_GRAPHS:      # each holds a workspace and a logits buffer
+                del self._graphs[min(self._graphs, key=lambda k: self._graphs[k].last_used)]
+            g = self._graphs[key] = _DecodeGraph()
+        g.last_used = self.steps_run
         if g.graph is None:
             g.workspace = Workspace(self.device)
             # the capture fixes grid sizes: they are sized for the widest context the tables can hold

@@ -245,6 +245,31 @@ def test_captured_decode_steps_equal_launched_ones(zoo, dtype):
     check_logits(runs[0][0:1], ref[len(prompts[0]) - 30:len(prompts[0]) - 29], dtype, "first decoded row")
 
 
+def test_captured_steps_are_kept_up_to_a_limit(zoo, monkeypatch):
+    """More batch shapes than the engine keeps captures for: the one unused for longest is dropped
+    and captured again when it comes back; every step equals the launched one."""
+    from imparo_amd.engine import StepEntry
+    import imparo_amd.engine.engine as engine_module
+    monkeypatch.setattr(engine_module, "MAX_GRAPHS", 2)
+    V = vocab_of(zoo, "A")
+    prompts = [prompt_tokens(V, 30 + i, 500 + i) for i in range(3)]
+    runs = []
+    for use_graphs in (True, False):
+        eng = make_engine(zoo[0]["A"], "bfloat16", page_size=16, max_tokens=1024, use_graphs=use_graphs)
+        out = []
+        for i in range(3):
+            eng.step([StepEntry(f"r{i}", prompts[i][:10], [])])
+        for s in range(10, 30):
+            rows = (3, 2, 1, 3, 1)[s % 5]            # three shapes in turn with room for two
+            out.append(eng.step([StepEntry(f"r{i}", [prompts[i][s]], [0]) for i in range(rows)]).cpu().clone())
+            for i in range(rows, 3):                 # the others keep pace in a step of their own
+                eng.step([StepEntry(f"r{i}", [prompts[i][s]], [])])
+        if use_graphs:
+            assert len(eng._graphs) == 2
+        runs.append(torch.cat(out))
+    assert torch.equal(runs[0], runs[1])
+
+
 def batch_r2(prompts, s):
     from imparo_amd.engine import StepEntry
     return StepEntry("r2", [prompts[2][len(prompts[2]) - 30 + s]], [0])
