@@ -457,10 +457,12 @@ static int launch_big(const bf16_t* x, const bf16_t* w, const float* bias, TOut*
 }
 
 // ------------------------------------------------------------------ bfloat16, many rows, loads straight into LDS
-// A 256x256 tile on four waves, one per SIMD, each with 128x128 of it (4x4 MFMA tiles of
-// 32x32, 256 accumulator registers): two fragments read from LDS per four products, half of
-// what the eight-wave kernel above reads. That only fits the register file because the
-// operands never pass through registers on their way in: global_load_lds writes 16 bytes per
+// A tile of 256 activation rows by 256, 192 or 128 weight rows. The 256 and the 128 wide tile
+// take eight waves, two per SIMD, each with 128 rows by 64 or 32 (4x2 or 4x1 MFMA tiles of 32x32,
+// 128 or 64 accumulator registers), so that one's products run while the other waits or writes
+// its results (12% faster than four waves of 128x128 on the gate/up product at 2,048 rows, 5 to
+// 15% on the narrow tile); the 192 wide tile four waves of 128 by 96, one per SIMD. The operands never pass through registers
+// on their way in: global_load_lds writes 16 bytes per
 // lane straight into LDS, a wave's 64 lanes to 1 KB in a row. LDS rows are the 128 bytes of
 // a K-step without padding, so the eight 16-byte pieces of row r are stored in the order
 // piece ^ swz(r), swz(r) = (r & 7) ^ ((r >> 3) & 1): the loading lane picks its global piece
@@ -494,16 +496,20 @@ __device__ __forceinline__ void load_to_lds(const bf16_t* src, bf16_t* dst_wave_
                                      (void __attribute__((address_space(3)))*)dst_wave_uniform, 16, 0, 0);
 }
 
-// TN: MFMA tiles across a wave's part of the weight rows: the block's tile is 256 activation rows
-// x 64 TN weight rows (256, 192 or 128), chosen by the launcher so that the blocks come out in
-// whole rounds of the CUs.
-template <typename TOut, int TN>
-__global__ __launch_bounds__(256) void k_gemm_bf16_dma(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
-                                                       const float* __restrict__ bias, TOut* __restrict__ Y,
-                                                       int M, int N, int K_all, int k_per, int tiles_m, int tiles_n,
-                                                       int epilogue) {
-    constexpr int BN = 64 * TN;                        // weight rows of the block's tile
-    constexpr int WN = 32 * TN;                        // of one wave's part
+// TN: MFMA tiles across a wave's part of the weight rows. The launcher chooses the tile's width so
+// that the blocks come out in whole rounds of the CUs.
+// NWN: waves across the weight rows (2: four waves, one per SIMD; 4: eight waves, two per SIMD, each
+// with half the accumulators, so that one's products run while the other waits).
+template <typename TOut, int TN, int NWN>
+__global__ __launch_bounds__(128 * NWN) void k_gemm_bf16_dma(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+                                                             const float* __restrict__ bias, TOut* __restrict__ Y,
+                                                             int M, int N, int K_all, int k_per, int tiles_m,
+                                                             int tiles_n, int epilogue) {
+    constexpr int NW = 2 * NWN;                        // waves of the block
+    constexpr int WN = 32 * TN;                        // weight rows of one wave's part
+    constexpr int BN = NWN * WN;                       // of the block's tile
+    constexpr int LX = DM_T / (8 * NW), LW = BN / (8 * NW);   // load instructions per wave and K-step
+    static_assert(BN % (8 * NW) == 0, "the waves share the tile's rows evenly");
     __shared__ __attribute__((aligned(1024))) bf16_t stage0[(DM_T + BN) * DM_BK];   // X rows, then W rows
     __shared__ __attribute__((aligned(1024))) bf16_t stage1[(DM_T + BN) * DM_BK];
     const int total = tiles_m * tiles_n;
@@ -526,24 +532,24 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_dma(const bf16_t* __restrict_
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    // loading: instruction j of a wave fills rows j*32 + wave*8 .. +7; lane -> row lane/8, slot lane%8
+    const int wm = wave / NWN, wn = wave % NWN;
+    // loading: instruction j of a wave fills rows j*8*NW + wave*8 .. +7; lane -> row lane/8, slot lane%8
     const int load_row = wave * 8 + (lane >> 3);
     const int load_piece = (lane & 7) ^ (lane >> 3) ^ (wave & 1);          // lane%8 ^ swz(row)
-    unsigned off_x[8], off_w[2 * TN];
+    unsigned off_x[LX], off_w[LW];
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-        off_x[j] = (unsigned)min(m0 + j * 32 + load_row, M - 1) * (unsigned)K_all + load_piece * 8;
+    for (int j = 0; j < LX; ++j)
+        off_x[j] = (unsigned)min(m0 + j * 8 * NW + load_row, M - 1) * (unsigned)K_all + load_piece * 8;
 #pragma unroll
-    for (int j = 0; j < 2 * TN; ++j)
-        off_w[j] = (unsigned)min(n0 + j * 32 + load_row, N - 1) * (unsigned)K_all + load_piece * 8;
+    for (int j = 0; j < LW; ++j)
+        off_w[j] = (unsigned)min(n0 + j * 8 * NW + load_row, N - 1) * (unsigned)K_all + load_piece * 8;
     auto load_step = [&](bf16_t* stage, int kt) __attribute__((always_inline)) {
         const bf16_t* xk = X + (size_t)kt * DM_BK;
         const bf16_t* wk = W + (size_t)kt * DM_BK;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) load_to_lds(xk + off_x[j], stage + (j * 32 + wave * 8) * DM_BK);
+        for (int j = 0; j < LX; ++j) load_to_lds(xk + off_x[j], stage + (j * 8 * NW + wave * 8) * DM_BK);
 #pragma unroll
-        for (int j = 0; j < 2 * TN; ++j) load_to_lds(wk + off_w[j], stage + (DM_T + j * 32 + wave * 8) * DM_BK);
+        for (int j = 0; j < LW; ++j) load_to_lds(wk + off_w[j], stage + (DM_T + j * 8 * NW + wave * 8) * DM_BK);
     };
     // fragments: lane holds row lane%32, K-half lane/32 of a 32x16 piece; sub-step ks is pieces 2ks, 2ks+1
     const int frag_row = lane & 31;
@@ -597,9 +603,9 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_dma(const bf16_t* __restrict_
         for (int q = 0; q < 4 * TN; ++q) {        // one product, (one fragment read,) one load or two
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             if (q < 4 + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            if (q < 8 - 2 * TN)
+            if (q < LX + LW - 4 * TN)
                 __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
-            else
+            else if (q < LX + LW)
                 __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -620,9 +626,11 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_dma(const bf16_t* __restrict_
     // stores. A staged row is 136 floats: the two rows a store instruction touches, 4 apart,
     // fall on disjoint banks. Each wave has a region of its own, so no barrier between passes.
     __syncthreads();                                   // every wave is done with the operands in LDS
-    constexpr int EP_LD = 136;
-    float* staged = reinterpret_cast<float*>((wave & 2) ? stage1 : stage0) + (wave & 1) * (32 * EP_LD);
-    const int out_col = (lane & 31) * 4;               // of the wave's columns: lanes past them (narrow tiles) sit out
+    constexpr int EP_LD = NWN == 2 ? 136 : WN + 8;
+    constexpr int LPR = (NWN == 2 || 64 % (WN / 4)) ? 32 : WN / 4;   // lanes to a staged row
+    static_assert((4 * EP_LD) % 64 == 32 && NW / 2 * 32 * EP_LD * 4 <= (DM_T + BN) * DM_BK * 2, "staging layout");
+    float* staged = reinterpret_cast<float*>(wave >= NW / 2 ? stage1 : stage0) + (wave % (NW / 2)) * (32 * EP_LD);
+    const int out_col = (lane % LPR) * 4;              // of the wave's columns: lanes past them (narrow tiles) sit out
     const bool lane_on = out_col < WN;
     const int n = n0 + wn * WN + out_col;
     float bn[4] = {0.f, 0.f, 0.f, 0.f};
@@ -645,9 +653,9 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_dma(const bf16_t* __restrict_
             for (int r = 0; r < 16; ++r)
                 staged[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * EP_LD + j * 32 + (lane & 31)] = acc[i][j][r];
 #pragma unroll 2
-        for (int it = 0; it < 16; ++it) {
+        for (int it = 0; it < 32 * LPR / 64; ++it) {
             if (!lane_on) continue;
-            const int row = it * 2 + (lane >> 5);
+            const int row = it * (64 / LPR) + lane / LPR;
             const float4 v = *reinterpret_cast<const float4*>(&staged[row * EP_LD + out_col]);
             const int m = m0 + wm * 128 + i * 32 + row;
             float o[4] = {v.x + bn[0], v.y + bn[1], v.z + bn[2], v.w + bn[3]};
@@ -677,12 +685,12 @@ static bool dma_tile_takes(int m, int n, int k) {
     return k % (2 * DM_BK) == 0 && (long long)m * k < (1LL << 31) && (long long)n * k < (1LL << 31);
 }
 
-// Which width of the four-wave tile (TN = 4, 3, 2: 256, 192, 128 weight rows) and how many slices
+// Which width of the tile (tn = 4, 3, 2: 256, 192, 128 weight rows) and how many slices
 // of K suit a product of many rows; tn = 0: none (too few blocks to keep the CUs busy, or a K the
 // kernel does not take). Blocks run in rounds of one per CU, so what counts is how many rounds a
 // choice needs and how long its blocks take: measured on this machine, a K-step of 64 takes a
-// block 0.25 + 0.18 TN us, and a block's beginning and end (first loads, the tile's way out)
-// 10 + 6 TN us; a slice beyond the first costs its consumer one more pass over rows x width of
+// block 0.25 + 0.18 tn us, and a block's beginning and end (first loads, the tile's way out)
+// 10 + 6 tn us (10 + 5 tn with eight waves); a slice beyond the first costs its consumer one more pass over rows x width of
 // float32. A narrower tile reads more operand bytes per product, which timing with warm caches
 // does not show: with operands beyond what the caches hold (48 MB here) a K-step was measured 30%
 // slower per 64 weight rows less than 256, inside the model, where weights come from HBM.
@@ -704,7 +712,8 @@ static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
             if (blocks < 160) continue;
             const long long rounds = (blocks + 255) / 256;
             const double step = (0.25 + 0.18 * tn) * (cold ? 1.0 + 0.3 * (4 - tn) : 1.0);
-            const double cost = rounds * (k / slices / 64 * step + 10.0 + 6.0 * tn) +
+            const double ends = tn == 3 ? 28.0 : 10.0 + 5.0 * tn;      // 256 and 128 wide: eight waves
+            const double cost = rounds * (k / slices / 64 * step + ends) +
                                 (slices - 1) * ((double)m * n * 8.0 / 5e6);
             if (best.tn == 0 || cost < best_cost) {
                 best = DmaPlan{tn, slices};
@@ -722,12 +731,12 @@ static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TOut*
     const int tiles_m = (m + DM_T - 1) / DM_T, tiles_n = (n + 64 * tn - 1) / (64 * tn);
     const long long total = (long long)tiles_m * tiles_n;
     const dim3 grid((unsigned)(((total + N_XCD - 1) / N_XCD) * N_XCD), (unsigned)slices);
-    if (tn == 4)
-        k_gemm_bf16_dma<TOut, 4><<<grid, 256, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
+    if (tn == 4)          // 256 wide: eight waves
+        k_gemm_bf16_dma<TOut, 2, 4><<<grid, 512, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
     else if (tn == 3)
-        k_gemm_bf16_dma<TOut, 3><<<grid, 256, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
-    else
-        k_gemm_bf16_dma<TOut, 2><<<grid, 256, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
+        k_gemm_bf16_dma<TOut, 3, 2><<<grid, 256, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
+    else                  // 128 wide: eight waves
+        k_gemm_bf16_dma<TOut, 1, 4><<<grid, 512, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
     return launch_status();
 }
 
@@ -1291,7 +1300,7 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
         }
         if (slices == 1 && (force == 256 || (force == 0 && big_tile_pays(m, n, k))))
             return launch_big<TOut, 2, 4, 4, 2>(x, w, bias, y, m, n, k, epilogue, s);
-        // 258: the four-wave tile 256 wide; 262, 263: 128 and 192 wide
+        // 258: the tile that loads straight into LDS, 256 wide; 262, 263: 128 and 192 wide
         if ((force == 258 || force == 262 || force == 263) && k % slices == 0 && dma_tile_takes(m, n, k / slices) &&
             dma_tile_takes(m, n, k))
             return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, force == 258 ? 4 : force - 260, slices, s);
