@@ -42,6 +42,32 @@ def step_all(engine, rid, tokens, cuts: Sequence[int]) -> torch.Tensor:
     return torch.cat(outs)
 
 
+def mixed_schedule(rng, lengths, max_live=4, sizes=(1, 1, 1, 2, 2, 3, 5, 9, 16, 40)):
+    """A schedule of steps: each step gives some live requests a portion or
+    one token. Returns [(step entries [(rid, lo, hi)], ends [rid])]."""
+    waiting = list(range(len(lengths)))
+    fed = {}
+    steps = []
+    while waiting or fed:
+        while waiting and len(fed) < max_live and (not fed or rng.random() < 0.6):
+            fed[waiting.pop(0)] = 0
+        entries, ends = [], []
+        for rid in sorted(fed):
+            if rng.random() < 0.25 and len(fed) > 1:
+                continue                                  # left out of this step, goes on later
+            left = lengths[rid] - fed[rid]
+            n = min(left, rng.choice(sizes))
+            entries.append((rid, fed[rid], fed[rid] + n))
+            fed[rid] += n
+            if fed[rid] == lengths[rid]:
+                ends.append(rid)
+        for rid in ends:
+            del fed[rid]
+        if entries:
+            steps.append((entries, ends))
+    return steps
+
+
 def hand_context(segments: Sequence[Tuple[int, int]], page_size: int, n_pages: int, dtype, device,
                  kv_sites: Dict[int, Tuple[int, int]] = None, fixed_sites: Dict[int, Tuple[int, ...]] = None,
                  n_slots: int = 8, tables: List[List[int]] = None, slots: List[int] = None,

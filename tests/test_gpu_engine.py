@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from conftest import prompt_tokens
-from gpu_helpers import make_engine, RefCache, step_all
+from gpu_helpers import make_engine, mixed_schedule, RefCache, step_all
 from tolerances import check_logits
 
 pytestmark = pytest.mark.gpu
@@ -94,32 +94,6 @@ def test_portions_of_changing_size(zoo, engines, name, dtype):
         check_logits(got, ref, dtype, f"{name} portions {cuts}", rel)
 
 
-def _mixed_schedule(rng, lengths, max_live=4):
-    """A schedule of steps: each step gives some live requests a portion or
-    one token. Returns [(step entries [(rid, lo, hi)], ends [rid])]."""
-    waiting = list(range(len(lengths)))
-    fed = {}
-    steps = []
-    while waiting or fed:
-        while waiting and len(fed) < max_live and (not fed or rng.random() < 0.6):
-            fed[waiting.pop(0)] = 0
-        entries, ends = [], []
-        for rid in sorted(fed):
-            if rng.random() < 0.25 and len(fed) > 1:
-                continue                                  # left out of this step, goes on later
-            left = lengths[rid] - fed[rid]
-            n = min(left, rng.choice([1, 1, 1, 2, 2, 3, 5, 9, 16, 40]))
-            entries.append((rid, fed[rid], fed[rid] + n))
-            fed[rid] += n
-            if fed[rid] == lengths[rid]:
-                ends.append(rid)
-        for rid in ends:
-            del fed[rid]
-        if entries:
-            steps.append((entries, ends))
-    return steps
-
-
 @pytest.mark.parametrize("name,dtype", CASES)
 def test_mixed_batches_with_pages_used_again(zoo, engines, name, dtype):
     from imparo_amd.engine import StepEntry
@@ -129,7 +103,7 @@ def test_mixed_batches_with_pages_used_again(zoo, engines, name, dtype):
     prompts = [prompt_tokens(V, n, 100 + i) for i, n in enumerate(lengths)]
     # pages of 8; four live requests of up to 121 tokens need at most 4*16 pages: 40 forces reuse
     eng = engines(name, dtype, page_size=8, max_tokens=40 * 8, max_requests=4)
-    steps = _mixed_schedule(rng, lengths)
+    steps = mixed_schedule(rng, lengths)
     got = {i: [] for i in range(len(lengths))}
     used = set()
     for entries, ends in steps:
