@@ -274,7 +274,7 @@ def main() -> int:
                   + args.batch * (mean_ctx * nums["kv_bytes_per_token"] * elem / 2 + nums["conv_state_bytes"]))
     achieved = step_bytes / (dt / args.steps) / 1e9
     line = {
-        "metric": "decode tok/s (LFM2-1.2B shape, batch 8, context 4096)",
+        "metric": f"decode tok/s (LFM2-1.2B shape, batch {args.batch}, context {args.context})",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic token ids, random weights (seed 2)",
