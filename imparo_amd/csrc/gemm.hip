@@ -7,6 +7,8 @@
 // weight-streaming one with the K range split over the waves of a block for
 // few rows (decode).
 #include "common.h"
+
+#include <algorithm>
 #include "api.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -457,9 +459,9 @@ static int launch_big(const bf16_t* x, const bf16_t* w, const float* bias, TOut*
 }
 
 // ------------------------------------------------------------------ bfloat16, many rows, loads straight into LDS
-// A tile of 256 activation rows by 256, 192 or 128 weight rows. The 256 and the 128 wide tile
-// take eight waves, two per SIMD, each with 128 rows by 64 or 32 (4x2 or 4x1 MFMA tiles of 32x32,
-// 128 or 64 accumulator registers), so that one's products run while the other waits or writes
+// A tile of 256 or 128 activation rows by 256, 192 or 128 weight rows. The 256 and the 128 wide tile
+// take eight waves, two per SIMD, each with 128 (or 64) rows by 64 or 32 (4x2 or 4x1 MFMA tiles of 32x32,
+// 128 or 64 accumulator registers; half of that with 128 activation rows), so that one's products run while the other waits or writes
 // its results (12% faster than four waves of 128x128 on the gate/up product at 2,048 rows, 5 to
 // 15% on the narrow tile); the 192 wide tile four waves of 128 by 96, one per SIMD. The operands never pass through registers
 // on their way in: global_load_lds writes 16 bytes per
@@ -472,7 +474,6 @@ static int launch_big(const bf16_t* x, const bf16_t* w, const float* bias, TOut*
 // fragments of the next K-sub-step in flight while it multiplies (two register sets), and the
 // barrier of a K-step sits before the last sub-step's products, so the matrix pipe has
 // work queued while the waves meet. Needs K a multiple of 128 (two K-steps).
-#define DM_T 256       // tile rows of each operand
 #define DM_BK 64
 
 // Two (`pair`) or four outputs of one row in one store; the address is aligned to the store
@@ -500,7 +501,8 @@ __device__ __forceinline__ void load_to_lds(const bf16_t* src, bf16_t* dst_wave_
 // that the blocks come out in whole rounds of the CUs.
 // NWN: waves across the weight rows (2: four waves, one per SIMD; 4: eight waves, two per SIMD, each
 // with half the accumulators, so that one's products run while the other waits).
-template <typename TOut, int TN, int NWN>
+// TMI: MFMA tiles down a wave's part of the activation rows (4: the block takes 256 rows, 2: 128).
+template <typename TOut, int TMI, int TN, int NWN>
 __global__ __launch_bounds__(128 * NWN) void k_gemm_bf16_dma(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                              const float* __restrict__ bias, TOut* __restrict__ Y,
                                                              int M, int N, int K_all, int k_per, int tiles_m,
@@ -508,10 +510,12 @@ __global__ __launch_bounds__(128 * NWN) void k_gemm_bf16_dma(const bf16_t* __res
     constexpr int NW = 2 * NWN;                        // waves of the block
     constexpr int WN = 32 * TN;                        // weight rows of one wave's part
     constexpr int BN = NWN * WN;                       // of the block's tile
-    constexpr int LX = DM_T / (8 * NW), LW = BN / (8 * NW);   // load instructions per wave and K-step
-    static_assert(BN % (8 * NW) == 0, "the waves share the tile's rows evenly");
-    __shared__ __attribute__((aligned(1024))) bf16_t stage0[(DM_T + BN) * DM_BK];   // X rows, then W rows
-    __shared__ __attribute__((aligned(1024))) bf16_t stage1[(DM_T + BN) * DM_BK];
+    constexpr int WM = 32 * TMI;                       // activation rows of one wave's part
+    constexpr int BM = 2 * WM;                         // of the block's tile
+    constexpr int LX = BM / (8 * NW), LW = BN / (8 * NW);   // load instructions per wave and K-step
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "the waves share the tile's rows evenly");
+    __shared__ __attribute__((aligned(1024))) bf16_t stage0[(BM + BN) * DM_BK];   // X rows, then W rows
+    __shared__ __attribute__((aligned(1024))) bf16_t stage1[(BM + BN) * DM_BK];
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + N_XCD - 1) / N_XCD;
     const int logical = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;
@@ -521,7 +525,7 @@ __global__ __launch_bounds__(128 * NWN) void k_gemm_bf16_dma(const bf16_t* __res
     const int gsize = min(tiles_m - first_m, BG_GROUP_M);
     const int tile_m = first_m + (logical % per_group) % gsize;
     const int tile_n = (logical % per_group) / gsize;
-    const int m0 = tile_m * DM_T, n0 = tile_n * BN;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
     // slices of K (gridDim.y > 1): block (x, y) sums K range [y * k_per, (y+1) * k_per) into Y + y * M * N
     const int k_lo = blockIdx.y * k_per;
     const int K = min(K_all, k_lo + k_per) - k_lo;
@@ -549,37 +553,37 @@ __global__ __launch_bounds__(128 * NWN) void k_gemm_bf16_dma(const bf16_t* __res
 #pragma unroll
         for (int j = 0; j < LX; ++j) load_to_lds(xk + off_x[j], stage + (j * 8 * NW + wave * 8) * DM_BK);
 #pragma unroll
-        for (int j = 0; j < LW; ++j) load_to_lds(wk + off_w[j], stage + (DM_T + j * 8 * NW + wave * 8) * DM_BK);
+        for (int j = 0; j < LW; ++j) load_to_lds(wk + off_w[j], stage + (BM + j * 8 * NW + wave * 8) * DM_BK);
     };
     // fragments: lane holds row lane%32, K-half lane/32 of a 32x16 piece; sub-step ks is pieces 2ks, 2ks+1
     const int frag_row = lane & 31;
     const int swz = (frag_row & 7) ^ ((frag_row >> 3) & 1);
-    const int a_base = (wm * 128 + frag_row) * DM_BK + (((lane >> 5) ^ swz) << 3);
-    const int b_base = (DM_T + wn * WN + frag_row) * DM_BK + (((lane >> 5) ^ swz) << 3);
-    f32x16 acc[4][TN];
+    const int a_base = (wm * WM + frag_row) * DM_BK + (((lane >> 5) ^ swz) << 3);
+    const int b_base = (BM + wn * WN + frag_row) * DM_BK + (((lane >> 5) ^ swz) << 3);
+    f32x16 acc[TMI][TN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TMI; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    auto read = [&](const bf16_t* stage, int ks, Frag8 (&fa)[4], Frag8 (&fb)[TN]) __attribute__((always_inline)) {
+    auto read = [&](const bf16_t* stage, int ks, Frag8 (&fa)[TMI], Frag8 (&fb)[TN]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < TMI; ++i)
             fa[i].u = *reinterpret_cast<const uint4*>(&stage[(a_base ^ (ks << 4)) + i * 32 * DM_BK]);
 #pragma unroll
         for (int j = 0; j < TN; ++j)
             fb[j].u = *reinterpret_cast<const uint4*>(&stage[(b_base ^ (ks << 4)) + j * 32 * DM_BK]);
     };
-    auto multiply = [&](const Frag8 (&fa)[4], const Frag8 (&fb)[TN]) __attribute__((always_inline)) {
+    auto multiply = [&](const Frag8 (&fa)[TMI], const Frag8 (&fb)[TN]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < TMI; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i].v, fb[j].v, acc[i][j], 0, 0, 0);
     };
     const int nk = K / DM_BK;
-    Frag8 fa0[4], fb0[TN], fa1[4], fb1[TN];
+    Frag8 fa0[TMI], fb0[TN], fa1[TMI], fb1[TN];
     // K-step kt from `cur`: on entry set 0 holds its first sub-step and the loads of step kt+1
     // into `next` are in flight; on exit set 0 holds the first sub-step of kt+1 and the loads
     // of kt+2 into `cur` are in flight
@@ -600,10 +604,10 @@ __global__ __launch_bounds__(128 * NWN) void k_gemm_bf16_dma(const bf16_t* __res
         load_step(cur, min(kt + 2, nk - 1));      // past the end: the last step again, into a stage nobody reads any more
         multiply(fa1, fb1);
 #pragma unroll
-        for (int q = 0; q < 4 * TN; ++q) {        // one product, (one fragment read,) one load or two
+        for (int q = 0; q < TMI * TN; ++q) {        // one product, (one fragment read,) one load or two
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (q < 4 + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            if (q < LX + LW - 4 * TN)
+            if (q < TMI + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (q < LX + LW - TMI * TN)
                 __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
             else if (q < LX + LW)
                 __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
@@ -628,7 +632,7 @@ __global__ __launch_bounds__(128 * NWN) void k_gemm_bf16_dma(const bf16_t* __res
     __syncthreads();                                   // every wave is done with the operands in LDS
     constexpr int EP_LD = NWN == 2 ? 136 : WN + 8;
     constexpr int LPR = (NWN == 2 || 64 % (WN / 4)) ? 32 : WN / 4;   // lanes to a staged row
-    static_assert((4 * EP_LD) % 64 == 32 && NW / 2 * 32 * EP_LD * 4 <= (DM_T + BN) * DM_BK * 2, "staging layout");
+    static_assert((4 * EP_LD) % 64 == 32 && NW / 2 * 32 * EP_LD * 4 <= (BM + BN) * DM_BK * 2, "staging layout");
     float* staged = reinterpret_cast<float*>(wave >= NW / 2 ? stage1 : stage0) + (wave % (NW / 2)) * (32 * EP_LD);
     const int out_col = (lane % LPR) * 4;              // of the wave's columns: lanes past them (narrow tiles) sit out
     const bool lane_on = out_col < WN;
@@ -643,10 +647,10 @@ __global__ __launch_bounds__(128 * NWN) void k_gemm_bf16_dma(const bf16_t* __res
     const int out_n = swiglu ? N / 2 : N;              // columns of Y
     const int per_lane = swiglu ? 2 : 4;               // outputs a lane holds of a row
     // whole vectors: every row of this tile inside, the lane's columns inside, rows of Y aligned
-    const bool vectors = m0 + DM_T <= M && n0 + BN <= N && out_n % per_lane == 0 &&
+    const bool vectors = m0 + BM <= M && n0 + BN <= N && out_n % per_lane == 0 &&
                          ((uintptr_t)Y % (per_lane * sizeof(TOut))) == 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < TMI; ++i) {
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -657,7 +661,7 @@ __global__ __launch_bounds__(128 * NWN) void k_gemm_bf16_dma(const bf16_t* __res
             if (!lane_on) continue;
             const int row = it * (64 / LPR) + lane / LPR;
             const float4 v = *reinterpret_cast<const float4*>(&staged[row * EP_LD + out_col]);
-            const int m = m0 + wm * 128 + i * 32 + row;
+            const int m = m0 + wm * WM + i * 32 + row;
             float o[4] = {v.x + bn[0], v.y + bn[1], v.z + bn[2], v.w + bn[3]};
             if (swiglu) {
                 o[0] = silu_mul_fast(o[0], o[1]);
@@ -685,58 +689,80 @@ static bool dma_tile_takes(int m, int n, int k) {
     return k % (2 * DM_BK) == 0 && (long long)m * k < (1LL << 31) && (long long)n * k < (1LL << 31);
 }
 
-// Which width of the tile (tn = 4, 3, 2: 256, 192, 128 weight rows) and how many slices
-// of K suit a product of many rows; tn = 0: none (too few blocks to keep the CUs busy, or a K the
-// kernel does not take). Blocks run in rounds of one per CU, so what counts is how many rounds a
-// choice needs and how long its blocks take: measured on this machine, a K-step of 64 takes a
-// block 0.25 + 0.18 tn us, and a block's beginning and end (first loads, the tile's way out)
-// 10 + 6 tn us (10 + 5 tn with eight waves); a slice beyond the first costs its consumer one more pass over rows x width of
-// float32. A narrower tile reads more operand bytes per product, which timing with warm caches
-// does not show: with operands beyond what the caches hold (48 MB here) a K-step was measured 30%
-// slower per 64 weight rows less than 256, inside the model, where weights come from HBM.
+// Which tile (bm = 256 or 128 activation rows, tn = 4, 3, 2 for 256, 192, 128 weight rows; 192 with
+// bm 256 only) and how many slices of K suit a product of many rows; tn = 0: none (a K the kernel
+// does not take). A model of the time, fitted to this machine (it picks the fastest or one within
+// a few percent of it on every shape measured, 128 to 4,096 rows):
+//   - a block alone on its CU takes 0.11 us + 0.0155 us per MFMA of a SIMD for a K-step of 64
+//     (bm * bn / 1024 of them), and 5 us + 0.03 us per such MFMA for its beginning and end;
+//   - two blocks fit a CU where their stages take 80 KB or less each (the 128x128 tile), and a
+//     step then takes what the products of both take;
+//   - the more CUs are busy the slower each runs (clocks, L2): up to 45% with all 256, and more
+//     with small tiles, which read more operand bytes per product;
+//   - blocks run in rounds of what fits the chip at once; the operands have to come from memory
+//     once (5.5 TB/s) and the results have to go there (5 TB/s); a slice beyond the first costs
+//     its consumer one more pass over rows x width of float32.
 // `fixed_slices` > 0: the caller has decided (1: its consumer cannot add slices).
 struct DmaPlan {
-    int tn, slices;
+    int bm, tn, slices;
 };
 static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
-    DmaPlan best{0, fixed_slices > 0 ? fixed_slices : 1};
+    DmaPlan best{0, 0, fixed_slices > 0 ? fixed_slices : 1};
     if (m <= 64 || !dma_tile_takes(m, n, k)) return best;
-    const long long tiles_m = (m + DM_T - 1) / DM_T;
     double best_cost = 0.0;
-    const bool cold = ((double)m + n) * k * 2.0 > 48e6;
     for (int slices = 1; slices <= 4; slices *= 2) {
         if (fixed_slices > 0 && slices != fixed_slices) continue;
-        if (k % (128 * slices) != 0 || (slices > 1 && k / slices < 1024)) continue;
-        for (int tn = 4; tn >= 2; --tn) {
-            const long long blocks = tiles_m * ((n + 64 * tn - 1) / (64 * tn)) * slices;
-            if (blocks < 160) continue;
-            const long long rounds = (blocks + 255) / 256;
-            const double step = (0.25 + 0.18 * tn) * (cold ? 1.0 + 0.3 * (4 - tn) : 1.0);
-            const double ends = tn == 3 ? 28.0 : 10.0 + 5.0 * tn;      // 256 and 128 wide: eight waves
-            const double cost = rounds * (k / slices / 64 * step + ends) +
-                                (slices - 1) * ((double)m * n * 8.0 / 5e6);
-            if (best.tn == 0 || cost < best_cost) {
-                best = DmaPlan{tn, slices};
-                best_cost = cost;
+        if (k % (128 * slices) != 0 || (slices > 1 && k / slices < 512)) continue;
+        for (int bm = 256; bm >= 128; bm /= 2) {
+            for (int tn = 4; tn >= 2; --tn) {
+                if (tn == 3 && bm != 256) continue;
+                const int bn = 64 * tn;
+                const long long blocks = (long long)((m + bm - 1) / bm) * ((n + bn - 1) / bn) * slices;
+                const int at_once = 256 * ((bm + bn) * DM_BK * 2 * 2 <= 80 * 1024 ? 2 : 1);
+                const long long rounds = (blocks + at_once - 1) / at_once;
+                const long long per_round = (blocks + rounds - 1) / rounds;
+                const double cus = (double)std::min<long long>(256, per_round);
+                const double per_cu = (double)((per_round + (long long)cus - 1) / (long long)cus);
+                const double mfmas = bm * bn / 1024.0;
+                const double small = 1.0 + 0.1 * (256.0 / bm - 1.0) + 0.1 * (256.0 / bn - 1.0);
+                const double step = std::max(0.11 + 0.0155 * mfmas, per_cu * 0.0155 * mfmas) *
+                                    (1.0 + 0.45 * cus / 256.0 * small);
+                const double ends = 5.0 + 0.03 * mfmas;
+                const double from_memory = ((double)m + n) * k * 2.0 / 5.5e6;
+                const double cost = std::max(rounds * (k / slices / DM_BK * step + ends), from_memory + ends) +
+                                    (double)slices * m * n * 4.0 / 5e6 + (slices - 1) * ((double)m * n * 4.0 / 5e6);
+                if (best.tn == 0 || cost < best_cost) {
+                    best = DmaPlan{bm, tn, slices};
+                    best_cost = cost;
+                }
             }
         }
     }
     return best;
 }
 
-// `slices` must leave every slice a multiple of 128 of K (dma_tile_takes(m, n, k / slices) and k % slices == 0)
+// `slices` must leave every slice a multiple of 128 of K (dma_tile_takes(m, n, k / slices) and k % slices == 0).
+// bm: 256 or 128 activation rows to a tile; tn: 4, 3 (bm 256 only) or 2 for 256, 192 or 128 weight rows.
 template <typename TOut>
 static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
-                      int tn, int slices, hipStream_t s) {
-    const int tiles_m = (m + DM_T - 1) / DM_T, tiles_n = (n + 64 * tn - 1) / (64 * tn);
+                      int bm, int tn, int slices, hipStream_t s) {
+    const int tiles_m = (m + bm - 1) / bm, tiles_n = (n + 64 * tn - 1) / (64 * tn);
     const long long total = (long long)tiles_m * tiles_n;
     const dim3 grid((unsigned)(((total + N_XCD - 1) / N_XCD) * N_XCD), (unsigned)slices);
-    if (tn == 4)          // 256 wide: eight waves
-        k_gemm_bf16_dma<TOut, 2, 4><<<grid, 512, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
+#define DMA_GO(TMI, TN, NWN)                                                                                         \
+    k_gemm_bf16_dma<TOut, TMI, TN, NWN><<<grid, 128 * NWN, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m,     \
+                                                                   tiles_n, epilogue)
+    if (bm == 128 && tn == 4)
+        DMA_GO(2, 2, 4);
+    else if (bm == 128)
+        DMA_GO(2, 1, 4);
+    else if (tn == 4)     // 256 wide: eight waves
+        DMA_GO(4, 2, 4);
     else if (tn == 3)
-        k_gemm_bf16_dma<TOut, 3, 2><<<grid, 256, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
+        DMA_GO(4, 3, 2);
     else                  // 128 wide: eight waves
-        k_gemm_bf16_dma<TOut, 1, 4><<<grid, 512, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
+        DMA_GO(4, 1, 4);
+#undef DMA_GO
     return launch_status();
 }
 
@@ -1296,14 +1322,17 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
         // straight into LDS (for measurements); otherwise by shape
         if (force == 0) {
             const DmaPlan plan = dma_plan(m, n, k, slices);
-            if (plan.tn) return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, plan.tn, slices, s);
+            if (plan.tn) return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, plan.bm, plan.tn, slices, s);
         }
         if (slices == 1 && (force == 256 || (force == 0 && big_tile_pays(m, n, k))))
             return launch_big<TOut, 2, 4, 4, 2>(x, w, bias, y, m, n, k, epilogue, s);
         // 258: the tile that loads straight into LDS, 256 wide; 262, 263: 128 and 192 wide
         if ((force == 258 || force == 262 || force == 263) && k % slices == 0 && dma_tile_takes(m, n, k / slices) &&
             dma_tile_takes(m, n, k))
-            return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, force == 258 ? 4 : force - 260, slices, s);
+            return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, 256, force == 258 ? 4 : force - 260, slices, s);
+        // 358, 352: 128 activation rows to a tile, 256 and 128 wide
+        if ((force == 358 || force == 352) && k % slices == 0 && dma_tile_takes(m, n, k / slices) && dma_tile_takes(m, n, k))
+            return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, 128, force == 358 ? 4 : 2, slices, s);
         const int tiles_m = (m + BG_BM - 1) / BG_BM, tiles_n = (n + BG_BN - 1) / BG_BN;
         const long long total = (long long)tiles_m * tiles_n;
         if (total > 0x7fffff00LL) return IMPARO_BAD_ARGUMENT;

@@ -90,8 +90,9 @@ def test_gemm_in_slices_of_k_and_the_norm_that_adds_them(m):
     assert ops().gemm_slices(m, 2048, 2048, torch.bfloat16) == (2 if m <= 16 else 4)    # 128 or 64 blocks
     assert ops().gemm_slices(m, 8192, k, torch.bfloat16) == 1       # a weight with many rows fills the chip by itself
     assert ops().gemm_slices(m, n, k, torch.float32) == 1
-    # many rows and few tiles: the 128x128 kernel takes slices too (at least 1024 of K each, at most 4)
-    assert ops().gemm_slices(300, n, k, torch.bfloat16) == 4 and ops().gemm_slices(300, n, 2048, torch.bfloat16) == 2
+    # many rows and few tiles: the tile kernels take slices too, at most 4 (this K, no multiple of 128, goes to
+    # the one with register staging: at least 1024 of K each; K = 2048 to the one that loads into LDS: 512)
+    assert ops().gemm_slices(300, n, k, torch.bfloat16) == 4 and ops().gemm_slices(300, n, 2048, torch.bfloat16) == 4
     assert ops().gemm_slices(2048, 16384, 2048, torch.bfloat16) == 1
     x3 = rnd(300, k, seed=7).to(torch.bfloat16)
     out3 = torch.full((4, 300, n), float("nan"), device=DEV)
@@ -140,13 +141,25 @@ def test_gemm_with_many_weight_rows(m, k):
     assert (act.cpu().double() - ref).abs().max() <= 1e-6 * math.sqrt(k) * y.abs().max() * max(1.0, y.abs().max().item())
 
 
-@pytest.mark.parametrize("m,n,k", [(2600, 3900, 256), (2600, 3904, 1152), (3900, 4002, 384), (1500, 3900, 640),
-                                   (2600, 3904, 200)])
-def test_gemm_with_large_tiles(m, n, k):
-    """Enough tiles (160 or more) for the large-tile kernels: K a multiple of 128 goes to the
-    four-wave kernel that loads straight into LDS, 256 rows by 192 (11 x 21 tiles), 256 (16 x 16)
-    or 128 (6 x 31) weight rows, whichever fills the CUs best; another K to the eight-wave one.
-    Edges in both directions, an odd number of column pairs, a bias, both epilogues and output types."""
+@pytest.mark.parametrize("m,n,k,tile", [(2600, 3900, 256, 0), (2600, 3904, 1152, 0), (3900, 4002, 384, 0),
+                                        (1500, 3900, 640, 0), (2600, 3904, 200, 0), (70, 100, 128, 0),
+                                        (700, 1000, 384, 258), (700, 1000, 384, 262), (700, 1000, 384, 263),
+                                        (700, 1000, 384, 358), (700, 1000, 384, 352)])
+def test_gemm_with_large_tiles(m, n, k, tile):
+    """Many rows: K a multiple of 128 goes to the kernel that loads straight into LDS, with a tile
+    of 256 or 128 rows by 256, 192 or 128 weight rows, whichever its plan finds fastest (`tile`
+    other than 0 names one, through the library's switch for measurements, so that each is met);
+    another K to the tile kernels with register staging. Edges in both directions, an odd number
+    of column pairs, a bias, both epilogues and output types."""
+    from imparo_amd.kernels import library
+    library().imparo_gemm_force_kernel(tile)
+    try:
+        _large_tile_case(m, n, k)
+    finally:
+        library().imparo_gemm_force_kernel(0)
+
+
+def _large_tile_case(m, n, k):
     x, w, b = rnd(m, k, seed=1, scale=0.5).to(torch.bfloat16), rnd(n, k, seed=2, scale=0.3).to(torch.bfloat16), rnd(n, seed=3)
     y = x.float() @ w.float().t() + b                       # float32 on the CPU: products exact, sums to 1e-6 sqrt(k)
     bound = 1e-6 * math.sqrt(k) * float(y.abs().max())
@@ -165,8 +178,7 @@ def test_gemm_with_large_tiles(m, n, k):
     assert torch.equal(outb.cpu(), out.cpu().to(torch.bfloat16))
 
 
-@pytest.mark.parametrize("m,n,k,slices", [(1900, 2000, 8192, 4), (1000, 2000, 8192, 4), (1900, 2100, 4096, 2),
-                                          (1900, 2000, 2048, 2)])
+@pytest.mark.parametrize("m,n,k,slices", [(1900, 2000, 8192, 2), (1000, 2000, 8192, 4), (1900, 2100, 4096, 2)])
 def test_gemm_with_large_tiles_in_slices_of_k(m, n, k, slices):
     """Few tiles and a long K: slices of K on the large tiles, as many as give one block per CU."""
     assert ops().gemm_slices(m, n, k, torch.bfloat16) == slices
