@@ -699,6 +699,9 @@ static bool dma_tile_takes(int m, int n, int k) {
 //     step then takes what the products of both take;
 //   - the more CUs are busy the slower each runs (clocks, L2): up to 45% with all 256, and more
 //     with small tiles, which read more operand bytes per product;
+//   - with one or two tiles down the rows (a decode batch of 65 to 256 rows) every block meets its
+//     weights first, and cold: a K-step then takes 1 us whatever the tile (measured: 32 us for 32
+//     steps at 128 rows), so such products are cut into up to 8 slices, others into up to 4;
 //   - blocks run in rounds of what fits the chip at once; the operands have to come from memory
 //     once (5.5 TB/s) and the results have to go there (5 TB/s); a slice beyond the first costs
 //     its consumer one more pass over rows x width of float32.
@@ -710,14 +713,16 @@ static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
     DmaPlan best{0, 0, fixed_slices > 0 ? fixed_slices : 1};
     if (m <= 64 || !dma_tile_takes(m, n, k)) return best;
     double best_cost = 0.0;
-    for (int slices = 1; slices <= 4; slices *= 2) {
+    for (int slices = 1; slices <= 8; slices *= 2) {
         if (fixed_slices > 0 && slices != fixed_slices) continue;
         if (k % (128 * slices) != 0 || (slices > 1 && k / slices < 512)) continue;
         for (int bm = 256; bm >= 128; bm /= 2) {
+            const int tiles_m = (m + bm - 1) / bm;
+            if (slices > 4 && tiles_m > 2) continue;
             for (int tn = 4; tn >= 2; --tn) {
                 if (tn == 3 && bm != 256) continue;
                 const int bn = 64 * tn;
-                const long long blocks = (long long)((m + bm - 1) / bm) * ((n + bn - 1) / bn) * slices;
+                const long long blocks = (long long)tiles_m * ((n + bn - 1) / bn) * slices;
                 const int at_once = 256 * ((bm + bn) * DM_BK * 2 * 2 <= 80 * 1024 ? 2 : 1);
                 const long long rounds = (blocks + at_once - 1) / at_once;
                 const long long per_round = (blocks + rounds - 1) / rounds;
@@ -725,8 +730,9 @@ static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
                 const double per_cu = (double)((per_round + (long long)cus - 1) / (long long)cus);
                 const double mfmas = bm * bn / 1024.0;
                 const double small = 1.0 + 0.1 * (256.0 / bm - 1.0) + 0.1 * (256.0 / bn - 1.0);
-                const double step = std::max(0.11 + 0.0155 * mfmas, per_cu * 0.0155 * mfmas) *
-                                    (1.0 + 0.45 * cus / 256.0 * small);
+                double step = std::max(0.11 + 0.0155 * mfmas, per_cu * 0.0155 * mfmas) *
+                              (1.0 + 0.45 * cus / 256.0 * small);
+                if (tiles_m <= 2) step = std::max(step, 1.0);     // nobody has read these weights before: memory is far
                 const double ends = 5.0 + 0.03 * mfmas;
                 const double from_memory = ((double)m + n) * k * 2.0 / 5.5e6;
                 const double cost = std::max(rounds * (k / slices / DM_BK * step + ends), from_memory + ends) +
