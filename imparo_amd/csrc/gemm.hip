@@ -1293,8 +1293,9 @@ static void launch_stream(const bf16_t* x, const bf16_t* w, const float* bias, T
         k_gemm_bf16_stream<TOut, MT, 2><<<grid, 2 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
 }
 
-// The 256x256 tile (one block per CU) pays once its tiles keep most of the chip's 256 CUs busy:
-// measured, from about 160 tiles on (192 tiles: +15% over 128x128; 96 tiles: -30%).
+// With a K that the kernel with loads straight into LDS does not take: the 256x256 tile with register
+// staging (one block per CU) pays once its tiles keep most of the chip's 256 CUs busy: measured, from
+// about 160 tiles on (192 tiles: +15% over 128x128; 96 tiles: -30%).
 static bool big_tile_pays(int m, int n, int k) {
     (void)k;
     return (long long)((m + 255) / 256) * ((n + 255) / 256) >= 160;
@@ -1324,8 +1325,8 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
         else
             launch_skinny<TOut, 4>(x, w, bias, y, m, n, k, epilogue, slices, s);
     } else {
-        // `force` 256: the 256x256 tile on eight waves; 258: 256x256 on four waves with loads
-        // straight into LDS (for measurements); otherwise by shape
+        // by shape: the tile kernel with loads straight into LDS where it takes the K, as its plan says;
+        // `force` (for measurements) 256: the 256x256 tile with register staging
         if (force == 0) {
             const DmaPlan plan = dma_plan(m, n, k, slices);
             if (plan.tn) return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, plan.bm, plan.tn, slices, s);
@@ -1351,9 +1352,11 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
 }
 
 
-// For measurements only: 0 lets the library choose the kernel, 1 forces the K-split kernel,
-// 2, 4 or 8 the shared-activation kernel with that many waves, 256/258 the large tiles;
-// plus 1000 times a number of K slices that imparo_gemm then accepts whatever the shape.
+// For measurements and tests only: 0 lets the library choose the kernel, 1 forces the K-split
+// kernel, 2, 4 or 8 the shared-activation kernel with that many waves, 256 the 256x256 tile with
+// register staging, 258 / 263 / 262 the tile with loads straight into LDS at 256 rows by 256 / 192 /
+// 128, 358 / 352 the same at 128 rows by 256 / 128; plus 1000 times a number of K slices that
+// imparo_gemm then accepts whatever the shape.
 extern "C" void imparo_gemm_force_kernel(int which) {
     g_force_slices = which / 1000;
     g_force_few_row_kernel = which % 1000;
