@@ -694,7 +694,8 @@ static bool dma_tile_takes(int m, int n, int k) {
 // does not take). A model of the time, fitted to this machine (it picks the fastest or one within
 // a few percent of it on every shape measured, 128 to 4,096 rows):
 //   - a block alone on its CU takes 0.11 us + 0.0155 us per MFMA of a SIMD for a K-step of 64
-//     (bm * bn / 1024 of them), and 5 us + 0.03 us per such MFMA for its beginning and end;
+//     (bm * bn / 1024 of them), and 5 us + 0.03 us per such MFMA for its beginning and end
+//     (the 192 wide tile on four waves: 0.62 us a step, 16 us for beginning and end);
 //   - two blocks fit a CU where their stages take 80 KB or less each (the 128x128 tile), and a
 //     step then takes what the products of both take;
 //   - the more CUs are busy the slower each runs (clocks, L2): up to 45% with all 256, and more
@@ -730,10 +731,11 @@ static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
                 const double per_cu = (double)((per_round + (long long)cus - 1) / (long long)cus);
                 const double mfmas = bm * bn / 1024.0;
                 const double small = 1.0 + 0.1 * (256.0 / bm - 1.0) + 0.1 * (256.0 / bn - 1.0);
-                double step = std::max(0.11 + 0.0155 * mfmas, per_cu * 0.0155 * mfmas) *
+                // (the 192 wide tile's four waves take their steps faster and their beginning and end slower)
+                double step = (tn == 3 ? 0.62 : std::max(0.11 + 0.0155 * mfmas, per_cu * 0.0155 * mfmas)) *
                               (1.0 + 0.45 * cus / 256.0 * small);
                 if (tiles_m <= 2) step = std::max(step, 1.0);     // nobody has read these weights before: memory is far
-                const double ends = 5.0 + 0.03 * mfmas;
+                const double ends = tn == 3 ? 16.0 : 5.0 + 0.03 * mfmas;
                 const double from_memory = ((double)m + n) * k * 2.0 / 5.5e6;
                 const double cost = std::max(rounds * (k / slices / DM_BK * step + ends), from_memory + ends) +
                                     (double)slices * m * n * 4.0 / 5e6 + (slices - 1) * ((double)m * n * 4.0 / 5e6);
