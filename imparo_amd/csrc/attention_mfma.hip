@@ -921,8 +921,10 @@ extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, cons
         // four heads of a kv head to a block where the group allows it, else more runs of queries
         const int group = heads / kv_heads;
         const int hpb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
-        // 32 queries a wave unless that leaves fewer waves than twice the SIMDs (n_tiles x 64 queries x heads at most)
-        const bool wide = (long long)n_tiles * 2 * heads >= 2048;
+        // 32 queries a wave where that still leaves twice as many waves as SIMDs (n_tiles x 64 queries x heads at most)
+        // and the contexts are long (the tables' width bounds them): measured with 32 heads of 64 and 2,048
+        // queries, 16 a wave are 9% faster on a fresh prompt, as fast at 4,096 keys and 5 to 9% slower from 16k on
+        const bool wide = (long long)n_tiles * 2 * heads >= 2048 && (long long)table_stride * page_size >= 8192;
         // n_tiles counts tiles of 64 queries per row: a row has at most that many blocks of 64 queries or more,
         // and 64 / qt times as many of fewer (blocks past a row's last find no tile and leave)
         const int qt = (wide ? 32 : 16) * (MFMA_WAVES / hpb);

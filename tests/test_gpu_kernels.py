@@ -345,7 +345,7 @@ def test_qk_norm_rope_store_many_tokens(H, Hk, D, rot, vt):
 
 # ---------------------------------------------------------------- attention
 def _attention_case(H, Hk, D, page_size, window, dtype, sharpen=None, seed=0, kernel="wave", v_transposed=None,
-                    ctx_lens=(70, 1, 200, 33), q_lens=(5, 1, 1, 33), attend=P.attend):
+                    ctx_lens=(70, 1, 200, 33), q_lens=(5, 1, 1, 33), attend=P.attend, table_width=0):
     """Rows at different depths of their contexts; the cache is filled by hand
     from whole-sequence k, v; the reference attends over the whole sequences."""
     # the last q_len positions of each context are queried
@@ -357,6 +357,8 @@ def _attention_case(H, Hk, D, page_size, window, dtype, sharpen=None, seed=0, ke
         k = (c + page_size - 1) // page_size
         tables.append(perm[nxt:nxt + k])
         nxt += k
+    if table_width:                            # room for longer contexts: entries nobody may read (their pages hold NaN)
+        tables[0] = tables[0] + perm[nxt:nxt + 3] * ((table_width - len(tables[0]) + 2) // 3)
     segments = [(c - ql, ql) for c, ql in zip(ctx_lens, q_lens)]
     ctx = hand_context(segments, page_size, n_pages, dtype, DEV, kv_sites={0: (Hk, D)}, tables=tables,
                        v_transposed=vt)
@@ -422,6 +424,17 @@ def test_matrix_core_attention(H, Hk, D, page_size, window):
     # and the general kernel reads the transposed layout too
     got, ref = _attention_case(H, Hk, D, page_size, window, torch.bfloat16, kernel="wave", v_transposed=True)
     torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)
+
+
+@pytest.mark.parametrize("H,Hk,D,ctx,q", [(64, 16, 32, 1100, 1024), (32, 8, 64, 2100, 2048)])
+def test_matrix_core_attention_with_32_queries_a_wave(H, Hk, D, ctx, q):
+    """Many query tiles and heads, and block tables with room for 8,192 positions: the prompt kernel
+    then gives each wave 32 queries. The same rows with narrow tables (16 queries a wave) agree."""
+    wide, ref = _attention_case(H, Hk, D, 64, None, torch.bfloat16, kernel="mfma", ctx_lens=(ctx, 40), q_lens=(q, 1),
+                                table_width=130)
+    torch.testing.assert_close(wide, ref, rtol=2 ** -6, atol=2 ** -6)
+    narrow, _ = _attention_case(H, Hk, D, 64, None, torch.bfloat16, kernel="mfma", ctx_lens=(ctx, 40), q_lens=(q, 1))
+    torch.testing.assert_close(wide, narrow, rtol=2 ** -7, atol=2 ** -7)
 
 
 def test_matrix_core_attention_refuses_other_sizes():
