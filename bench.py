@@ -161,9 +161,9 @@ def serving_workload(dtype):
     return 0
 
 
-def long_workload(dtype, requests, prompt_len):
+def long_workload(dtype, requests, prompt_len, portion=2048):
     """Long contexts: `requests` concurrent requests, each a prompt of `prompt_len` tokens fed in
-    2,048-token portions, then 128 decoded tokens each. LFM2-350M shape."""
+    portions of `portion` tokens (2,048), then 128 decoded tokens each. LFM2-350M shape."""
     import torch
     from imparo_amd import write_random_model
     from imparo_amd.engine import DeviceToken, Engine, StepEntry
@@ -180,8 +180,8 @@ def long_workload(dtype, requests, prompt_len):
     last = []
     for rid in ids:
         prompt = torch.randint(0, cfg["vocab_size"], (prompt_len,), generator=g).tolist()
-        for lo in range(0, prompt_len, 2048):
-            hi = min(prompt_len, lo + 2048)
+        for lo in range(0, prompt_len, portion):
+            hi = min(prompt_len, lo + portion)
             out = engine.step([StepEntry(rid, prompt[lo:hi], [hi - lo - 1] if hi == prompt_len else [])])
         last.append(out)
         if rid % 8 == 7:
@@ -204,7 +204,7 @@ def long_workload(dtype, requests, prompt_len):
         "prefill_tok_s": round(requests * prompt_len / (t1 - t0), 1), "prefill_seconds": round(t1 - t0, 3),
         "decode_ms_per_step": round((t2 - t1) / 127 * 1e3, 3), "dtype": "bf16" if dtype == "bfloat16" else "fp32",
         "data": "synthetic token ids, random weights (seed 4)",
-        "config": {"model": "LFM2-350M shape", "requests": requests, "prompt_len": prompt_len, "portion": 2048,
+        "config": {"model": "LFM2-350M shape", "requests": requests, "prompt_len": prompt_len, "portion": portion,
                    "decode_tokens": 128, "hidden_size": 1024, "heads": 16, "kv_heads": 8, "ff_dim": 4608, "layers": 16,
                    "cache_pages_used": engine.cache.groups[0].pool.n_pages - engine.free_pages()[0]}}), flush=True)
     return 0
@@ -227,6 +227,7 @@ def main() -> int:
                          "each (LFM2-350M shape). The last two print a line of their own")
     ap.add_argument("--requests", type=int, default=64, help="--workload long: concurrent requests")
     ap.add_argument("--prompt-len", type=int, default=32768, help="--workload long: tokens per prompt")
+    ap.add_argument("--portion", type=int, default=2048, help="--workload long: tokens of a prompt per step")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -234,7 +235,7 @@ def main() -> int:
     if args.workload == "serving":
         return serving_workload(args.dtype)
     if args.workload == "long":
-        return long_workload(args.dtype, args.requests, args.prompt_len)
+        return long_workload(args.dtype, args.requests, args.prompt_len, args.portion)
 
     import torch
     from imparo_amd import write_random_model

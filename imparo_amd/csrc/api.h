@@ -84,8 +84,13 @@ int imparo_attention_decode(const void* q, const void* k_cache, const void* v_ca
                             int n_splits, imparo_stream stream);
 
 // Prompt portions: the listed rows' segments in tiles of 64 queries;
-// n_tiles = sum over the rows of ceil(seg_len / 64).
+// n_tiles = sum over the rows of ceil(seg_len / 64). n_splits (from
+// imparo_attention_prefill_splits, or 1) parts of each block's keys, merged by a
+// second launch; then part_o holds [tokens, heads, n_splits, head_dim] floats
+// and part_ml [tokens, heads, n_splits, 2], tokens counted over the whole batch.
+int imparo_attention_prefill_splits(int n_tiles, int heads, int kv_heads, int head_dim, int max_context);
 int imparo_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
+                             float* part_o, float* part_ml, int n_splits,
                              const int32_t* rows, int n_rows, int n_tiles,
                              const int32_t* seg_start, const int32_t* seg_len, const int32_t* positions,
                              const int32_t* block_table, int table_stride, int page_size,

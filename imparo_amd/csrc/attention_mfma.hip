@@ -12,6 +12,8 @@
 // operand layout, so the softmax weights feed the second product as they are.
 // Cache layouts: K [page, kv head, slot, dim], V [page, kv head, dim, slot].
 #include "common.h"
+
+#include <algorithm>
 #include "api.h"
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -580,7 +582,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     bf16_t* __restrict__ out, const int32_t* __restrict__ rows, int n_rows,
     const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int n_pages,
-    float scale, int window, int heads_per_block) {
+    float scale, int window, int heads_per_block, float* __restrict__ part_o, float* __restrict__ part_ml) {
     constexpr int D = ND * 16, NK = ND / 2;
     constexpr int LDK = D + 8, LDV = PX_KEYS + 8;
     static_assert(ND % 2 == 0, "head sizes in steps of 32");
@@ -612,10 +614,21 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     const int pos0 = positions[t0];
     const int32_t* table = block_table + (size_t)row * table_stride;
 
-    // the block's key range: from the lowest key its first query may read to its last query's position
+    // the block's key range: from the lowest key its first query may read to its last query's position;
+    // with splits (gridDim.z > 1: few queries over long contexts) block z takes the z-th part of its tiles
+    // of keys and leaves (max, sum, unnormalised output) per query for the merge kernel
     const int blk_first = pos0 + tile * qt;
-    const int blk_last = pos0 + min(len, tile * qt + qt) - 1;
-    const int blk_lo = window > 0 ? max(0, blk_first + 1 - window) : 0;
+    int blk_last = pos0 + min(len, tile * qt + qt) - 1;
+    int blk_lo = window > 0 ? max(0, blk_first + 1 - window) : 0;
+    const int n_splits = (int)gridDim.z, split = (int)blockIdx.z;
+    if (n_splits > 1) {
+        const int first_tile = blk_lo / PX_KEYS, tiles_all = blk_last / PX_KEYS - first_tile + 1;
+        const int per = (tiles_all + n_splits - 1) / n_splits;
+        blk_lo = max(blk_lo, (first_tile + split * per) * PX_KEYS);
+        blk_last = min(blk_last, (first_tile + (split + 1) * per) * PX_KEYS - 1);
+    }
+    const bool has_keys = blk_lo <= blk_last;
+    if (!has_keys) blk_lo = blk_last = max(blk_first, 0);       // nothing to add: one masked tile, a partial of zero weight
 
     // this wave's queries: q_first + 16 h + c for the halves h
     const int q_first = tile * qt + (wave / heads_per_block) * QW;
@@ -634,8 +647,8 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
         const int qi = q_first + 16 * h + c;
         qvalid[h] = qi < len;
         const int pos_q = pos0 + qi;
-        lo_q[h] = window > 0 ? max(0, pos_q + 1 - window) : 0;
-        hi_q[h] = qvalid[h] ? pos_q : -1;
+        lo_q[h] = max(window > 0 ? max(0, pos_q + 1 - window) : 0, blk_lo);
+        hi_q[h] = (qvalid[h] && has_keys) ? min(pos_q, blk_last) : -1;
         const bf16_t* qrow = q + ((size_t)(t0 + min(qi, len - 1)) * heads + head) * D + 8 * g;
 #pragma unroll
         for (int dk = 0; dk < NK; ++dk)
@@ -734,7 +747,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
         load_pages(kb + 3 * PX_KEYS);
         // this wave's part of the tile: keys lo_all .. pos_last
         if (wave_on && kb <= pos_last && kb + PX_KEYS - 1 >= lo_all) {
-            const bool full = kb >= lo_max && kb + PX_KEYS - 1 <= pos_first;
+            const bool full = kb >= lo_max && kb + PX_KEYS - 1 <= pos_first && kb >= blk_lo && kb + PX_KEYS - 1 <= blk_last;
             f32x4 sc[HALVES][4];
 #pragma unroll
             for (int s16 = 0; s16 < 4; ++s16) {
@@ -839,6 +852,22 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
         tile_step(kb + PX_KEYS, 1, kr_a, vr_a, kr_b, vr_b);
     }
     if (!wave_on) return;
+    if (n_splits > 1) {
+#pragma unroll
+        for (int h = 0; h < HALVES; ++h) {
+            if (!qvalid[h]) continue;
+            const size_t slot = ((size_t)(t0 + q_first + 16 * h + c) * heads + head) * n_splits + split;
+            if (g == 0) {
+                part_ml[slot * 2] = m_run[h];               // of unscaled scores; -inf: no key, weight zero
+                part_ml[slot * 2 + 1] = l_run[h];
+            }
+            float* dst = part_o + slot * D + 4 * g;
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt)
+                *reinterpret_cast<float4*>(dst + dt * 16) = make_float4(o[h][dt][0], o[h][dt][1], o[h][dt][2], o[h][dt][3]);
+        }
+        return;
+    }
 #pragma unroll
     for (int h = 0; h < HALVES; ++h) {
         if (!qvalid[h]) continue;
@@ -851,6 +880,48 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
             for (int i = 0; i < 4; ++i) v[i] = pack_bf16(o[h][dt][i] * inv);
             *reinterpret_cast<s16x4*>(dst + dt * 16) = v;
         }
+    }
+}
+
+// One wave per (token, head) of the launch's portion rows merges the splits of the kernel above, in
+// split order: weights exp2((max_s - max) * scale * log2 e), as the kernel itself weighs its tiles.
+__global__ void k_attn_prefill_merge(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                     bf16_t* __restrict__ out, const int32_t* __restrict__ rows, int n_rows,
+                                     const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len,
+                                     int heads, int head_dim, int n_splits, float scale) {
+    int tok = blockIdx.x, t = -1;
+    for (int i = 0; i < n_rows; ++i) {                   // the tok-th token of the listed rows
+        const int r = rows[i];
+        if (tok < seg_len[r]) {
+            t = seg_start[r] + tok;
+            break;
+        }
+        tok -= seg_len[r];
+    }
+    if (t < 0) return;
+    const int lane = threadIdx.x & 63, head = blockIdx.y * (blockDim.x / 64) + (threadIdx.x >> 6);
+    if (head >= heads) return;
+    const size_t base = ((size_t)t * heads + head) * n_splits;
+    const float scale_log2 = scale * 1.44269504088896340736f;
+    float ms = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) ms = fmaxf(ms, part_ml[(base + s) * 2]);
+    float acc[2] = {0.f, 0.f}, ls = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+        const float m = part_ml[(base + s) * 2];
+        if (m == -INFINITY) continue;                    // no key in that part: its output was never a sum
+        const float wgt = __builtin_amdgcn_exp2f((m - ms) * scale_log2);
+        ls += part_ml[(base + s) * 2 + 1] * wgt;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int d = lane + j * 64;
+            if (d < head_dim) acc[j] += part_o[(base + s) * head_dim + d] * wgt;
+        }
+    }
+    const float inv = ls > 0.f ? 1.0f / ls : 0.f;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int d = lane + j * 64;
+        if (d < head_dim) out[((size_t)t * heads + head) * head_dim + d] = f32_to_bf16(acc[j] * inv);
     }
 }
 
@@ -905,7 +976,44 @@ extern "C" int imparo_attention_decode(const void* q, const void* k_cache, const
     return launch_status();
 }
 
+// How the prompt kernel for head sizes in steps of 32 lays a launch out: heads of a kv head to a block,
+// 16 or 32 queries a wave, queries of a head per block.
+struct PrefillShape {
+    int hpb, qt;
+    bool wide;
+    long long blocks;
+};
+static PrefillShape prefill_shape(int n_tiles, int heads, int kv_heads, long long context_bound) {
+    PrefillShape p;
+    // four heads of a kv head to a block where the group allows it, else more runs of queries
+    const int group = heads / kv_heads;
+    p.hpb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+    // 32 queries a wave where that still leaves twice as many waves as SIMDs (n_tiles x 64 queries x heads at most)
+    // and the contexts are long: measured with 32 heads of 64 and 2,048 queries, 16 a wave are 9% faster
+    // on a fresh prompt, as fast at 4,096 keys and 5 to 9% slower from 16k on
+    p.wide = (long long)n_tiles * 2 * heads >= 2048 && context_bound >= 8192;
+    // n_tiles counts tiles of 64 queries per row: a row has at most that many blocks of 64 queries or more,
+    // and 64 / qt times as many of fewer (blocks past a row's last find no tile and leave)
+    p.qt = (p.wide ? 32 : 16) * (MFMA_WAVES / p.hpb);
+    p.blocks = (long long)n_tiles * (p.qt < 64 ? 64 / p.qt : 1) * (heads / p.hpb);
+    return p;
+}
+
+// Into how many parts the keys of a launch of prompt portions are cut (1: none). Few queries over a
+// long context leave the chip idle (512 queries of 16 heads are 128 blocks, each walking all the keys:
+// 474 us over 30,000 keys, 144 us in 8 parts): up to 8 parts, towards four blocks per CU, at least
+// 1,024 keys of the longest context each; the caller brings room for the parts' results
+// ([tokens, heads, parts, head size] and [.., 2] floats).
+extern "C" int imparo_attention_prefill_splits(int n_tiles, int heads, int kv_heads, int head_dim, int max_context) {
+    if (n_tiles <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || head_dim % 32 != 0) return 1;
+    const PrefillShape p = prefill_shape(n_tiles, heads, kv_heads, max_context);
+    const long long blocks = p.blocks * (p.wide ? 2 : 1);       // a block of 32 queries a wave counts as two
+    if (blocks >= 1024 || max_context < 2048) return 1;
+    return (int)std::max<long long>(1, std::min<long long>({8, 1024 / blocks, max_context / 1024}));
+}
+
 extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                        float* part_o, float* part_ml, int n_splits,
                                         const int32_t* rows, int n_rows, int n_tiles,
                                         const int32_t* seg_start, const int32_t* seg_len, const int32_t* positions,
                                         const int32_t* block_table, int table_stride, int page_size,
@@ -915,29 +1023,26 @@ extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, cons
                                  page_size, heads, kv_heads, head_dim, n_pages, window);
     if (bad) return bad;
     if (!seg_len || n_rows < 0 || n_tiles < 0 || heads > 65535) return IMPARO_BAD_ARGUMENT;
+    if (n_splits < 1 || n_splits > 64 || (n_splits > 1 && (!part_o || !part_ml || head_dim % 32 != 0)))
+        return IMPARO_BAD_ARGUMENT;
     if (n_rows == 0 || n_tiles == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;
     if (head_dim % 32 == 0) {
-        // four heads of a kv head to a block where the group allows it, else more runs of queries
-        const int group = heads / kv_heads;
-        const int hpb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
-        // 32 queries a wave where that still leaves twice as many waves as SIMDs (n_tiles x 64 queries x heads at most)
-        // and the contexts are long (the tables' width bounds them): measured with 32 heads of 64 and 2,048
-        // queries, 16 a wave are 9% faster on a fresh prompt, as fast at 4,096 keys and 5 to 9% slower from 16k on
-        const bool wide = (long long)n_tiles * 2 * heads >= 2048 && (long long)table_stride * page_size >= 8192;
-        // n_tiles counts tiles of 64 queries per row: a row has at most that many blocks of 64 queries or more,
-        // and 64 / qt times as many of fewer (blocks past a row's last find no tile and leave)
-        const int qt = (wide ? 32 : 16) * (MFMA_WAVES / hpb);
-        dim3 grid32((unsigned)(n_tiles * (qt < 64 ? 64 / qt : 1)), heads / hpb);
+        const PrefillShape p = prefill_shape(n_tiles, heads, kv_heads, (long long)table_stride * page_size);
+        const int hpb = p.hpb;
+        const bool wide = p.wide;
+        dim3 grid32((unsigned)(n_tiles * (p.qt < 64 ? 64 / p.qt : 1)), heads / hpb, n_splits);
 #define PREFILL_X32(ND)                                                                                              \
     if (wide)                                                                                                        \
         k_attn_prefill_x32<ND, 2><<<grid32, MFMA_WAVES * 64, 0, s>>>(                                                \
             (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, rows, n_rows, seg_start, \
-            seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, hpb); \
+            seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, hpb,  \
+            part_o, part_ml);                                                                                        \
     else                                                                                                             \
         k_attn_prefill_x32<ND, 1><<<grid32, MFMA_WAVES * 64, 0, s>>>(                                                \
             (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, rows, n_rows, seg_start, \
-            seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, hpb)
+            seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, hpb,  \
+            part_o, part_ml)
         switch (head_dim / 32) {
             case 1: PREFILL_X32(2); break;
             case 2: PREFILL_X32(4); break;
@@ -945,6 +1050,12 @@ extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, cons
             default: PREFILL_X32(8);
         }
 #undef PREFILL_X32
+        if (launch_status()) return IMPARO_LAUNCH_FAILED;
+        if (n_splits == 1) return IMPARO_OK;
+        // a block of four waves per token and four heads; tokens past the portions' last find none and leave
+        dim3 merge_grid((unsigned)n_tiles * 64, (unsigned)((heads + 3) / 4));
+        k_attn_prefill_merge<<<merge_grid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, rows, n_rows, seg_start, seg_len,
+                                                       heads, head_dim, n_splits, scale);
         return launch_status();
     }
     dim3 grid(n_tiles, heads);

@@ -33,7 +33,8 @@ _SIGNATURES = {
     "imparo_qk_norm_rope_store": [P, P, P, F, P, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, P],
     "imparo_attention": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
     "imparo_attention_decode": [P, P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
-    "imparo_attention_prefill": [P, P, P, P, P, I, I, P, P, P, P, I, I, I, I, I, I, F, I, P],
+    "imparo_attention_prefill": [P, P, P, P, P, P, I, P, I, I, P, P, P, P, I, I, I, I, I, I, F, I, P],
+    "imparo_attention_prefill_splits": [I, I, I, I, I],
     "imparo_short_conv": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
     "imparo_short_conv_state": [P, P, P, P, P, I, I, I, I, I, P],
     "imparo_argmax_rows": [P, P, I, I, P],

@@ -279,13 +279,31 @@ def attention_decode(q, k_cache, v_cache, out, part_o, part_ml, rows, n_rows: in
     return out
 
 
+def attention_prefill_splits(n_tiles: int, heads: int, kv_heads: int, head_dim: int, max_context: int) -> int:
+    """Into how many parts the keys of a launch of prompt portions are cut (1: none): few queries
+    over long contexts would leave most of the chip idle."""
+    return int(library().imparo_attention_prefill_splits(n_tiles, heads, kv_heads, head_dim, max_context))
+
+
 def attention_prefill(q, k_cache, v_cache, out, rows, n_rows: int, n_tiles: int, seg_start, seg_len, positions,
-                      block_table, scale: float, window: Optional[int]) -> torch.Tensor:
+                      block_table, scale: float, window: Optional[int], part_o: Optional[torch.Tensor] = None,
+                      part_ml: Optional[torch.Tensor] = None, n_splits: int = 1) -> torch.Tensor:
     """Tiled attention for rows that bring a portion of a prompt. `n_tiles` is
-    the sum over the listed rows of ceil(seg_len / 64)."""
+    the sum over the listed rows of ceil(seg_len / 64). With `n_splits` > 1
+    (attention_prefill_splits) each block's keys are walked in that many parts,
+    merged by a second launch: `part_o` [n, heads, n_splits, head_dim] and
+    `part_ml` [n, heads, n_splits, 2] float32 hold the parts."""
     n, heads, head_dim, n_pages, kv_heads, page_size = _check_mfma(q, k_cache, v_cache, out)
+    if n_splits > 1:
+        if part_o is None or part_ml is None:
+            raise KernelArgumentError("attention_prefill: parts of the keys need buffers for their results")
+        _dev(part_o, "part_o", torch.float32)
+        _dev(part_ml, "part_ml", torch.float32)
+        if part_o.numel() < n * heads * n_splits * head_dim or part_ml.numel() < n * heads * n_splits * 2:
+            raise KernelArgumentError("attention_prefill: the buffers for the parts are too small")
     _check(library().imparo_attention_prefill(
         _dev(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
+        part_o.data_ptr() if n_splits > 1 else None, part_ml.data_ptr() if n_splits > 1 else None, int(n_splits),
         _dev(rows, "prefill rows", torch.int32), n_rows, n_tiles, _dev(seg_start, "seg_start", torch.int32),
         _dev(seg_len, "seg_len", torch.int32), _dev(positions, "positions", torch.int32, (n,)),
         _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size, heads, kv_heads, head_dim,

@@ -106,9 +106,17 @@ class Attention:
                 ops.attention_decode(q, k_cache, v_cache, o, part_o, part_ml, ctx.decode_rows, ctx.n_decode_rows,
                                      ctx.seg_start, ctx.positions, table, self.scale, self.window, ctx.max_context)
             if ctx.n_prefill_rows:
+                # few queries over long contexts: each block's keys in parts, merged by a second launch
+                parts = ops.attention_prefill_splits(ctx.n_prefill_tiles, self.heads, self.kv_heads, self.head_dim,
+                                                     ctx.max_context)
+                part_o = part_ml = None
+                if parts > 1:
+                    part_o = ctx.workspace.get("attn_prefill_part_o", (T * self.heads * parts * self.head_dim,),
+                                               torch.float32)
+                    part_ml = ctx.workspace.get("attn_prefill_part_ml", (T * self.heads * parts * 2,), torch.float32)
                 ops.attention_prefill(q, k_cache, v_cache, o, ctx.prefill_rows, ctx.n_prefill_rows,
                                       ctx.n_prefill_tiles, ctx.seg_start, ctx.seg_len, ctx.positions, table,
-                                      self.scale, self.window)
+                                      self.scale, self.window, part_o, part_ml, parts)
         else:
             ops.attention(q, k_cache, v_cache, o, ctx.positions, ctx.row_of_token, table, self.scale, self.window,
                           v_transposed=vt)

@@ -345,7 +345,7 @@ def test_qk_norm_rope_store_many_tokens(H, Hk, D, rot, vt):
 
 # ---------------------------------------------------------------- attention
 def _attention_case(H, Hk, D, page_size, window, dtype, sharpen=None, seed=0, kernel="wave", v_transposed=None,
-                    ctx_lens=(70, 1, 200, 33), q_lens=(5, 1, 1, 33), attend=P.attend, table_width=0):
+                    ctx_lens=(70, 1, 200, 33), q_lens=(5, 1, 1, 33), attend=P.attend, table_width=0, prefill_splits=1):
     """Rows at different depths of their contexts; the cache is filled by hand
     from whole-sequence k, v; the reference attends over the whole sequences."""
     # the last q_len positions of each context are queried
@@ -397,8 +397,13 @@ def _attention_case(H, Hk, D, page_size, window, dtype, sharpen=None, seed=0, ke
         part_ml = torch.full((ctx.n_decode_rows * H * n_splits * 2,), float("nan"), device=DEV)
         ops().attention_decode(q_all, k_cache, v_cache, out, part_o, part_ml, ctx.decode_rows, ctx.n_decode_rows,
                                ctx.seg_start, ctx.positions, table, scale, window, ctx.max_context)
+        parts_o = parts_ml = None
+        if prefill_splits > 1:                 # NaN where no part writes: a part without keys must not be read
+            parts_o = torch.full((ctx.n_tokens, H, prefill_splits, D), float("nan"), device=DEV)
+            parts_ml = torch.full((ctx.n_tokens, H, prefill_splits, 2), float("nan"), device=DEV)
         ops().attention_prefill(q_all, k_cache, v_cache, out, ctx.prefill_rows, ctx.n_prefill_rows,
-                                ctx.n_prefill_tiles, ctx.seg_start, ctx.seg_len, ctx.positions, table, scale, window)
+                                ctx.n_prefill_tiles, ctx.seg_start, ctx.seg_len, ctx.positions, table, scale, window,
+                                parts_o, parts_ml, prefill_splits)
     return out.cpu().float().reshape(-1, H, D), torch.cat(refs)
 
 
@@ -424,6 +429,23 @@ def test_matrix_core_attention(H, Hk, D, page_size, window):
     # and the general kernel reads the transposed layout too
     got, ref = _attention_case(H, Hk, D, page_size, window, torch.bfloat16, kernel="wave", v_transposed=True)
     torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)
+
+
+@pytest.mark.parametrize("H,Hk,D", [(6, 3, 64), (40, 2, 32), (12, 3, 96), (8, 1, 128)])
+@pytest.mark.parametrize("page_size,window", [(16, None), (32, 19), (128, 300)])
+@pytest.mark.parametrize("parts", [3, 8])
+def test_matrix_core_attention_with_the_keys_in_parts(H, Hk, D, page_size, window, parts):
+    """Prompt portions whose blocks walk their keys in parts, merged by a second launch (few queries
+    over long contexts); short contexts leave some parts without keys."""
+    got, ref = _attention_case(H, Hk, D, page_size, window, torch.bfloat16, kernel="mfma", prefill_splits=parts,
+                               ctx_lens=(70, 1, 700, 33, 300, 513, 256), q_lens=(5, 1, 1, 33, 150, 1, 1))
+    torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)
+    assert ops().attention_prefill_splits(8, 16, 8, 64, 30000) == 8          # 128 blocks: eight parts make 1024
+    assert ops().attention_prefill_splits(8, 16, 8, 64, 3000) == 2           # at least 1024 keys to a part
+    assert ops().attention_prefill_splits(8, 16, 8, 64, 1500) == 1           # a short context is walked whole
+    assert ops().attention_prefill_splits(32, 16, 8, 64, 30000) == 2         # 512 blocks
+    assert ops().attention_prefill_splits(32, 32, 8, 64, 30000) == 1         # 512 blocks of 32 queries a wave: enough
+    assert ops().attention_prefill_splits(8, 16, 8, 80, 30000) == 1          # (the kernel for other head sizes has none)
 
 
 @pytest.mark.parametrize("H,Hk,D,ctx,q", [(64, 16, 32, 1100, 1024), (32, 8, 64, 2100, 2048)])

@@ -32,22 +32,25 @@ def long_model(tmp_path_factory):
 
 def test_long_context_bfloat16_against_float32(long_model):
     """16,500 tokens in portions of 2,048 (tiles of 64 queries over hundreds of
-    key tiles, a window of 700 that gives pages back), then single tokens over
-    more than 64 splits of 256 keys, through captured steps."""
+    key tiles, a window of 700 that gives pages back), two short portions (their
+    keys walked in parts), then single tokens over more than 64 splits of 256
+    keys, through captured steps."""
     from imparo_amd.engine import StepEntry
     N = 16500
-    toks = prompt_tokens(512, N + 40, 99)
+    toks = prompt_tokens(512, N + 137 + 40, 99)
     runs = {}
     for dtype in ("float32", "bfloat16"):
-        eng = make_engine(long_model, dtype, page_size=64, max_tokens=N + 128, max_requests=2)
+        eng = make_engine(long_model, dtype, page_size=64, max_tokens=N + 256, max_requests=2)
         out = []
         for lo in range(0, N, 2048):
             hi = min(N, lo + 2048)
             out.append(eng.step([StepEntry("l", toks[lo:hi], list(range(hi - lo - 8, hi - lo)))]).cpu())
-        for i in range(N, N + 40):
+        for lo, hi in ((N, N + 100), (N + 100, N + 137)):
+            out.append(eng.step([StepEntry("l", toks[lo:hi], list(range(hi - lo)))]).cpu())
+        for i in range(N + 137, N + 137 + 40):
             out.append(eng.step([StepEntry("l", toks[i:i + 1], [0])]).cpu().clone())
         held = eng.cache.held_pages("l")
-        assert held[0] == (N + 40 + 63) // 64 and held[1] <= 700 // 64 + 2     # the window's group holds a dozen pages
+        assert held[0] == (N + 177 + 63) // 64 and held[1] <= 700 // 64 + 3    # the window's group holds a dozen pages
         runs[dtype] = torch.cat(out)
     check_logits(runs["bfloat16"], runs["float32"], "bfloat16", "long context")
 
