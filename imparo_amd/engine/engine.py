@@ -84,10 +84,10 @@ class _Upload:
 
 
 class _DecodeGraph:
-    """A captured step for one batch shape: the rows' token counts and wanted
-    counts, in order, and block tables `table_width` pages wide. Its index
-    arrays, its scratch and its logits live at fixed addresses; a replay reads
-    new indices from the same place."""
+    """A captured decode step for one batch shape: `rows` single-token requests
+    whose block tables are `table_width` pages wide. Its index arrays, its
+    scratch and its logits live at fixed addresses; a replay reads new indices
+    from the same place."""
 
     def __init__(self):
         self.graph = None
@@ -97,22 +97,8 @@ class _DecodeGraph:
         self.last_used = 0
 
 
-TABLE_BUCKET = 8     # captured steps round their block-table width up to this many pages, and in steps of a quarter beyond 64
+TABLE_BUCKET = 8     # captured steps round their block-table width up to this many pages
 MAX_GRAPHS = 96      # captured batch shapes kept; beyond that the one unused for longest goes
-MAX_GRAPH_BYTES = 8 << 30    # and their scratch together stays under this
-SHAPES_REMEMBERED = 512      # batch shapes seen once are remembered so that the second coming is captured
-
-
-def table_bucket(pages: int) -> int:
-    """The block-table width a captured step is made for: every 8 pages up to
-    64, then widths a quarter apart (a prompt that grows by a portion a step
-    meets a new width ever more rarely)."""
-    if pages <= 64:
-        return max(TABLE_BUCKET, -(-pages // TABLE_BUCKET) * TABLE_BUCKET)
-    b = 64
-    while b < pages:
-        b = -(-(b * 5 // 4) // TABLE_BUCKET) * TABLE_BUCKET
-    return b
 
 
 class Engine:
@@ -142,12 +128,10 @@ class Engine:
         self.storage = CacheStorage(self.cache, self.dtype, self.device)
         self.workspace = Workspace(self.device)
         self._upload = _Upload(self.device)
-        # steps replay a captured HIP graph where their shape has come before (decode steps: where it
-        # comes at all): the launches of a step cost the host about 1.5 ms, more than the kernels
-        # of a decode step or of a short prompt portion take
+        # decode steps (every request brings one token and wants its logits) replay a captured
+        # HIP graph: the launches of a step cost more host time than the step's kernels take
         self.use_graphs = use_graphs
-        self._graphs: Dict[Tuple, _DecodeGraph] = {}
-        self._shapes_seen: Dict[Tuple, int] = {}
+        self._graphs: Dict[Tuple[int, int], _DecodeGraph] = {}
         self._decode_code_loaded = False
         self._graph_pool = None
         self.vocab_size = self.plan.vocab_size
@@ -203,10 +187,13 @@ class Engine:
         try:
             for slot in batch.new_slots[batch.new_slots >= 0].tolist():
                 self.storage.zero_slot(slot)
-            if self.use_graphs and self.model.graph_safe:
-                logits = self._captured_step(entries, batch)
+            if (self.use_graphs and self.model.graph_safe and batch.T == len(entries)
+                    and bool((batch.n_want == 1).all())):
+                logits = self._decode_step(entries, batch)       # one token each, wanted
             else:
-                logits = self._launched_step(batch)
+                ctx, token_ids, want_rows = self._pack(batch)
+                with ops.on_current_stream():
+                    logits = self.model.forward(ctx, token_ids, want_rows)
         except BaseException:
             self.cache.abort_step(batch)
             raise
@@ -230,32 +217,22 @@ class Engine:
             return f"request {e.request!r}: wanted place {bad} is outside its {len(e.tokens)} tokens"
         return f"request {e.request!r}: the cache manager refused the step with code {code}"
 
-    def _launched_step(self, batch) -> Optional[torch.Tensor]:
-        ctx, token_ids, want_rows = self._pack(batch)
-        with ops.on_current_stream():
-            return self.model.forward(ctx, token_ids, want_rows)
-
-    def _captured_step(self, entries: Sequence[StepEntry], batch) -> Optional[torch.Tensor]:
-        """A step whose shape (the rows' token counts and wanted counts, in
-        order, and the bucket of its block tables' width) may come again. A
-        shape of single tokens that are all wanted, a decode step, is captured
-        when it first comes, any other when it comes the second time; from then
-        on it is replayed. The engine's first decode step runs launch by launch
-        like any shape's first: a capture cannot load code onto the device, and
-        every module of kernels a shape uses is loaded once it has run."""
-        width = table_bucket(batch.widest)
-        key = (tuple(batch.n_tok.tolist()), tuple(batch.n_want.tolist()), width)
-        decode = batch.T == len(entries) and bool((batch.n_want == 1).all())
+    def _decode_step(self, entries: Sequence[StepEntry], batch) -> torch.Tensor:
+        """A step of single tokens. The engine's first such step runs launch by
+        launch (a capture cannot load code onto the device, and every module of
+        kernels a decode step uses is loaded once one has run); after that a
+        batch shape is captured when it first comes and replayed from then on."""
+        width = -(-batch.widest // TABLE_BUCKET) * TABLE_BUCKET
+        key = (len(entries), width)
+        if not self._decode_code_loaded:
+            self._decode_code_loaded = True
+            ctx, token_ids, want_rows = self._pack(batch)
+            with ops.on_current_stream():
+                return self.model.forward(ctx, token_ids, want_rows)
         g = self._graphs.get(key)
         if g is None:
-            seen = self._shapes_seen.pop(key, 0)
-            if (decode and not self._decode_code_loaded) or (not decode and seen == 0):
-                self._decode_code_loaded = self._decode_code_loaded or decode
-                if len(self._shapes_seen) >= SHAPES_REMEMBERED:
-                    del self._shapes_seen[next(iter(self._shapes_seen))]
-                self._shapes_seen[key] = seen + 1
-                return self._launched_step(batch)
-            self._make_room_for_a_graph()
+            if len(self._graphs) >= MAX_GRAPHS:      # each holds a workspace and a logits buffer
+                del self._graphs[min(self._graphs, key=lambda k: self._graphs[k].last_used)]
             g = self._graphs[key] = _DecodeGraph()
         g.last_used = self.steps_run
         if g.graph is None:
@@ -272,13 +249,6 @@ class Engine:
             self._pack(batch, table_width=width, workspace=g.workspace, graph=g)
         g.graph.replay()
         return g.logits
-
-    def _make_room_for_a_graph(self) -> None:
-        """Each captured shape holds a workspace and a logits buffer: the ones unused for longest go."""
-        def held() -> int:
-            return sum(x.workspace.nbytes() for x in self._graphs.values() if x.workspace is not None)
-        while self._graphs and (len(self._graphs) >= MAX_GRAPHS or held() > MAX_GRAPH_BYTES):
-            del self._graphs[min(self._graphs, key=lambda k: self._graphs[k].last_used)]
 
     def _pack(self, batch, table_width: Optional[int] = None,
               workspace: Optional[Workspace] = None, graph: Optional[_DecodeGraph] = None):
@@ -315,9 +285,7 @@ class Engine:
             block_tables=block_tables, page_size=self.page_size, dtype=self.dtype,
             workspace=workspace or self.workspace, storage=self.storage, group_of_site=self.cache.group_of_site,
             max_seg_len=lay["max_seg_len"],
-            # (a bound: the same whether the step is launched or captured, so that both choose alike
-            # where a choice hangs on it, as the number of parts a prompt portion's keys are walked in)
-            max_context=(table_bucket(P) if table_width is None else table_width) * self.page_size,
+            max_context=lay["max_context"] if table_width is None else table_width * self.page_size,
             decode_rows=dev[o_lists:o_lists + n_dec], n_decode_rows=n_dec,
             prefill_rows=dev[o_lists + n_dec:o_lists + R], n_prefill_rows=lay["n_multi"],
             n_prefill_tiles=lay["n_prefill_tiles"],

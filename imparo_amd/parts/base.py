@@ -37,9 +37,6 @@ class Workspace:
             self._buffers[key] = buf
         return buf[:n].view(shape)
 
-    def nbytes(self) -> int:
-        return sum(b.numel() * b.element_size() for b in self._buffers.values())
-
 
 @dataclass
 class StepContext:

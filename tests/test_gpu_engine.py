@@ -219,39 +219,6 @@ def test_captured_decode_steps_equal_launched_ones(zoo, dtype):
     check_logits(runs[0][0:1], ref[len(prompts[0]) - 30:len(prompts[0]) - 29], dtype, "first decoded row")
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_captured_prompt_portions_equal_launched_ones(zoo, dtype):
-    """Any batch shape that comes a second time is captured and replayed from then on: prompts fed
-    in equal portions, alone and beside decoding rows, with and without wanted places. Every
-    step is compared, bit for bit, with the engine that launches each kernel."""
-    from imparo_amd.engine import StepEntry
-    V = vocab_of(zoo, "C_keen")
-    long_one, other = prompt_tokens(V, 48 * 9, 610), prompt_tokens(V, 300, 611)
-    deco = [prompt_tokens(V, 70, 620 + i) for i in range(2)]
-    runs = []
-    for use_graphs in (True, False):
-        eng = make_engine(zoo[0]["C_keen"], dtype, page_size=16, max_tokens=4096, use_graphs=use_graphs)
-        out = []
-        for i in range(2):
-            eng.step([StepEntry(f"d{i}", deco[i][:30], [])])
-        for s in range(9):                               # the same shape nine times: launched, captured, replayed
-            lo = 48 * s
-            batch = [StepEntry("p", long_one[lo:lo + 48], [0, 47])]
-            if s >= 3:                                   # then beside two decoding rows: another shape, six times
-                batch += [StepEntry(f"d{i}", [deco[i][30 + s]], [0]) for i in range(2)]
-            out.append(eng.step(batch).cpu().clone())
-        for s in range(6):                               # a portion of which nothing is wanted
-            assert eng.step([StepEntry("o", other[50 * s:50 * s + 50], [])]) is None
-        out.append(eng.step([StepEntry("p2", other[:50], [49])]).cpu().clone())
-        if use_graphs:
-            assert sum(g.graph is not None for g in eng._graphs.values()) >= 3
-        runs.append(torch.cat(out))
-    assert torch.equal(runs[0], runs[1])
-    ref = zoo[1]["C_keen"](long_one)
-    # rows of `out`: two for each of the first three steps, then four a step; step 5 starts at row 14
-    check_logits(runs[0][14:15], ref[48 * 5:48 * 5 + 1], dtype, "a replayed portion's first place")
-
-
 def test_captured_steps_are_kept_up_to_a_limit(zoo, monkeypatch):
     """More batch shapes than the engine keeps captures for: the one unused for longest is dropped
     and captured again when it comes back; every step equals the launched one."""
