@@ -702,7 +702,7 @@ static bool dma_tile_takes(int m, int n, int k) {
 //     with small tiles, which read more operand bytes per product;
 //   - with one or two tiles down the rows (a decode batch of 65 to 256 rows) every block meets its
 //     weights first, and cold: a K-step then takes 1 us whatever the tile (measured: 32 us for 32
-//     steps at 128 rows), so such products are cut into up to 8 slices, others into up to 4;
+//     steps at 128 rows), so such products gain most from many slices (up to 8);
 //   - blocks run in rounds of what fits the chip at once; the operands have to come from memory
 //     once (5.5 TB/s) and the results have to go there (5 TB/s); a slice beyond the first costs
 //     its consumer one more pass over rows x width of float32.
@@ -714,12 +714,11 @@ static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
     DmaPlan best{0, 0, fixed_slices > 0 ? fixed_slices : 1};
     if (m <= 64 || !dma_tile_takes(m, n, k)) return best;
     double best_cost = 0.0;
-    for (int slices = 1; slices <= 8; slices *= 2) {
+    for (int slices : {1, 2, 3, 4, 6, 8}) {                 // (3 and 6: a K of 27 or 9 times 256 has no other cut)
         if (fixed_slices > 0 && slices != fixed_slices) continue;
         if (k % (128 * slices) != 0 || (slices > 1 && k / slices < 512)) continue;
         for (int bm = 256; bm >= 128; bm /= 2) {
             const int tiles_m = (m + bm - 1) / bm;
-            if (slices > 4 && tiles_m > 2) continue;
             for (int tn = 4; tn >= 2; --tn) {
                 if (tn == 3 && bm != 256) continue;
                 const int bn = 64 * tn;
