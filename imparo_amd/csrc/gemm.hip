@@ -107,6 +107,74 @@ __global__ __launch_bounds__(256) void k_gemm_f32(const float* __restrict__ X, c
     }
 }
 
+// The same sums for at most 16 rows (a decode step in the float32 engine): the tile above would
+// leave three quarters of its rows empty and, with a weight of few rows, most CUs idle. A block
+// takes 32 weight rows; thread (row, pair of weight rows) adds k = 0, 1, 2, ... exactly as the
+// tile kernel does, so a token's sums are the same bits whichever kernel its batch met. The next
+// chunk of K is asked for before the current one is multiplied.
+#define F32R_BN 32
+#define F32R_BK 64
+template <typename TOut>
+__global__ __launch_bounds__(256) void k_gemm_f32_rows(const float* __restrict__ X, const float* __restrict__ W,
+                                                       const float* __restrict__ bias, TOut* __restrict__ Y,
+                                                       int M, int N, int K, int epilogue) {
+    __shared__ float Ws[F32R_BK][F32R_BN + 1];
+    __shared__ float Xs[F32R_BK][16 + 1];
+    const int tid = threadIdx.x;
+    const int tx = tid % 16, ty = tid / 16;
+    const int n0 = blockIdx.x * F32R_BN;
+    float acc0 = 0.f, acc1 = 0.f;
+    float wr[8], xr[4];
+    auto fetch = [&](int k0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {                    // 32 weight rows x 64 k, a row's 64 values side by side
+            const int e = tid + j * 256;
+            const int r = e / F32R_BK, k = k0 + e % F32R_BK;
+            wr[j] = (n0 + r < N && k < K) ? W[(size_t)(n0 + r) * K + k] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {                    // 16 activation rows x 64 k
+            const int e = tid + j * 256;
+            const int r = e / F32R_BK, k = k0 + e % F32R_BK;
+            xr[j] = (r < M && k < K) ? X[(size_t)r * K + k] : 0.f;
+        }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += F32R_BK) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int e = tid + j * 256;
+            Ws[e % F32R_BK][e / F32R_BK] = wr[j];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int e = tid + j * 256;
+            Xs[e % F32R_BK][e / F32R_BK] = xr[j];
+        }
+        __syncthreads();
+        fetch(k0 + F32R_BK);                             // (past the end: nothing is read, zeros)
+#pragma unroll 16
+        for (int kk = 0; kk < F32R_BK; ++kk) {
+            const float a = Xs[kk][ty];
+            acc0 = fmaf(a, Ws[kk][2 * tx], acc0);
+            acc1 = fmaf(a, Ws[kk][2 * tx + 1], acc1);
+        }
+        __syncthreads();
+    }
+    const int m = ty, n = n0 + 2 * tx;
+    if (m >= M) return;
+    if (bias) {
+        if (n < N) acc0 += bias[n];
+        if (n + 1 < N) acc1 += bias[n + 1];
+    }
+    if (epilogue == EPI_SWIGLU) {
+        if (n + 1 < N) store_f32<TOut>(Y, (size_t)m * (N / 2) + n / 2, silu_mul_f(acc0, acc1));
+        return;
+    }
+    if (n < N) store_f32<TOut>(Y, (size_t)m * N + n, acc0);
+    if (n + 1 < N) store_f32<TOut>(Y, (size_t)m * N + n + 1, acc1);
+}
+
 // ------------------------------------------------------------------ bfloat16, many rows
 // 128x128 output tile per block of four waves (2x2, 64x64 each as 2x2 MFMA
 // tiles of 32x32x16), K in steps of 64. Global loads run three K-steps ahead
@@ -1376,6 +1444,16 @@ extern "C" int imparo_gemm(const void* x, const void* w, const float* bias, void
     if (m == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;
     if (dtype == IMPARO_F32) {
+        if (m <= 16 && out_dtype == IMPARO_F32) {
+            k_gemm_f32_rows<float><<<(n + F32R_BN - 1) / F32R_BN, 256, 0, s>>>((const float*)x, (const float*)w, bias,
+                                                                             (float*)y, m, n, k, epilogue);
+            return launch_status();
+        }
+        if (m <= 16 && out_dtype == IMPARO_BF16) {
+            k_gemm_f32_rows<bf16_t><<<(n + F32R_BN - 1) / F32R_BN, 256, 0, s>>>((const float*)x, (const float*)w, bias,
+                                                                              (bf16_t*)y, m, n, k, epilogue);
+            return launch_status();
+        }
         dim3 grid((n + F32_BN - 1) / F32_BN, (m + F32_BM - 1) / F32_BM);
         if (grid.y > 65535) return IMPARO_BAD_ARGUMENT;
         if (out_dtype == IMPARO_F32)
