@@ -46,6 +46,18 @@ def test_gemm(m, n, k):
     assert torch.equal(outb.cpu(), out.cpu().to(torch.bfloat16))      # only the final rounding differs
 
 
+def test_float32_gemm_sums_the_same_way_for_few_rows_and_many():
+    """Up to 16 rows take a kernel of their own: a row's results are the same bits as in a batch of 40."""
+    x, w, b = rnd(40, 1000, seed=1), rnd(210, 1000, seed=2, scale=0.3), rnd(210, seed=3)
+    for swiglu in (False, True):
+        many = torch.empty(40, 105 if swiglu else 210, device=DEV)
+        ops().gemm(x.to(DEV), w.to(DEV), many, bias=b.to(DEV), swiglu=swiglu)
+        for rows in (1, 7, 16):
+            few = torch.empty(rows, many.shape[1], device=DEV)
+            ops().gemm(x[:rows].to(DEV), w.to(DEV), few, bias=b.to(DEV), swiglu=swiglu)
+            assert torch.equal(few, many[:rows])
+
+
 @pytest.mark.parametrize("m", [1, 20, 64, 150])
 def test_gemm_epilogues(m):
     """A bias, and the SwiGLU epilogue over a weight whose rows alternate gate and up, in the
