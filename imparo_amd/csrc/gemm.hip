@@ -527,11 +527,11 @@ static int launch_big(const bf16_t* x, const bf16_t* w, const float* bias, TOut*
 }
 
 // ------------------------------------------------------------------ bfloat16, many rows, loads straight into LDS
-// A tile of 256 or 128 activation rows by 256, 192 or 128 weight rows. The 256 and the 128 wide tile
-// take eight waves, two per SIMD, each with 128 (or 64) rows by 64 or 32 (4x2 or 4x1 MFMA tiles of 32x32,
-// 128 or 64 accumulator registers; half of that with 128 activation rows), so that one's products run while the other waits or writes
-// its results (12% faster than four waves of 128x128 on the gate/up product at 2,048 rows, 5 to
-// 15% on the narrow tile); the 192 wide tile four waves of 128 by 96, one per SIMD. The operands never pass through registers
+// A tile of 256 or 128 activation rows by 256, 192 or 128 weight rows on eight waves, two per
+// SIMD, so that one's products run while the other waits or writes its results (12% faster than
+// four waves of 128x128 on the gate/up product at 2,048 rows, 5 to 15% on the narrower tiles).
+// A wave has 128 (or 64) rows by 64 or 32 of it, 4x2 or 4x1 MFMA tiles of 32x32 (2x2, 2x1 with
+// 128 activation rows); the 192 wide tile's waves 64 rows by 96 (2x3). The operands never pass through registers
 // on their way in: global_load_lds writes 16 bytes per
 // lane straight into LDS, a wave's 64 lanes to 1 KB in a row. LDS rows are the 128 bytes of
 // a K-step without padding, so the eight 16-byte pieces of row r are stored in the order
@@ -565,21 +565,19 @@ __device__ __forceinline__ void load_to_lds(const bf16_t* src, bf16_t* dst_wave_
                                      (void __attribute__((address_space(3)))*)dst_wave_uniform, 16, 0, 0);
 }
 
-// TN: MFMA tiles across a wave's part of the weight rows. The launcher chooses the tile's width so
-// that the blocks come out in whole rounds of the CUs.
-// NWN: waves across the weight rows (2: four waves, one per SIMD; 4: eight waves, two per SIMD, each
-// with half the accumulators, so that one's products run while the other waits).
-// TMI: MFMA tiles down a wave's part of the activation rows (4: the block takes 256 rows, 2: 128).
-template <typename TOut, int TMI, int TN, int NWN>
-__global__ __launch_bounds__(128 * NWN) void k_gemm_bf16_dma(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+// TMI, TN: MFMA tiles of 32x32 down a wave's part of the activation rows and across its part of
+// the weight rows; NWM, NWN: waves down and across (eight in all). The launcher's plan chooses
+// the tile so that the blocks come out in whole rounds of the CUs.
+template <typename TOut, int TMI, int TN, int NWN, int NWM = 2>
+__global__ __launch_bounds__(64 * NWM * NWN) void k_gemm_bf16_dma(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                              const float* __restrict__ bias, TOut* __restrict__ Y,
                                                              int M, int N, int K_all, int k_per, int tiles_m,
                                                              int tiles_n, int epilogue) {
-    constexpr int NW = 2 * NWN;                        // waves of the block
+    constexpr int NW = NWM * NWN;                      // waves of the block
     constexpr int WN = 32 * TN;                        // weight rows of one wave's part
     constexpr int BN = NWN * WN;                       // of the block's tile
     constexpr int WM = 32 * TMI;                       // activation rows of one wave's part
-    constexpr int BM = 2 * WM;                         // of the block's tile
+    constexpr int BM = NWM * WM;                       // of the block's tile
     constexpr int LX = BM / (8 * NW), LW = BN / (8 * NW);   // load instructions per wave and K-step
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "the waves share the tile's rows evenly");
     __shared__ __attribute__((aligned(1024))) bf16_t stage0[(BM + BN) * DM_BK];   // X rows, then W rows
@@ -698,8 +696,8 @@ __global__ __launch_bounds__(128 * NWN) void k_gemm_bf16_dma(const bf16_t* __res
     // stores. A staged row is 136 floats: the two rows a store instruction touches, 4 apart,
     // fall on disjoint banks. Each wave has a region of its own, so no barrier between passes.
     __syncthreads();                                   // every wave is done with the operands in LDS
-    constexpr int EP_LD = NWN == 2 ? 136 : WN + 8;
-    constexpr int LPR = (NWN == 2 || 64 % (WN / 4)) ? 32 : WN / 4;   // lanes to a staged row
+    constexpr int EP_LD = (NWN == 2 && NWM == 2) ? 136 : WN + 8;
+    constexpr int LPR = ((NWN == 2 && NWM == 2) || 64 % (WN / 4)) ? 32 : WN / 4;   // lanes to a staged row
     static_assert((4 * EP_LD) % 64 == 32 && NW / 2 * 32 * EP_LD * 4 <= (BM + BN) * DM_BK * 2, "staging layout");
     float* staged = reinterpret_cast<float*>(wave >= NW / 2 ? stage1 : stage0) + (wave % (NW / 2)) * (32 * EP_LD);
     const int out_col = (lane % LPR) * 4;              // of the wave's columns: lanes past them (narrow tiles) sit out
@@ -762,8 +760,7 @@ static bool dma_tile_takes(int m, int n, int k) {
 // does not take). A model of the time, fitted to this machine (it picks the fastest or one within
 // a few percent of it on every shape measured, 128 to 4,096 rows):
 //   - a block alone on its CU takes 0.11 us + 0.0155 us per MFMA of a SIMD for a K-step of 64
-//     (bm * bn / 1024 of them), and 5 us + 0.03 us per such MFMA for its beginning and end
-//     (the 192 wide tile on four waves: 0.62 us a step, 16 us for beginning and end);
+//     (bm * bn / 1024 of them), and 5 us + 0.03 us per such MFMA for its beginning and end;
 //   - two blocks fit a CU where their stages take 80 KB or less each (the 128x128 tile), and a
 //     step then takes what the products of both take;
 //   - the more CUs are busy the slower each runs (clocks, L2): up to 45% with all 256, and more
@@ -798,11 +795,10 @@ static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
                 const double per_cu = (double)((per_round + (long long)cus - 1) / (long long)cus);
                 const double mfmas = bm * bn / 1024.0;
                 const double small = 1.0 + 0.1 * (256.0 / bm - 1.0) + 0.1 * (256.0 / bn - 1.0);
-                // (the 192 wide tile's four waves take their steps faster and their beginning and end slower)
-                double step = (tn == 3 ? 0.62 : std::max(0.11 + 0.0155 * mfmas, per_cu * 0.0155 * mfmas)) *
+                double step = std::max(0.11 + 0.0155 * mfmas, per_cu * 0.0155 * mfmas) *
                               (1.0 + 0.45 * cus / 256.0 * small);
                 if (tiles_m <= 2) step = std::max(step, 1.0);     // nobody has read these weights before: memory is far
-                const double ends = tn == 3 ? 16.0 : 5.0 + 0.03 * mfmas;
+                const double ends = 5.0 + 0.03 * mfmas;
                 const double from_memory = ((double)m + n) * k * 2.0 / 5.5e6;
                 const double cost = std::max(rounds * (k / slices / DM_BK * step + ends), from_memory + ends) +
                                     (double)slices * m * n * 4.0 / 5e6 + (slices - 1) * ((double)m * n * 4.0 / 5e6);
@@ -833,8 +829,8 @@ static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TOut*
         DMA_GO(2, 1, 4);
     else if (tn == 4)     // 256 wide: eight waves
         DMA_GO(4, 2, 4);
-    else if (tn == 3)
-        DMA_GO(4, 3, 2);
+    else if (tn == 3)     // 192 wide: eight waves of 64 rows by 96
+        k_gemm_bf16_dma<TOut, 2, 3, 2, 4><<<grid, 512, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
     else                  // 128 wide: eight waves
         DMA_GO(4, 1, 4);
 #undef DMA_GO
