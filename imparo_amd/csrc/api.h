@@ -1,7 +1,7 @@
 // C entry points of the gfx950 kernel library. Every pointer is device memory
 // unless named host_*. Every entry validates its sizes, launches on `stream`
-// and returns IMPARO_OK, IMPARO_BAD_ARGUMENT (nothing launched) or
-// IMPARO_LAUNCH_FAILED. dtype codes: 0 = float32, 1 = bfloat16.
+// and returns IMPARO_OK (0), IMPARO_BAD_ARGUMENT (1, nothing launched) or
+// IMPARO_LAUNCH_FAILED (2). dtype codes: 0 = float32, 1 = bfloat16.
 #pragma once
 #include <stdint.h>
 
@@ -82,6 +82,24 @@ int imparo_attention_decode(const void* q, const void* k_cache, const void* v_ca
                             const int32_t* block_table, int table_stride, int page_size,
                             int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
                             int n_splits, imparo_stream stream);
+
+// imparo_attention_decode for callers that cannot allocate device memory: code under HIP graph
+// capture, tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the
+// reference. The splits' partial results go through a buffer of IMPARO_STATIC_SCRATCH_BYTES that the
+// library holds itself on every GPU it runs on (until the process ends) instead of part_o / part_ml;
+// the call allocates and frees nothing. rows x heads x n_splits x (head_dim + 2) floats (the first
+// part rounded up to 64 floats) must fit, else nothing is launched, a line on stderr says what was
+// asked for, and IMPARO_SCRATCH_TOO_SMALL (3) is returned. All calls on one GPU share that GPU's
+// buffer: calls that overlap there (two streams, two threads) race; calls on one stream do not.
+// The buffer keeps the last call's contents; no call relies on them. The first call on a device
+// looks the buffer's address up (no allocation, but not a stream operation: make it outside a capture).
+#define IMPARO_STATIC_SCRATCH_BYTES (16u << 20)
+int imparo_attention_decode_static(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                   const int32_t* rows, int n_rows,
+                                   const int32_t* seg_start, const int32_t* positions,
+                                   const int32_t* block_table, int table_stride, int page_size,
+                                   int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
+                                   int n_splits, imparo_stream stream);
 
 // Prompt portions: the listed rows' segments in tiles of 64 queries;
 // n_tiles = sum over the rows of ceil(seg_len / 64). n_splits (from

@@ -14,6 +14,9 @@
 #include "common.h"
 
 #include <algorithm>
+#include <atomic>
+#include <cstdio>
+#include <mutex>
 #include "api.h"
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -951,6 +954,24 @@ static int check_common(const void* q, const void* k_cache, const void* v_cache,
         default: return IMPARO_BAD_ARGUMENT;                                                                         \
     }
 
+static int attention_decode_launch(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                   float* part_o, float* part_ml, const int32_t* rows, int n_rows,
+                                   const int32_t* seg_start, const int32_t* positions,
+                                   const int32_t* block_table, int table_stride, int page_size,
+                                   int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
+                                   int n_splits, hipStream_t s) {
+    const int G = heads / kv_heads;
+    dim3 grid(n_splits, kv_heads * ((G + 15) / 16), n_rows);
+    DISPATCH_ND(head_dim / 16, (k_attn_decode<ND><<<grid, MFMA_WAVES * 64, 0, s>>>(
+        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, part_o, part_ml, (bf16_t*)out, rows, seg_start,
+        positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, n_splits)));
+    if (launch_status()) return IMPARO_LAUNCH_FAILED;
+    if (n_splits == 1) return IMPARO_OK;
+    k_attn_decode_merge<<<n_rows * heads, 64, 0, s>>>(part_o, part_ml, (bf16_t*)out, rows, seg_start, positions, heads,
+                                                      head_dim, n_splits, window);
+    return launch_status();
+}
+
 extern "C" int imparo_attention_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
                                        float* part_o, float* part_ml, const int32_t* rows, int n_rows,
                                        const int32_t* seg_start, const int32_t* positions,
@@ -963,17 +984,75 @@ extern "C" int imparo_attention_decode(const void* q, const void* k_cache, const
     if (!part_o || !part_ml || n_rows < 0 || n_splits <= 0 || n_splits > 65535) return IMPARO_BAD_ARGUMENT;
     if (n_rows == 0) return IMPARO_OK;
     if (n_rows > 65535) return IMPARO_BAD_ARGUMENT;
-    hipStream_t s = (hipStream_t)stream;
-    const int G = heads / kv_heads;
-    dim3 grid(n_splits, kv_heads * ((G + 15) / 16), n_rows);
-    DISPATCH_ND(head_dim / 16, (k_attn_decode<ND><<<grid, MFMA_WAVES * 64, 0, s>>>(
-        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, part_o, part_ml, (bf16_t*)out, rows, seg_start,
-        positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, n_splits)));
-    if (launch_status()) return IMPARO_LAUNCH_FAILED;
-    if (n_splits == 1) return IMPARO_OK;
-    k_attn_decode_merge<<<n_rows * heads, 64, 0, s>>>(part_o, part_ml, (bf16_t*)out, rows, seg_start, positions, heads,
-                                                      head_dim, n_splits, window);
-    return launch_status();
+    return attention_decode_launch(q, k_cache, v_cache, out, part_o, part_ml, rows, n_rows, seg_start, positions,
+                                   block_table, table_stride, page_size, heads, kv_heads, head_dim, n_pages, scale,
+                                   window, n_splits, (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------- decode without a workspace argument
+// The splits' partial results live in an array of this library's own instead of a buffer the caller
+// brings, so that the call allocates nothing. Every GPU holds its own copy of the array at its own
+// address: the address is asked for once per device, with that device current, and kept. In host code
+// the array's name is only a stand-in for the symbol, never a device address; kernels and copies get
+// the kept pointer.
+static __device__ __align__(256) float scratch[IMPARO_STATIC_SCRATCH_BYTES / sizeof(float)];
+
+static constexpr int SCRATCH_DEVICES = 64;
+static std::mutex scratch_mutex;
+static std::atomic<float*> scratch_of_device[SCRATCH_DEVICES];
+
+static int static_scratch(float** ptr) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SCRATCH_DEVICES) return IMPARO_LAUNCH_FAILED;
+    float* p = scratch_of_device[dev].load(std::memory_order_acquire);
+    if (!p) {
+        std::lock_guard<std::mutex> hold(scratch_mutex);
+        p = scratch_of_device[dev].load(std::memory_order_acquire);
+        if (!p) {
+            void* address = nullptr;
+            if (hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)) != hipSuccess || !address) {
+                (void)hipGetLastError();
+                return IMPARO_LAUNCH_FAILED;
+            }
+            p = static_cast<float*>(address);
+            scratch_of_device[dev].store(p, std::memory_order_release);
+        }
+    }
+    *ptr = p;
+    return IMPARO_OK;
+}
+
+extern "C" int imparo_attention_decode_static(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                              const int32_t* rows, int n_rows,
+                                              const int32_t* seg_start, const int32_t* positions,
+                                              const int32_t* block_table, int table_stride, int page_size,
+                                              int heads, int kv_heads, int head_dim, int n_pages, float scale,
+                                              int window, int n_splits, imparo_stream stream) {
+    const int bad = check_common(q, k_cache, v_cache, out, rows, seg_start, positions, block_table, table_stride,
+                                 page_size, heads, kv_heads, head_dim, n_pages, window);
+    if (bad) return bad;
+    if (n_rows < 0 || n_splits <= 0 || n_splits > 65535) return IMPARO_BAD_ARGUMENT;
+    if (n_rows == 0) return IMPARO_OK;
+    if (n_rows > 65535) return IMPARO_BAD_ARGUMENT;
+    // [rows, heads, splits, head_dim] partial outputs, then, at the next multiple of 64 floats,
+    // [rows, heads, splits, 2] maxima and sums
+    const unsigned long long slots = (unsigned long long)n_rows * heads * n_splits;
+    const unsigned long long o_floats = (slots * head_dim + 63) / 64 * 64;
+    if ((o_floats + slots * 2) * sizeof(float) > IMPARO_STATIC_SCRATCH_BYTES) {
+        fprintf(stderr, "imparo_attention_decode_static: %d rows x %d heads x %d splits of head size %d need %llu bytes "
+                        "for partial results, the library's own buffer holds %llu; use imparo_attention_decode with a "
+                        "workspace, or fewer rows a call\n", n_rows, heads, n_splits, head_dim,
+                (o_floats + slots * 2) * (unsigned long long)sizeof(float), (unsigned long long)IMPARO_STATIC_SCRATCH_BYTES);
+        return IMPARO_SCRATCH_TOO_SMALL;
+    }
+    float* base = nullptr;
+    const int st = static_scratch(&base);
+    if (st) return st;
+    // nothing here has to start at zero: the merge reads a (row, head, split) only if this call's
+    // first kernel wrote it
+    return attention_decode_launch(q, k_cache, v_cache, out, base, base + o_floats, rows, n_rows, seg_start, positions,
+                                   block_table, table_stride, page_size, heads, kv_heads, head_dim, n_pages, scale,
+                                   window, n_splits, (hipStream_t)stream);
 }
 
 // How the prompt kernel for head sizes in steps of 32 lays a launch out: heads of a kv head to a block,

@@ -7,6 +7,7 @@
 #define IMPARO_OK 0
 #define IMPARO_BAD_ARGUMENT 1
 #define IMPARO_LAUNCH_FAILED 2
+#define IMPARO_SCRATCH_TOO_SMALL 3
 
 // dtype codes shared with the Python side
 #define IMPARO_F32 0
