@@ -65,6 +65,9 @@ class ModelPlan:
     final_norm: PartSpec
     head: PartSpec
     stop_token_ids: tuple = ()
+    # a tensor name no part declares -> a declared one that a file may restate
+    # under it (a stored head beside a tied embedding): accepted only if equal
+    restated_tensors: Dict[str, str] = field(default_factory=dict)
 
     def validate(self) -> None:
         from .errors import Inconsistent

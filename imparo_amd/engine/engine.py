@@ -110,13 +110,17 @@ class Engine:
         if not torch.cuda.is_available():
             raise RuntimeError("imparo_amd runs on a GPU; none is visible to this process")
         self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise ValueError(f"imparo_amd runs on a GPU; {device!r} is none")
+        if self.device.index is None:       # "cuda" means the current one; tensors report an index
+            self.device = torch.device("cuda", torch.cuda.current_device())
         torch.cuda.set_device(self.device)
         self.dtype = DTYPES[dtype]
         self.model_dir = model_dir
         self.config_json = read_config_json(model_dir)
         self.config, self.plan = plan_from_config(self.config_json)
         declared = declared_tensors(self.plan)
-        tensors = load_weights(model_dir, {k: d for k, (d, _) in declared.items()})
+        tensors = load_weights(model_dir, {k: d for k, (d, _) in declared.items()}, self.plan.restated_tensors)
         self.model = Model(self.plan, tensors, self.device, self.dtype)
         f = tensors.pop("__file__", None)
         del tensors

@@ -127,6 +127,21 @@ class Scheduler:
             raise ValueError("a request needs at least one prompt token")
         r = Request(request_id, list(prompt), params, pending=list(prompt), arrival=self._arrivals)
         self._arrivals += 1
+        # a request the step function would refuse ends here, alone, instead of failing a step that
+        # carries other requests (the reference answers such a request with an error of its own before
+        # it reaches the engine, /root/reference/crates/imparo-server/src/main.rs:1981-1987)
+        vocab = getattr(self.engine, "vocab_size", None)
+        if vocab is not None:
+            bad = next((t for t in r.prompt if isinstance(t, bool) or not isinstance(t, int) or not 0 <= t < vocab),
+                       None)
+            if bad is not None:
+                self._finish(r, f"error: token id {bad!r} is outside the vocabulary of {vocab}")
+                return r
+        limit = getattr(self.engine, "max_position", None)
+        if limit is not None and len(r.prompt) + max(params.max_tokens, 1) - 1 > limit:
+            self._finish(r, f"error: {len(r.prompt)} prompt tokens and {params.max_tokens} new ones pass the "
+                            f"model's {limit} positions")
+            return r
         h = self.engine.cache.handle(request_id)
         rc = self._lib.imparo_sched_add(self._s, h, len(prompt), params.max_tokens)
         if rc == 1:
@@ -344,6 +359,8 @@ def generate(model, input_ids: Sequence[Sequence[int]], max_tokens: int = 16, te
     for i, prompt in enumerate(input_ids):
         sched.add(i, prompt, SamplingParams(temperature=temperature, max_tokens=max_tokens, seed=seed + i,
                                             stop_token_ids=stops))
+        if sched.finished.get(i) is not None and sched.finished[i].finish_reason.startswith("error"):
+            raise ValueError(f"request {i}: {sched.finished[i].finish_reason[7:]}")
     done = sched.run()
     for i in range(len(input_ids)):
         if done[i].finish_reason.startswith("error"):

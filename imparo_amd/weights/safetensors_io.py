@@ -57,9 +57,14 @@ class SafetensorsFile:
             count = 1
             for s in shape:
                 count *= s
-            if end - begin != count * torch.empty((), dtype=dtype).element_size() or self._base + end > size:
+            if (not 0 <= begin <= end or end - begin != count * torch.empty((), dtype=dtype).element_size()
+                    or self._base + end > size):
                 raise SafetensorsError(f"{path}: tensor {name!r} has inconsistent offsets")
             self.entries[name] = (dtype, shape, begin, end)
+        spans = sorted((b, e, name) for name, (_, _, b, e) in self.entries.items() if e > b)
+        for (b0, e0, n0), (b1, e1, n1) in zip(spans, spans[1:]):
+            if b1 < e0:
+                raise SafetensorsError(f"{path}: tensors {n0!r} and {n1!r} overlap in the file")
         self._map = mmap.mmap(self._file.fileno(), 0, access=mmap.ACCESS_READ) if size > 0 else None
 
     def names(self) -> List[str]:

@@ -121,16 +121,17 @@ def argmax_first(logits):
 
 
 def ff_dim_from_config(cfg):
-    """The SwiGLU width as config.json gives it: block_ff_dim, two thirds of it
-    times the multiplier rounded up to multiple_of when auto-adjust is on."""
-    if cfg.get("block_auto_adjust_ff_dim", False):
-        f = int(2 * cfg["block_ff_dim"] / 3)
+    """The SwiGLU width as config.json gives it: block_ff_dim (intermediate_size
+    where a file has only that), two thirds of it times the multiplier rounded
+    up to multiple_of unless auto-adjust is switched off."""
+    if cfg.get("block_auto_adjust_ff_dim", True):
+        f = int(2 * cfg.get("block_ff_dim", cfg.get("intermediate_size")) / 3)
         mult = cfg.get("block_ffn_dim_multiplier", 1.0)
         if mult is not None:
             f = int(mult * f)
         m = cfg.get("block_multiple_of", 256)
         return m * ((f + m - 1) // m)
-    return cfg.get("intermediate_size", cfg.get("block_ff_dim"))
+    return cfg.get("block_ff_dim", cfg.get("intermediate_size"))
 
 
 # --------------------------------------------------------------------------- model

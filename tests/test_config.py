@@ -39,7 +39,7 @@ def test_benchmark_shape():
 
 
 @pytest.mark.parametrize("key", ["vocab_size", "hidden_size", "num_hidden_layers", "layer_types",
-                                 "num_attention_heads", "num_key_value_heads", "conv_L_cache"])
+                                 "num_attention_heads", "num_key_value_heads", "conv_L_cache", "block_ff_dim"])
 def test_missing_key(key):
     d = copy.deepcopy(TINY_A)
     del d[key]
@@ -67,6 +67,92 @@ def test_inconsistent():
         Lfm2Config.from_dict(dict(TINY_A, conv_L_cache=1))
     with pytest.raises(Inconsistent, match="sliding_window"):
         Lfm2Config.from_dict(dict(TINY_A, layer_types=["conv", "sliding_attention", "conv", "full_attention"]))
+
+
+# ---- the spellings checkpoints of this architecture carry: each works or is refused by name
+def _without(d, *keys):
+    return {k: v for k, v in d.items() if k not in keys}
+
+
+def test_full_attn_idxs_stands_in_for_layer_types():
+    d = dict(_without(TINY_B, "layer_types"), full_attn_idxs=[2, 4, 5])
+    assert Lfm2Config.from_dict(d).layer_types == TINY_B["layer_types"]
+    # both, agreeing, is fine; disagreeing or out of range is refused
+    Lfm2Config.from_dict(dict(TINY_B, full_attn_idxs=[2, 4, 5]))
+    with pytest.raises(Inconsistent, match="full_attn_idxs"):
+        Lfm2Config.from_dict(dict(TINY_B, full_attn_idxs=[1, 4, 5]))
+    with pytest.raises(Inconsistent, match="full_attn_idxs"):
+        Lfm2Config.from_dict(dict(d, full_attn_idxs=[2, 9]))
+    with pytest.raises(BadValue, match="full_attn_idxs"):
+        Lfm2Config.from_dict(dict(d, full_attn_idxs="2,4,5"))
+    with pytest.raises(MissingKey, match="layer_types.*full_attn_idxs"):
+        Lfm2Config.from_dict(_without(TINY_B, "layer_types"))
+
+
+def test_rope_theta_inside_rope_parameters():
+    d = dict(_without(TINY_A, "rope_theta"), rope_parameters=dict(rope_theta=12345.0, rope_type="default"))
+    cfg, plan = plan_from_config(d)
+    assert cfg.rope_theta == 12345.0 and plan.layers[1].mixer["position"]["base"] == 12345.0
+    Lfm2Config.from_dict(dict(TINY_A, rope_parameters=dict(rope_theta=10000.0)))          # said twice, agreeing
+    with pytest.raises(Inconsistent, match="rope_theta"):
+        Lfm2Config.from_dict(dict(TINY_A, rope_parameters=dict(rope_theta=12345.0)))
+    with pytest.raises(BadValue, match="rope_type"):
+        Lfm2Config.from_dict(dict(d, rope_parameters=dict(rope_theta=1e4, rope_type="yarn")))
+    with pytest.raises(BadValue, match="factor"):
+        Lfm2Config.from_dict(dict(d, rope_parameters=dict(rope_theta=1e4, factor=4.0)))
+    with pytest.raises(BadValue, match="rope_scaling"):
+        Lfm2Config.from_dict(dict(TINY_A, rope_scaling=dict(type="linear", factor=2.0)))
+    assert Lfm2Config.from_dict(_without(TINY_A, "rope_theta")).rope_theta == 1000000.0  # the architecture's default
+
+
+def test_tie_word_embeddings_is_read():
+    d = dict(_without(TINY_A, "tie_embedding"), tie_word_embeddings=False)
+    cfg, plan = plan_from_config(d)
+    assert not cfg.tie_embedding and plan.head.prefix == "lm_head"
+    assert plan_from_config(dict(d, tie_word_embeddings=True))[1].head.prefix == "model.embed_tokens"
+    with pytest.raises(Inconsistent, match="tie_word_embeddings"):
+        Lfm2Config.from_dict(dict(TINY_A, tie_word_embeddings=False))
+    with pytest.raises(BadValue, match="tie_word_embeddings"):
+        Lfm2Config.from_dict(dict(d, tie_word_embeddings="no"))
+
+
+def test_eos_token_id_as_an_id_or_a_list():
+    assert plan_from_config(dict(TINY_A, eos_token_id=7))[1].stop_token_ids == (7,)
+    assert plan_from_config(dict(TINY_A, eos_token_id=[7, 2]))[1].stop_token_ids == (7, 2)
+    assert plan_from_config(TINY_A)[1].stop_token_ids == ()
+    for bad in ([], "7", [7, "2"], 7.0, True):
+        with pytest.raises(BadValue, match="eos_token_id"):
+            Lfm2Config.from_dict(dict(TINY_A, eos_token_id=bad))
+    with pytest.raises(Inconsistent, match="eos_token_id"):
+        Lfm2Config.from_dict(dict(TINY_A, eos_token_id=[7, 256]))
+
+
+def test_feed_forward_width_keys():
+    base = _without(TINY_B, "block_ff_dim", "block_auto_adjust_ff_dim")
+    # intermediate_size alone is the width before adjustment; adjustment is on unless the file says otherwise
+    assert Lfm2Config.from_dict(dict(base, intermediate_size=480)).ff_dim == 320
+    assert Lfm2Config.from_dict(dict(base, intermediate_size=480, block_auto_adjust_ff_dim=False)).ff_dim == 480
+    # block_ff_dim wins where a file carries both
+    assert Lfm2Config.from_dict(dict(base, intermediate_size=1000, block_ff_dim=480)).ff_dim == 320
+    assert Lfm2Config.from_dict(dict(base, intermediate_size=1000, block_ff_dim=480,
+                                     block_auto_adjust_ff_dim=False)).ff_dim == 480
+    with pytest.raises(MissingKey, match="block_ff_dim.*intermediate_size"):
+        Lfm2Config.from_dict(base)
+
+
+def test_restated_and_unsupported_keys_are_refused_and_unknown_ones_are_listed():
+    full = dict(TINY_A, block_dim=64, conv_dim=64, conv_dim_out=64, num_heads=4, block_norm_eps=1e-5, theta=10000.0,
+                block_use_swiglu=True, use_pos_enc=True, torch_dtype="bfloat16", bos_token_id=1, pad_token_id=0,
+                use_cache=True, initializer_range=0.02, transformers_version="x", block_mlp_init_scale=1.0)
+    assert Lfm2Config.from_dict(full).unread_keys == []
+    for key, value in (("block_dim", 128), ("conv_dim", 32), ("conv_dim_out", 32), ("num_heads", 8),
+                       ("block_norm_eps", 1e-6), ("theta", 5.0)):
+        with pytest.raises(Inconsistent, match=key):
+            Lfm2Config.from_dict(dict(full, **{key: value}))
+    for key, value in (("block_use_swiglu", False), ("use_pos_enc", False)):
+        with pytest.raises(BadValue, match=key):
+            Lfm2Config.from_dict(dict(full, **{key: value}))
+    assert Lfm2Config.from_dict(dict(full, some_new_switch=3)).unread_keys == ["some_new_switch"]
 
 
 def test_registry():

@@ -169,6 +169,26 @@ def test_zero_max_tokens_runs_nothing():
     assert s.run()["a"].generated == [] and eng.steps == []
 
 
+def test_a_request_the_step_function_would_refuse_ends_alone():
+    """A token outside the vocabulary, or a reply that would pass the model's
+    positions, ends that request with an error when it is added; the others run
+    as if it had never come and nothing of it is left in the cache."""
+    eng, s = make()
+    eng.vocab_size, eng.max_position = VOCAB, 40
+    s.add("good", [1, 2, 3], SamplingParams(max_tokens=5))
+    bad = s.add("bad id", [1, VOCAB, 3], SamplingParams(max_tokens=5))
+    long = s.add("too long", list(range(30)), SamplingParams(max_tokens=12))
+    fits = s.add("just fits", list(range(30)), SamplingParams(max_tokens=11))
+    assert bad.finished and "outside the vocabulary" in bad.finish_reason
+    assert long.finished and "positions" in long.finish_reason and not fits.finished
+    done = s.run()
+    assert done["good"].generated == expected([1, 2, 3], 5)
+    assert done["just fits"].generated == expected(list(range(30)), 11)
+    assert all(kind != "bad id" and kind != "too long" for step in eng.steps for kind, _, _ in step)
+    assert not eng.history and eng.cache.slots.n_free == eng.cache.n_slots
+    eng.cache.check()
+
+
 def test_waits_at_the_head_of_the_line_until_pages_free_up():
     # 6 pages of 4: a (prompt 12 -> 3 pages) runs; b needs 3 pages + 1 of headroom for a: waits
     eng, s = make(n_pages=6, max_batch_tokens=64, portion=64)

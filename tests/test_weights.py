@@ -114,3 +114,77 @@ def test_random_mode_is_seeded_and_has_the_stated_spreads(tmp_path):
     n = w1["model.layers.0.operator_norm.weight"].float()
     assert 0.9 <= n.min() and n.max() <= 1.1 and abs(n.mean().item() - 1.0) < 0.03
     assert abs(w1["model.layers.0.conv.in_proj.bias"].float().std().item() - 0.02) < 0.005
+
+
+def test_a_sharded_checkpoint_is_read_through_its_index(tmp_path):
+    d = str(tmp_path / "whole")
+    write_random_model(TINY_B, 1, d)
+    whole = load_weights(d, _declared(TINY_B))
+    names = sorted(_declared(TINY_B))
+    s = str(tmp_path / "sharded")
+    os.makedirs(s)
+    parts = {"model-00001-of-00003.safetensors": names[0::3], "model-00002-of-00003.safetensors": names[1::3],
+             "model-00003-of-00003.safetensors": names[2::3]}
+    for shard, held in parts.items():
+        save_file({n: whole[n] for n in held}, os.path.join(s, shard))
+    index = {"metadata": {}, "weight_map": {n: shard for shard, held in parts.items() for n in held}}
+    with open(os.path.join(s, "model.safetensors.index.json"), "w") as f:
+        json.dump(index, f)
+    got = load_weights(s, _declared(TINY_B))
+    for n in names:
+        assert torch.equal(got[n], whole[n])
+    # faults of a sharded folder come in the same one error, named after the index
+    del index["weight_map"][names[4]]
+    held = [n for n in parts["model-00002-of-00003.safetensors"] if n != names[4]]
+    save_file({n: whole[n] for n in held}, os.path.join(s, "model-00002-of-00003.safetensors"))
+    with open(os.path.join(s, "model.safetensors.index.json"), "w") as f:
+        json.dump(index, f)
+    with pytest.raises(WeightsError, match="index.json") as e:
+        load_weights(s, _declared(TINY_B))
+    assert e.value.missing == [names[4]]
+    # a shard the index names but the folder lacks
+    os.remove(os.path.join(s, "model-00003-of-00003.safetensors"))
+    with pytest.raises(FileNotFoundError, match="model-00003-of-00003"):
+        load_weights(s, _declared(TINY_B))
+    with pytest.raises(FileNotFoundError, match="neither"):
+        load_weights(str(tmp_path), _declared(TINY_B))
+
+
+def test_a_stored_head_beside_a_tied_embedding_must_equal_it(tmp_path):
+    from imparo_amd.config import plan_from_config
+    d = str(tmp_path / "m")
+    write_random_model(TINY_A, 0, d)
+    _, plan = plan_from_config(TINY_A)
+    assert plan.restated_tensors == {"lm_head.weight": "model.embed_tokens.weight"}
+    from safetensors.torch import load_file
+    t = load_file(os.path.join(d, "model.safetensors"))
+    t["lm_head.weight"] = t["model.embed_tokens.weight"].clone()
+    save_file(t, os.path.join(d, "model.safetensors"))
+    with pytest.raises(WeightsError) as e:          # nobody said what it may restate
+        load_weights(d, _declared(TINY_A))
+    assert e.value.unexpected == ["lm_head.weight"]
+    w = load_weights(d, _declared(TINY_A), plan.restated_tensors)
+    assert "lm_head.weight" not in w
+    t["lm_head.weight"][3, 5] += 1.0
+    save_file(t, os.path.join(d, "model.safetensors"))
+    with pytest.raises(WeightsError) as e:
+        load_weights(d, _declared(TINY_A), plan.restated_tensors)
+    assert e.value.unexpected == ["lm_head.weight"]
+    # an untied model has no such allowance: it declares its head
+    assert plan_from_config(TINY_B)[1].restated_tensors == {}
+
+
+def test_offsets_that_overlap_or_run_backwards_are_refused(tmp_path):
+    import struct
+    def write(path, header, n_bytes):
+        blob = json.dumps(header).encode()
+        with open(path, "wb") as f:
+            f.write(struct.pack("<Q", len(blob)) + blob + b"\0" * n_bytes)
+    p = str(tmp_path / "x.safetensors")
+    write(p, {"a": {"dtype": "F32", "shape": [2], "data_offsets": [0, 8]},
+              "b": {"dtype": "F32", "shape": [2], "data_offsets": [4, 12]}}, 12)
+    with pytest.raises(SafetensorsError, match="overlap"):
+        SafetensorsFile(p)
+    write(p, {"a": {"dtype": "F32", "shape": [2], "data_offsets": [-8, 0]}}, 8)
+    with pytest.raises(SafetensorsError, match="inconsistent offsets"):
+        SafetensorsFile(p)
