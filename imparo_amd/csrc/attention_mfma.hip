@@ -357,6 +357,22 @@ __global__ void k_attn_decode_merge(const float* __restrict__ part_o, const floa
 #define PF_LD_K(D) ((D) + 8)
 #define PF_LD_V (PF_KEYS + 8)
 
+// Later tiles of a prompt have more keys to walk, and blocks whose numbers differ by the number
+// of CUs tend to share a CU: every other run of 256 blocks (counted along x, then y) takes its
+// blocks in reverse, so that a long walk sits beside a short one. The reversal is inside a run
+// (the last run may be shorter), so every (tile, y) is still taken exactly once whatever the grid.
+__device__ __forceinline__ void snake_block(int& tile, int& by) {
+    const int gx = (int)gridDim.x, total = gx * (int)gridDim.y;
+    int linear = (int)blockIdx.y * gx + (int)blockIdx.x;
+    const int run = linear / 256;
+    if (run & 1) {
+        const int first = run * 256, last = min(first + 256, total) - 1;
+        linear = first + (last - linear);
+    }
+    by = linear / gx;
+    tile = linear - by * gx;
+}
+
 template <int ND>
 __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
@@ -369,11 +385,8 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
     const int page_shift = __ffs(page_size) - 1;          // a power of two: divisions by it are shifts
     __shared__ __attribute__((aligned(16))) bf16_t ks[2][PF_KEYS * LDK];
     __shared__ __attribute__((aligned(16))) bf16_t vs[2][D * PF_LD_V];
-    // Later tiles of a prompt have more keys to walk. Blocks whose numbers differ by the number
-    // of CUs tend to share a CU: every other group of 256 blocks takes the tiles in reverse, so
-    // that a long walk sits beside a short one.
-    int tile = blockIdx.x, row = -1;
-    if (((blockIdx.y * gridDim.x + blockIdx.x) / 256) & 1) tile = (int)gridDim.x - 1 - tile;
+    int tile, by, row = -1;
+    snake_block(tile, by);
     for (int i = 0; i < n_rows; ++i) {
         const int r = rows[i];
         const int nt = (seg_len[r] + 63) >> 6;
@@ -388,7 +401,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
     const int lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int len = seg_len[row];
-    const int head = blockIdx.y;
+    const int head = by;
     const int kvh = head / (heads / kv_heads);
     const int t0 = seg_start[row];
     const int pos0 = positions[t0];
@@ -595,8 +608,8 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     constexpr int QW = 16 * HALVES;                       // queries of a wave
     const int runs = MFMA_WAVES / heads_per_block;        // runs of QW queries per block
     const int qt = QW * runs;                             // queries per block and head
-    int tile = blockIdx.x, row = -1;
-    if (((blockIdx.y * gridDim.x + blockIdx.x) / 256) & 1) tile = (int)gridDim.x - 1 - tile;
+    int tile, by, row = -1;
+    snake_block(tile, by);
     for (int i = 0; i < n_rows; ++i) {
         const int r = rows[i];
         const int nt = (seg_len[r] + qt - 1) / qt;
@@ -611,8 +624,8 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     const int lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int len = seg_len[row];
-    const int head = blockIdx.y * heads_per_block + wave % heads_per_block;
-    const int kvh = (blockIdx.y * heads_per_block) / (heads / kv_heads);
+    const int head = by * heads_per_block + wave % heads_per_block;
+    const int kvh = (by * heads_per_block) / (heads / kv_heads);
     const int t0 = seg_start[row];
     const int pos0 = positions[t0];
     const int32_t* table = block_table + (size_t)row * table_stride;

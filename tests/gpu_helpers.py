@@ -68,6 +68,19 @@ def mixed_schedule(rng, lengths, max_live=4, sizes=(1, 1, 1, 2, 2, 3, 5, 9, 16, 
     return steps
 
 
+def peak_pages(steps, page_size: int) -> int:
+    """The most pages a schedule of mixed_schedule holds at any time (a request
+    holds ceil(fed / page_size) pages from its first step to its end)."""
+    held, peak = {}, 0
+    for entries, ends in steps:
+        for rid, lo, hi in entries:
+            held[rid] = -(-hi // page_size)
+        peak = max(peak, sum(held.values()))
+        for rid in ends:
+            del held[rid]
+    return peak
+
+
 def hand_context(segments: Sequence[Tuple[int, int]], page_size: int, n_pages: int, dtype, device,
                  kv_sites: Dict[int, Tuple[int, int]] = None, fixed_sites: Dict[int, Tuple[int, ...]] = None,
                  n_slots: int = 8, tables: List[List[int]] = None, slots: List[int] = None,

@@ -160,18 +160,28 @@ class PlainLfm2:
         self.theta = c.get("rope_theta", 1000000.0)
         self.bias = c.get("conv_bias", False)
 
-    def mixer_attention(self, i, h, positions, window, shared_kv=None):
+    def norm_and_rotate(self, x, weight, rope_positions):
+        """crates/imparo-model/src/cpu_support.rs:361-376 -- per (token, head):
+        the RMS norm over the head with one weight [D] for all heads FIRST,
+        then the rotation of the normed row."""
+        return rope_neox(rms_norm(x, weight, self.eps), rope_positions, self.theta, self.D)
+
+    def mixer_attention(self, i, h, positions, window, shared_kv=None, rope_positions=None):
         """Returns the mixer's output and the (k, v) it attended over; with
-        `shared_kv` the layer projects only q and reads another call's k, v."""
+        `shared_kv` the layer projects only q and reads another call's k, v.
+        `positions` index the request's own keys (0..T-1); `rope_positions`
+        are the angles' positions when they differ from those."""
         p = f"model.layers.{i}.self_attn."
         T = h.shape[0]
+        if rope_positions is None:
+            rope_positions = positions
         q = linear(h, self.w[p + "q_proj.weight"]).reshape(T, self.H, self.D)
-        # per-head norm, then rotation, on q and k; v untouched (cpu_support.rs:361-376)
-        q = rope_neox(rms_norm(q, self.w[p + "q_layernorm.weight"], self.eps), positions, self.theta, self.D)
+        # on q and k; v untouched (workflow_cpu.rs:209-229)
+        q = self.norm_and_rotate(q, self.w[p + "q_layernorm.weight"], rope_positions)
         if shared_kv is None:
             k = linear(h, self.w[p + "k_proj.weight"]).reshape(T, self.Hk, self.D)
             v = linear(h, self.w[p + "v_proj.weight"]).reshape(T, self.Hk, self.D)
-            k = rope_neox(rms_norm(k, self.w[p + "k_layernorm.weight"], self.eps), positions, self.theta, self.D)
+            k = self.norm_and_rotate(k, self.w[p + "k_layernorm.weight"], rope_positions)
         else:
             k, v = shared_kv
         o = attend(q, k, v, positions, 1.0 / math.sqrt(self.D), window)
@@ -184,12 +194,14 @@ class PlainLfm2:
         y, _ = short_conv(bcx, self.w[p + "conv.weight"], b("conv.bias"))
         return linear(y, self.w[p + "out_proj.weight"], b("out_proj.bias"))
 
-    def hidden(self, tokens, order=None):
+    def hidden(self, tokens, order=None, first_position=0):
         """`order`: list of (layer, cache_of) calls; None runs every layer once.
-        cache_of names an earlier call whose k, v this call reads."""
+        cache_of names an earlier call whose k, v this call reads.
+        `first_position` turns every rotation as if the sequence began there."""
         tokens = torch.as_tensor(tokens, dtype=torch.long)
         T = tokens.shape[0]
         positions = np.arange(T)
+        rope_positions = positions + first_position
         x = self.w["model.embed_tokens.weight"][tokens]
         if order is None:
             order = [(i, None) for i in range(len(self.cfg["layer_types"]))]
@@ -203,16 +215,17 @@ class PlainLfm2:
             else:
                 window = self.cfg.get("sliding_window") if kind == "sliding_attention" else None
                 m, kv_of_call[c] = self.mixer_attention(i, h, positions, window,
-                                                        None if cache_of is None else kv_of_call[cache_of])
+                                                        None if cache_of is None else kv_of_call[cache_of],
+                                                        rope_positions)
             x = x + m
             n = rms_norm(x, self.w[p + "ffn_norm.weight"], self.eps)
             x = x + swiglu(n, self.w[p + "feed_forward.w1.weight"], self.w[p + "feed_forward.w3.weight"],
                            self.w[p + "feed_forward.w2.weight"])
         return x
 
-    def logits(self, tokens, order=None):
+    def logits(self, tokens, order=None, first_position=0):
         """Logits [T, V] of one whole sequence from position 0."""
-        x = self.hidden(tokens, order)
+        x = self.hidden(tokens, order, first_position)
         head = self.w["model.embed_tokens.weight"] if self.cfg.get("tie_embedding", True) \
             else self.w["lm_head.weight"]
         return linear(rms_norm(x, self.w["model.embedding_norm.weight"], self.eps), head)

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from conftest import prompt_tokens
-from gpu_helpers import make_engine, mixed_schedule, RefCache, step_all
+from gpu_helpers import make_engine, mixed_schedule, peak_pages, RefCache, step_all
 from tolerances import check_logits
 
 pytestmark = pytest.mark.gpu
@@ -101,9 +101,14 @@ def test_mixed_batches_with_pages_used_again(zoo, engines, name, dtype):
     lengths = [70, 33, 121, 9, 64, 50, 97, 18]
     V = vocab_of(zoo, name)
     prompts = [prompt_tokens(V, n, 100 + i) for i, n in enumerate(lengths)]
-    # pages of 8; four live requests of up to 121 tokens need at most 4*16 pages: 40 forces reuse
-    eng = engines(name, dtype, page_size=8, max_tokens=40 * 8, max_requests=4)
+    # float32 on pages of 8; bfloat16 on pages of 16, the smallest the matrix-core attention kernels
+    # take, so that they meet portions beside single tokens on pages that were another request's.
+    # The pool is the schedule's peak: every page is in use at some time, and later requests get
+    # pages that earlier ones gave back.
+    page = 8 if dtype == "float32" else 16
     steps = mixed_schedule(rng, lengths)
+    n_pool = peak_pages(steps, page)
+    eng = engines(name, dtype, page_size=page, max_tokens=n_pool * page, max_requests=4)
     got = {i: [] for i in range(len(lengths))}
     used = set()
     for entries, ends in steps:
@@ -119,9 +124,9 @@ def test_mixed_batches_with_pages_used_again(zoo, engines, name, dtype):
         for rid in ends:
             eng.release(f"m{rid}")
         eng.cache.check()
-    total_pages_asked = sum((n + 7) // 8 for n in lengths)
-    assert total_pages_asked > 40 >= len(used), "the schedule must make requests share pages over time"
-    assert eng.free_pages() == [40] * len(eng.cache.groups)
+    total_pages_asked = sum((n + page - 1) // page for n in lengths)
+    assert total_pages_asked > n_pool >= len(used), "the schedule must make requests share pages over time"
+    assert eng.free_pages() == [n_pool] * len(eng.cache.groups)
     for rid, n in enumerate(lengths):
         check_logits(torch.cat(got[rid]), zoo[1][name](prompts[rid]), dtype, f"{name} mixed request {rid}")
 

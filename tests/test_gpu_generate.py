@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import prompt_tokens, ROOT
+from conftest import assert_varied, prompt_tokens, ROOT
 from tolerances import BF16_REL
 
 pytestmark = pytest.mark.gpu
@@ -47,6 +47,25 @@ def test_greedy_generation_tiny_a(model_dirs, plain_models):
     assert got == want
 
 
+def test_greedy_generation_follows_every_token(loud_model_dirs, loud_plain_models):
+    """The same workloads on models whose continuation moves with every token
+    (with the stated spreads it is one token repeated): greedy, whole and in
+    small portions under a small budget, Tiny B with its biases and its head."""
+    from imparo_amd import generate
+    for name, vocab, lens in (("A", 256, (5, 17, 31)), ("B", 384, (1, 9, 40, 63))):
+        prompts = [prompt_tokens(vocab, n, 40 + n) for n in lens]
+        want = [loud_plain_models[name].greedy(p, 16) for p in prompts]
+        assert_varied(want)
+        assert generate(loud_model_dirs[name], prompts, max_tokens=16, dtype="float32", page_size=8) == want
+        os.environ["IMPARO_BATCH"] = "4"
+        try:
+            got = generate(loud_model_dirs[name], prompts, max_tokens=16, dtype="float32", page_size=8,
+                           max_batch_tokens=9)
+        finally:
+            del os.environ["IMPARO_BATCH"]
+        assert got == want
+
+
 def test_greedy_generation_bfloat16_stays_on_a_best_token(model_dirs, plain_models):
     """In bfloat16 a near-tie may fall the other way; every token the engine
     picks must be the plain implementation's best up to the logit tolerance."""
@@ -81,12 +100,14 @@ def test_temperature_sampling_tiny_b(model_dirs, plain_models):
 
 
 @pytest.mark.parametrize("overlap", [False, True])
-def test_preemption_by_recompute_keeps_greedy_outputs(model_dirs, plain_models, overlap):
+def test_preemption_by_recompute_keeps_greedy_outputs(loud_model_dirs, loud_plain_models, overlap):
+    model_dirs, plain_models = loud_model_dirs, loud_plain_models
     from imparo_amd.engine import Engine
     from imparo_amd.engine.scheduler import Scheduler
     from imparo_amd.sampling import Sampler, SamplingParams
     prompts = [prompt_tokens(256, n, 80 + n) for n in (20, 22, 18)]
     want = [plain_models["A"].greedy(p, 20) for p in prompts]
+    assert_varied(want)          # a recompute that dropped or repeated a token would change what follows
     eng = Engine(model_dirs["A"], dtype="float32", page_size=8, max_tokens=10 * 8, max_requests=4)
     sampler = Sampler(eng.device)
     sched = Scheduler(eng, sampler.pick, max_batch_tokens=64, pick_async=sampler.pick_async if overlap else None)
@@ -98,15 +119,19 @@ def test_preemption_by_recompute_keeps_greedy_outputs(model_dirs, plain_models, 
     assert eng.free_pages() == [10]
 
 
-def test_stop_token_and_entry_point_defaults(model_dirs, plain_models):
+def test_stop_token_and_entry_point_defaults(loud_model_dirs, loud_plain_models):
     from imparo_amd import generate
     p = prompt_tokens(256, 12, 5)
-    full = plain_models["A"].greedy(p, 10)
-    got = generate(model_dirs["A"], [p], max_tokens=10, dtype="float32", stop_token_ids=[full[4]])
-    assert got == [full[:full.index(full[4])]]
+    full = loud_plain_models["A"].greedy(p, 10)
+    assert_varied([full])
+    at = next(i for i in range(3, 10) if full[i] not in full[:i])       # a token that comes first at place 3 or later
+    # the reply ends at the stop token, which is not handed out
+    got = generate(loud_model_dirs["A"], [p], max_tokens=10, dtype="float32", stop_token_ids=[full[at]])
+    assert got == [full[:at]]
 
 
-def test_waiting_after_every_step_generates_the_same(model_dirs, plain_models):
+def test_waiting_after_every_step_generates_the_same(loud_model_dirs):
+    model_dirs = loud_model_dirs
     """By default a step is queued before the tokens of the step before are read back (they
     are fed from the device); overlap=False waits after every step. Same tokens either way:
     greedy and sampled, with a stop token that is noticed a step late, in both dtypes."""
@@ -126,9 +151,11 @@ def test_waiting_after_every_step_generates_the_same(model_dirs, plain_models):
             assert a == b and len(a[0]) <= 3 and all(t not in stops for out in a for t in out)
 
 
-def test_command_line(model_dirs, plain_models, tmp_path):
+def test_command_line(loud_model_dirs, loud_plain_models, tmp_path):
+    model_dirs = loud_model_dirs
     p = prompt_tokens(256, 9, 3)
-    want = plain_models["A"].greedy(p, 6)
+    want = loud_plain_models["A"].greedy(p, 6)
+    assert_varied([want])
     env = dict(os.environ, PYTHONPATH=ROOT)
     r = subprocess.run([sys.executable, "-m", "imparo_amd", "generate", "-m", model_dirs["A"], "--dtype", "float32",
                         "--input-ids", ",".join(map(str, p)), "--max-tokens", "6", "-np", "2", "-c", "64"],

@@ -428,6 +428,19 @@ def test_attention(H, Hk, D, page_size, window):
     torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)      # one rounding of the output, P in float32
 
 
+@pytest.mark.parametrize("H,Hk,D", [(32, 8, 64), (24, 8, 48), (28, 4, 32), (9, 3, 80)])
+def test_matrix_core_attention_grids_of_any_width(H, Hk, D):
+    """Sixteen fresh prompts in one launch: more than 256 blocks, in rows of the grid whose width
+    does not divide 256. Every (tile, head) must be taken exactly once however the blocks are
+    ordered (an output nobody wrote stays NaN)."""
+    lens = (64, 63, 1, 47, 38, 23, 70, 85, 36, 15, 4, 32, 50, 54, 33, 65)
+    got, ref = _attention_case(H, Hk, D, 64, None, torch.bfloat16, kernel="mfma", ctx_lens=lens, q_lens=lens)
+    torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)
+    lens = (300, 1, 129, 77, 191)                 # several tiles a row
+    got, ref = _attention_case(H, Hk, D, 16, 100, torch.bfloat16, kernel="mfma", ctx_lens=lens, q_lens=lens)
+    torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)
+
+
 @pytest.mark.parametrize("H,Hk,D", [(1, 1, 16), (6, 2, 48), (5, 5, 64), (8, 1, 128), (4, 2, 80), (40, 2, 32),
                                     (6, 3, 64), (12, 3, 96)])
 @pytest.mark.parametrize("page_size,window", [(16, None), (64, None), (32, 19), (16, 64), (16, 1), (128, 300)])

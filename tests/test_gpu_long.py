@@ -7,7 +7,7 @@ import random
 import pytest
 import torch
 
-from conftest import prompt_tokens
+from conftest import assert_varied, prompt_tokens
 from gpu_helpers import make_engine
 from tolerances import check_logits
 
@@ -55,7 +55,19 @@ def test_long_context_bfloat16_against_float32(long_model):
     check_logits(runs["bfloat16"], runs["float32"], "bfloat16", "long context")
 
 
-def test_serving_workload_under_page_pressure(long_model):
+@pytest.fixture(scope="module")
+def loud_long_model(tmp_path_factory):
+    """The same shape with louder layers: a request's continuation then moves
+    with every token, so an output that survived pre-emption, waiting and
+    batching was recomputed from the right tokens and the right state."""
+    from imparo_amd import write_random_model
+    d = str(tmp_path_factory.mktemp("loud_long"))
+    write_random_model(LONG, 5, d, layer_gain=8.0)
+    return d
+
+
+def test_serving_workload_under_page_pressure(loud_long_model):
+    long_model = loud_long_model
     """32 requests in waves, prompts of 20..600 tokens, 5..40 new tokens each, a pool that holds
     about a third of them at once: every output equals the request's output when it runs alone."""
     from imparo_amd.engine import Engine
@@ -77,7 +89,9 @@ def test_serving_workload_under_page_pressure(long_model):
     assert any(e[0] == "preempt" for e in sched.log) and any(e[0] == "wait" for e in sched.log)
     assert eng.free_pages() == [200, 200] and eng.cache.slots.n_free == 12
     alone = Engine(long_model, dtype="float32", page_size=16, max_tokens=1024, max_requests=2)
-    for i in rng.sample(range(32), 10):
+    checked = rng.sample(range(32), 10)
+    assert_varied([sched.finished[i].generated for i in checked if reqs[i][1] >= 8])
+    for i in checked:
         prompt, n = reqs[i]
         assert sched.finished[i].finish_reason == "length"
         assert sched.finished[i].generated == generate(alone, [prompt], max_tokens=n)[0], f"request {i}"

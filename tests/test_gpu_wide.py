@@ -3,11 +3,13 @@ heads, feed-forward 8192, vocabulary 65536) with few layers, so that the plain
 implementation can follow on the CPU: the kernels' paths for these sizes (the
 128x128 MFMA tiles, the wide few-row products, the float4 norm, matrix-core
 attention at head size 64, pages of 64) are compared end to end."""
+import random
+
 import pytest
 import torch
 
 from conftest import prompt_tokens
-from gpu_helpers import make_engine, step_all
+from gpu_helpers import make_engine, mixed_schedule, peak_pages, step_all
 from tolerances import check_logits
 
 pytestmark = pytest.mark.gpu
@@ -30,12 +32,12 @@ def wide(tmp_path_factory):
     write_random_model(WIDE, 2, d)
     plain = PlainLfm2(d)
     toks = prompt_tokens(65536, 200, 77)
-    return d, toks, plain.logits(toks)
+    return d, toks, plain.logits(toks), plain
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_benchmark_width_layers(wide, dtype):
-    d, toks, ref = wide
+    d, toks, ref, _ = wide
     eng = make_engine(d, dtype, page_size=64, max_tokens=1024, max_requests=4)
     check_logits(step_all(eng, "w", toks, [200]), ref, dtype, "wide whole")
     eng.release("w")
@@ -43,3 +45,71 @@ def test_benchmark_width_layers(wide, dtype):
     got = step_all(eng, "p", toks, [60] + [1] * 10 + [100, 2, 28])
     check_logits(got, ref, dtype, "wide portions and single tokens")
     eng.release("p")
+
+
+def _logits_at(plain, tokens, rows):
+    """The plain implementation's logits at some places of a sequence (the head over a
+    vocabulary of 65,536 is most of its time, so only where they are compared)."""
+    import plain_lfm2 as P
+    x = plain.hidden(tokens)[rows]
+    return P.linear(P.rms_norm(x, plain.w["model.embedding_norm.weight"], plain.eps),
+                    plain.w["model.embed_tokens.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("live", [24, 64])
+def test_many_decoding_requests_at_benchmark_width(wide, dtype, live):
+    """24 and 64 live requests of different contexts decode six tokens each, every row held
+    to the plain implementation: the step run launch by launch, the captured one and its
+    replays. Beyond 16 rows the few-row products take more weight rows a block, the conv
+    mixer takes two launches instead of the fused one, and the captured graph is another."""
+    from imparo_amd.engine import StepEntry
+    d, _, _, plain = wide
+    rng = random.Random(live)
+    contexts = [rng.randint(1, 90) for _ in range(live)]
+    contexts[0], contexts[1], contexts[2] = 64, 63, 1            # a page's edge among them
+    seqs = [prompt_tokens(65536, c + 6, 300 + i) for i, c in enumerate(contexts)]
+    want = [_logits_at(plain, s, list(range(c, c + 6))) for s, c in zip(seqs, contexts)]
+    eng = make_engine(d, dtype, page_size=64, max_tokens=live * 128, max_requests=live)
+    for lo in range(0, live, 16):                                 # prompts, sixteen requests a step
+        eng.step([StepEntry(i, seqs[i][:contexts[i]], []) for i in range(lo, min(live, lo + 16))])
+    for j in range(6):
+        out = eng.step([StepEntry(i, [seqs[i][contexts[i] + j]], [0]) for i in range(live)]).cpu()
+        ref = torch.stack([w[j] for w in want])
+        check_logits(out, ref, dtype, f"{live} decoding rows, step {j}")
+    assert not eng.use_graphs or len(eng._graphs) == 1           # steps 1.. ran from one captured graph
+    for i in range(live):
+        eng.release(i)
+    assert eng.free_pages() == [eng.cache.groups[0].pool.n_pages]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_batches_at_benchmark_width_with_pages_used_again(wide, dtype):
+    """Up to four live requests, portions of some beside decoded tokens of others, pages of 64
+    and a pool no larger than the schedule's peak, so that later requests get earlier ones' pages."""
+    from imparo_amd.engine import StepEntry
+    d, _, _, plain = wide
+    rng = random.Random(5)
+    lengths = [150, 70, 200, 40, 130, 90, 65]
+    prompts = [prompt_tokens(65536, n, 400 + i) for i, n in enumerate(lengths)]
+    steps = mixed_schedule(rng, lengths, sizes=(1, 1, 1, 2, 3, 17, 40, 64, 100))
+    pool = peak_pages(steps, 64)
+    assert sum((n + 63) // 64 for n in lengths) > pool
+    eng = make_engine(d, dtype, page_size=64, max_tokens=pool * 64, max_requests=4)
+    got = {i: [] for i in range(len(lengths))}
+    kinds = set()
+    for entries, ends in steps:
+        sizes = [hi - lo for _, lo, hi in entries]
+        kinds.add((any(n == 1 for n in sizes), any(n > 1 for n in sizes)))
+        out = eng.step([StepEntry(f"m{rid}", prompts[rid][lo:hi], list(range(hi - lo))) for rid, lo, hi in entries]).cpu()
+        at = 0
+        for rid, lo, hi in entries:
+            got[rid].append(out[at:at + hi - lo])
+            at += hi - lo
+        for rid in ends:
+            eng.release(f"m{rid}")
+        eng.cache.check()
+    assert (True, True) in kinds, "the schedule must put single tokens beside portions"
+    assert eng.free_pages() == [pool]
+    for rid in range(len(lengths)):
+        check_logits(torch.cat(got[rid]), plain.logits(prompts[rid]), dtype, f"wide mixed request {rid}")

@@ -205,3 +205,91 @@ def test_whole_model_is_causal_and_one_expert_head_cases(plain_models):
     b = m.logits(toks[:12] + [200] * 8)
     torch.testing.assert_close(a[:12], b[:12], rtol=1e-5, atol=1e-6)
     assert not torch.allclose(a[12:], b[12:], atol=1e-4)
+
+
+# ---------------------------------------------------------------- the whole model's composition
+# What fixes the arrangement of the parts beside the reference's text
+# (/root/reference/crates/imparo-model/src/lfm2/workflow_cpu.rs:8-15,203-229): each case below
+# fails for one plausible way of putting right parts together wrongly.
+
+def test_only_distances_count_because_the_head_norm_comes_before_the_rotation(plain_models):
+    """Turning every position by the same amount changes no logit: conv blocks
+    know no positions and rotated scores depend on distances only. That holds
+    only if q and k are normed first and rotated after: a per-dimension weight
+    applied after the rotation scales the two halves of a pair differently and
+    the score of a pair of positions then depends on where they are."""
+    for name, vocab in (("A", 256), ("B", 384)):
+        m = plain_models[name]
+        toks = [(7 * i + 3) % vocab for i in range(24)]
+        a, b = m.logits(toks), m.logits(toks, first_position=57)
+        torch.testing.assert_close(a, b, rtol=2e-4, atol=2e-5)
+
+        class RotatesFirst(type(m)):
+            def norm_and_rotate(self, x, weight, rope_positions):
+                return P.rms_norm(P.rope_neox(x, rope_positions, self.theta, self.D), weight, self.eps)
+        wrong = RotatesFirst.__new__(RotatesFirst)
+        wrong.__dict__.update(m.__dict__)
+        wa, wb = wrong.logits(toks), wrong.logits(toks, first_position=57)
+        assert (wa - wb).abs().max() > 50 * (a - b).abs().max()      # the mistake would show
+
+
+def test_blocks_add_to_the_stream_and_the_last_norm_feeds_the_head(plain_models):
+    """With every block's way back into the stream silenced (out_proj and w2
+    zero) the logits are head(rms_norm(embedding, embedding_norm)): the blocks
+    only ever add, nothing scales or norms the stream itself, and the head
+    reads the normed stream (tied: the embedding table; untied: lm_head)."""
+    import copy
+    for name, vocab in (("A", 256), ("B", 384)):
+        m = copy.copy(plain_models[name])
+        m.w = dict(m.w)
+        for k in list(m.w):
+            if k.endswith("out_proj.weight") or k.endswith("out_proj.bias") or k.endswith("feed_forward.w2.weight"):
+                m.w[k] = torch.zeros_like(m.w[k])
+        toks = [(5 * i + 1) % vocab for i in range(9)]
+        e = m.w["model.embed_tokens.weight"][toks]
+        head = m.w["model.embed_tokens.weight"] if name == "A" else m.w["lm_head.weight"]
+        want = torch.nn.functional.rms_norm(e, (e.shape[-1],), m.w["model.embedding_norm.weight"], m.eps) @ head.t()
+        torch.testing.assert_close(m.logits(toks), want, rtol=1e-5, atol=1e-6)
+
+
+def test_mixers_and_feed_forwards_read_the_normed_stream(plain_models):
+    """Pre-norm: a block's mixer and feed-forward see rms_norm(x), so doubling
+    the embedding table (with eps far below the rows' mean square) leaves the
+    delta a part adds as it was: hidden(2 e) - hidden(e) = e. Post-norm, or a
+    part fed the raw stream, would change its delta too. One part at a time,
+    the other silenced, since the second part of a block sees the first's
+    delta beside the stream."""
+    import copy
+    toks = [(11 * i + 2) % 256 for i in range(12)]
+    for layer in (0, 1):                                  # a conv block, an attention block
+        for silenced in ("feed_forward.w2.weight", "out_proj.weight"):
+            m = copy.copy(plain_models["A"])
+            m.w = dict(m.w)
+            m.eps = 1e-12
+            for k in list(m.w):
+                if k.endswith(silenced):
+                    m.w[k] = torch.zeros_like(m.w[k])
+            e = m.w["model.embed_tokens.weight"][toks]
+            h1 = m.hidden(toks, order=[(layer, None)])
+            m.w["model.embed_tokens.weight"] = 2 * m.w["model.embed_tokens.weight"]
+            h2 = m.hidden(toks, order=[(layer, None)])
+            torch.testing.assert_close(h2 - h1, e, rtol=1e-4, atol=1e-6)
+            assert (h1 - e).abs().max() > 1e-4          # and the part did add something, far above the tolerance
+
+
+def test_a_conv_block_is_the_library_conv_between_two_gates(plain_models):
+    """The conv mixer of Tiny B (biases on) from library routines: in_proj as
+    F.linear, the depthwise causal conv with ITS bias as F.conv1d (so the bias
+    lands on the conv's output, before the C gate), out_proj as F.linear."""
+    F = torch.nn.functional
+    m = plain_models["B"]
+    g = torch.Generator().manual_seed(3)
+    h = torch.randn(11, m.E, generator=g)
+    p = "model.layers.0.conv."
+    bcx = F.linear(h, m.w[p + "in_proj.weight"], m.w[p + "in_proj.bias"])
+    B, C, x = bcx.split(m.E, dim=-1)                                   # in that order
+    L = m.w[p + "conv.weight"].shape[-1]
+    conv = F.conv1d(F.pad((B * x).t().unsqueeze(0), (L - 1, 0)), m.w[p + "conv.weight"], m.w[p + "conv.bias"],
+                    groups=m.E)[0].t()
+    want = F.linear(C * conv, m.w[p + "out_proj.weight"], m.w[p + "out_proj.bias"])
+    torch.testing.assert_close(m.mixer_conv(0, h), want, rtol=1e-5, atol=1e-6)
