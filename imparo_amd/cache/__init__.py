@@ -1,2 +1,2 @@
-from .pages import (PagePool, CacheGroup, CacheManager, PagedSpec, FixedSpec, StateSpec,
+from .pages import (PagePool, CacheGroup, CacheManager, PagedSpec, PagedArray, PAGE, kv_spec, FixedSpec, StateSpec,
                     OutOfPages, CacheError)

@@ -20,7 +20,7 @@ _SIGNATURES = {
     "imparo_pool_new": ([I], P), "imparo_pool_delete": ([P], None), "imparo_pool_alloc": ([P], I),
     "imparo_pool_free": ([P, I], I), "imparo_pool_n_free": ([P], I), "imparo_pool_n_pages": ([P], I),
     "imparo_pool_high_water": ([P], I), "imparo_pool_is_free": ([P, I], I), "imparo_pool_scramble": ([P, c_uint64], I),
-    "imparo_cache_new": ([I, P, I, I, I], P), "imparo_cache_delete": ([P], None),
+    "imparo_cache_new": ([I, P, I, P, I], P), "imparo_cache_delete": ([P], None),
     "imparo_cache_group_pool": ([P, I], P), "imparo_cache_slot_pool": ([P], P),
     "imparo_cache_admit": ([P, c_int64], I), "imparo_cache_release": ([P, c_int64], I),
     "imparo_cache_reserve": ([P, c_int64, I], I), "imparo_cache_rollback": ([P, c_int64], I),
@@ -54,6 +54,16 @@ E_LOST_PAGE, E_SHARED_PAGE, E_SLOTS = -9, -10, -11
 E_TWICE, E_EMPTY, E_POSITIONS, E_TOKEN, E_WANT = -12, -13, -14, -15, -16
 
 
+def _built_from(lib: ctypes.CDLL) -> str:
+    try:
+        fn = lib.imparo_host_source_hash
+    except AttributeError:
+        return "none"
+    fn.restype = ctypes.c_char_p
+    fn.argtypes = []
+    return fn().decode("ascii", "replace")
+
+
 def host_library() -> ctypes.CDLL:
     global _lib
     if _lib is not None:
@@ -65,11 +75,14 @@ def host_library() -> ctypes.CDLL:
         if not os.path.isfile(path):
             path = _build.build_host(verbose=True)
         lib = ctypes.CDLL(path)
-        if not all(hasattr(lib, name) for name in _SIGNATURES):
-            # a library from an older build: the host runtime needs no GPU and builds in seconds
+        if _built_from(lib) != _build.host_source_hash():
+            # a library older than its sources: the host runtime needs no GPU and builds in seconds
             import _ctypes
             _ctypes.dlclose(lib._handle)
-            lib = ctypes.CDLL(_build.build_host(verbose=True))
+            path = _build.build_host(verbose=True)
+            lib = ctypes.CDLL(path)
+            if _built_from(lib) != _build.host_source_hash():
+                raise RuntimeError(f"{path} still does not match its sources after a rebuild")
         for name, (argtypes, restype) in _SIGNATURES.items():
             try:
                 fn = getattr(lib, name)

@@ -85,19 +85,63 @@ class PagePool:
             raise CacheError("placement can only be scrambled while every page is free")
 
 
+PAGE = -1     # in a PagedArray's page shape: the dimension that runs over the positions of a page
+
+
+@dataclass(frozen=True)
+class PagedArray:
+    """One tensor of a paged cache site: the shape of one page of it, with
+    PAGE where the page's positions run, and whether it is kept in float32
+    instead of the engine's dtype. The device tensor is [n_pages, *page_shape]."""
+    name: str
+    page_shape: Tuple[int, ...]
+    float32: bool = False
+
+    def shape(self, n_pages: int, page_size: int) -> Tuple[int, ...]:
+        return (n_pages,) + tuple(page_size if d == PAGE else d for d in self.page_shape)
+
+    def elements_per_position(self) -> int:
+        n = 1
+        for d in self.page_shape:
+            n *= 1 if d == PAGE else d
+        return n
+
+
 @dataclass(frozen=True)
 class PagedSpec:
-    """State that grows with the context: keys and values per position.
-    `window` None keeps every position; a number keeps only that many."""
-    kv_heads: int
-    head_dim: int
+    """State that grows with the context, in pages: the arrays a mixer keeps
+    per position (keys and values, a latent, whatever it declares), laid out
+    as the mixer's kernels read them. `window` None keeps every position; a
+    number keeps only that many. Sites with equal specs share a pool and a
+    block table per request."""
+    arrays: Tuple[PagedArray, ...]
     window: Optional[int] = None
+
+    def __post_init__(self):
+        names = [a.name for a in self.arrays]
+        if len(set(names)) != len(names):
+            raise ValueError(f"a paged spec names an array twice: {names}")
+        for a in self.arrays:
+            if list(a.page_shape).count(PAGE) != 1:
+                raise ValueError(f"array {a.name!r}: exactly one dimension of a page's shape runs over its positions")
+
+    def bytes_per_position(self, element_size: int) -> int:
+        return sum(a.elements_per_position() * (4 if a.float32 else element_size) for a in self.arrays)
+
+
+def kv_spec(kv_heads: int, head_dim: int, window: Optional[int] = None, v_transposed: bool = False) -> PagedSpec:
+    """Keys and values of grouped-query attention: K [kv_heads, page, head_dim]
+    and V the same, or transposed inside the page [kv_heads, head_dim, page]."""
+    v_shape = (kv_heads, head_dim, PAGE) if v_transposed else (kv_heads, PAGE, head_dim)
+    return PagedSpec((PagedArray("k", (kv_heads, PAGE, head_dim)), PagedArray("v", v_shape)), window)
 
 
 @dataclass(frozen=True)
 class FixedSpec:
-    """State of a fixed size per request (a conv history, a recurrent matrix)."""
+    """State of a fixed size per request (a conv history, a recurrent matrix),
+    float32; a request that has seen nothing starts from `init` everywhere."""
     shape: Tuple[int, ...]
+    init: float = 0.0
 
 
 StateSpec = Union[PagedSpec, FixedSpec, None]
@@ -184,25 +228,38 @@ class CacheManager:
     `release`, which gives back everything it holds.
     """
 
-    def __init__(self, site_specs: Sequence[StateSpec], page_size: int, n_pages: int, n_slots: int):
+    @staticmethod
+    def groups_of(site_specs: Sequence[StateSpec]) -> List[Tuple[PagedSpec, List[int]]]:
+        """The groups a list of site specs makes: (spec, its sites), in order of first appearance."""
+        out: List[Tuple[PagedSpec, List[int]]] = []
+        for site, spec in enumerate(site_specs):
+            if isinstance(spec, PagedSpec):
+                for known, sites in out:
+                    if known == spec:
+                        sites.append(site)
+                        break
+                else:
+                    out.append((spec, [site]))
+        return out
+
+    def __init__(self, site_specs: Sequence[StateSpec], page_size: int, n_pages: Union[int, Sequence[int]],
+                 n_slots: int):
+        """`n_pages`: the pool size of every group, or one size per group (in the order of `groups_of`)."""
         if page_size <= 0 or page_size & (page_size - 1):
             raise ValueError(f"page size must be a power of two, got {page_size}")
         self._lib = N.host_library()
         self.page_size = page_size
         self.site_specs = list(site_specs)
-        specs: List[PagedSpec] = []
-        self.group_of_site: Dict[int, int] = {}
-        sites_of: List[List[int]] = []
-        for site, spec in enumerate(self.site_specs):
-            if isinstance(spec, PagedSpec):
-                if spec not in specs:
-                    specs.append(spec)
-                    sites_of.append([])
-                g = specs.index(spec)
-                sites_of[g].append(site)
-                self.group_of_site[site] = g
+        grouped = self.groups_of(self.site_specs)
+        specs = [spec for spec, _ in grouped]
+        sites_of = [sites for _, sites in grouped]
+        self.group_of_site: Dict[int, int] = {site: g for g, sites in enumerate(sites_of) for site in sites}
+        sizes = [int(n_pages)] * len(specs) if isinstance(n_pages, int) else [int(n) for n in n_pages]
+        if len(sizes) != len(specs):
+            raise ValueError(f"{len(sizes)} pool sizes were given for {len(specs)} groups")
         windows = (ctypes.c_int32 * max(1, len(specs)))(*[s.window or 0 for s in specs])
-        self._c = self._lib.imparo_cache_new(len(specs), windows, page_size, n_pages, n_slots)
+        pool_sizes = (ctypes.c_int32 * max(1, len(specs)))(*sizes)
+        self._c = self._lib.imparo_cache_new(len(specs), windows, page_size, pool_sizes, n_slots)
         if not self._c:
             raise ValueError("the cache manager refused its sizes")
         self.groups: List[CacheGroup] = []
@@ -384,7 +441,7 @@ class CacheManager:
         self._lib.imparo_cache_end_step(self._c, len(b.requests), b.reqs.ctypes.data, b.n_tok.ctypes.data)
 
     # ------------------------------------------------------------ a step's index arrays
-    LAYOUT = ("T", "R", "W", "G", "P", "n_single", "n_multi", "n_prefill_tiles", "max_seg_len", "max_context", "total")
+    LAYOUT = ("T", "R", "W", "G", "P", "n_single", "n_multi", "max_seg_len", "max_context", "total")
 
     def pack(self, requests: Sequence[Hashable], token_lists: Sequence[Sequence[int]],
              want_lists: Sequence[Sequence[int]], table_width: int = 0) -> Tuple[np.ndarray, Dict[str, int]]:

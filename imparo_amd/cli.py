@@ -35,6 +35,17 @@ def _top10(row) -> str:
     return " ".join(f"{int(i)}:{float(v):.4f}" for v, i in zip(vals, idx))
 
 
+def _pool_sizing(a, default_tokens: int) -> dict:
+    """How the cache pools are sized: --num-pages, --kv-gb, or enough for the run."""
+    if a.num_pages is not None and a.kv_gb is not None:
+        raise SystemExit("give one of --num-pages and --kv-gb")
+    if a.num_pages is not None:
+        return dict(num_pages=a.num_pages)
+    if a.kv_gb is not None:
+        return dict(kv_budget_bytes=int(a.kv_gb * (1 << 30)))
+    return dict(max_tokens=default_tokens)
+
+
 def cmd_forward(a) -> int:
     import torch
     from .engine import Engine, StepEntry
@@ -42,8 +53,9 @@ def cmd_forward(a) -> int:
     tokens = [int(t) for t in a.tokens]
     cap = a.ctx or (len(tokens) + a.decode + 64)
     n_conv = max(1, a.cobatch)
-    eng = Engine(a.model, dtype=a.dtype, max_tokens=(cap // a.page_size + 2) * a.page_size * n_conv,
-                 page_size=a.page_size, max_requests=max(2, n_conv))
+    sizing = _pool_sizing(a, (cap // a.page_size + 2) * a.page_size * n_conv)
+    eng = Engine(a.model, dtype=a.dtype, page_size=a.page_size, max_requests=max(2, n_conv),
+                 max_step_tokens=max(len(tokens) * n_conv, 1), **sizing)
 
     def argmax(row) -> int:
         out = torch.empty(1, dtype=torch.int32, device=row.device)
@@ -113,8 +125,8 @@ def cmd_forward(a) -> int:
                 if trail != base[1]:
                     status = 1
     if a.scramble_kv:
-        eng2 = Engine(a.model, dtype=a.dtype, max_tokens=(cap // a.page_size + 2) * a.page_size,
-                      page_size=a.page_size, max_requests=2)
+        eng2 = Engine(a.model, dtype=a.dtype, page_size=a.page_size, max_requests=2,
+                      max_step_tokens=max(len(tokens), 1), **_pool_sizing(a, (cap // a.page_size + 2) * a.page_size))
         eng2.cache.scramble(seed=1)
         row = eng2.step([StepEntry("s", tokens, [len(tokens) - 1])])[0]
         delta = float((row - base[0]).abs().max())
@@ -129,7 +141,8 @@ def cmd_generate(a) -> int:
     t0 = time.time()
     out = generate(a.model, prompts, max_tokens=a.max_tokens, temperature=a.temperature, seed=a.seed,
                    dtype=a.dtype, ctx=a.ctx, parallel=a.parallel, max_batch_tokens=a.max_batch_tokens,
-                   page_size=a.page_size)
+                   page_size=a.page_size, num_pages=a.num_pages,
+                   kv_budget_bytes=None if a.kv_gb is None else int(a.kv_gb * (1 << 30)))
     dt = time.time() - t0
     for i, ids in enumerate(out):
         print(json.dumps({"index": i, "output_ids": ids}))
@@ -157,6 +170,9 @@ def main(argv=None) -> int:
         p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
         p.add_argument("-c", "--ctx", type=int, default=None, help="most tokens one request may hold")
         p.add_argument("--page-size", type=int, default=64)
+        p.add_argument("--num-pages", type=int, default=None,
+                       help="pages in every cache pool (a small number makes requests wait or be recomputed)")
+        p.add_argument("--kv-gb", type=float, default=None, help="memory for the paged caches, in GiB")
 
     f = sub.add_parser("forward", help="run explicit token ids and print top logits")
     common(f)

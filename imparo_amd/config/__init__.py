@@ -1,5 +1,5 @@
 from .errors import ConfigError, UnknownArchitecture, MissingKey, BadValue, Inconsistent
-from .plan import PartSpec, LayerPlan, LayerCall, ModelPlan
+from .plan import PartSpec, LayerPlan, LayerCall, ModelPlan, pre_norm_layer
 from .registry import (register_architecture, known_architectures, architecture_of,
                        read_config_json, plan_from_config)
 from . import lfm2 as _lfm2

@@ -14,7 +14,7 @@ from dataclasses import dataclass, field, asdict
 from typing import Any, Dict, List, Optional
 
 from .errors import MissingKey, BadValue, Inconsistent
-from .plan import PartSpec, LayerPlan, LayerCall, ModelPlan
+from .plan import PartSpec, LayerPlan, LayerCall, ModelPlan, pre_norm_layer
 
 ARCHITECTURE = "Lfm2ForCausalLM"
 LAYER_KINDS = ("conv", "full_attention", "sliding_attention")
@@ -317,7 +317,7 @@ def build_plan(cfg: Lfm2Config) -> ModelPlan:
                 position=PartSpec("rope_neox", "", dict(base=cfg.rope_theta, rotary_dim=D)),
                 names=dict(q="q_proj", k="k_proj", v="v_proj", o="out_proj",
                            q_norm="q_layernorm", k_norm="k_layernorm")))
-        layers.append(LayerPlan(
+        layers.append(pre_norm_layer(
             mixer=mixer,
             ffn=PartSpec("swiglu", f"{base}.feed_forward", dict(
                 width=E, hidden=cfg.ff_dim, names=dict(gate="w1", up="w3", down="w2"))),

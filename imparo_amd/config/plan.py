@@ -12,7 +12,7 @@ KvSource records (/root/reference/crates/imparo-model/src/lib.rs:90-141,
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional
+from typing import Any, Dict, List, Optional, Tuple
 
 
 @dataclass(frozen=True)
@@ -32,12 +32,34 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerPlan:
-    """A block: two norms, a mixer and a feed-forward, in a named arrangement."""
-    mixer: PartSpec
-    ffn: PartSpec
-    mixer_norm: PartSpec
-    ffn_norm: PartSpec
+    """A block: named parts, each with its role (the registry it is looked up
+    in) and its spec, and the arrangement, a registered block kind that knows
+    what to do with parts of these names. The builder and the loader walk
+    `parts` and never ask which names they are."""
+    parts: Dict[str, Tuple[str, PartSpec]]       # name -> (role, spec), in the order the block runs them
     arrangement: str = "pre_norm"
+
+    def spec(self, name: str) -> PartSpec:
+        return self.parts[name][1]
+
+    def with_part(self, name: str, spec: PartSpec, role: Optional[str] = None) -> "LayerPlan":
+        """This layer with the part `name` replaced (same role unless given) or, for a new name, added."""
+        if role is None:
+            role = self.parts[name][0]
+        return LayerPlan(dict(self.parts, **{name: (role, spec)}), self.arrangement)
+
+    def __getattr__(self, name: str) -> PartSpec:
+        # layer.mixer, layer.ffn_norm, ...: whatever the arrangement names its parts
+        parts = object.__getattribute__(self, "parts")
+        if name in parts:
+            return parts[name][1]
+        raise AttributeError(name)
+
+
+def pre_norm_layer(mixer: PartSpec, ffn: PartSpec, mixer_norm: PartSpec, ffn_norm: PartSpec) -> LayerPlan:
+    """The parts of a pre-norm block, under the names that arrangement reads."""
+    return LayerPlan(dict(mixer_norm=("norm", mixer_norm), mixer=("mixer", mixer),
+                          ffn_norm=("norm", ffn_norm), ffn=("feed_forward", ffn)), "pre_norm")
 
 
 @dataclass(frozen=True)

@@ -11,6 +11,9 @@ extern "C" {
 
 typedef void* imparo_stream;
 
+// The hash of the sources this library was built from, as the build computed it.
+const char* imparo_hip_source_hash();
+
 // x[t, :] = table[ids[t], :] as float32.
 int imparo_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* x,
                         int n_tokens, int width, int vocab, imparo_stream stream);
@@ -29,13 +32,6 @@ int imparo_rms_norm(float* x, const float* delta, int n_delta, int n_x_rows, con
                     void* out, int out_dtype, int n_rows, int width, float eps, int write_back,
                     imparo_stream stream);
 
-// out[t, j] = silu(gu[t, j]) * gu[t, hidden + j]; gu is [n, 2*hidden].
-int imparo_silu_mul(const void* gu, int in_dtype, void* out, int out_dtype, int n_tokens, int hidden,
-                    imparo_stream stream);
-
-// y = x (+ bias): adds a float32 bias [n] to every row of a float32 [m, n] in place.
-int imparo_add_bias(float* y, const float* bias, int m, int n, imparo_stream stream);
-
 // Y[m, n] = X[m, k] . W[n, k]^T (+ bias[n], float32, may be null), float32
 // accumulate. X and W share `dtype`. epilogue 0: Y is [m, n]. epilogue 1
 // (SwiGLU): W's rows alternate gate, up; Y is [m, n/2] with
@@ -46,16 +42,22 @@ int imparo_add_bias(float* y, const float* bias, int m, int n, imparo_stream str
 int imparo_gemm(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
                 int m, int n, int k, int epilogue, int slices, imparo_stream stream);
 int imparo_gemm_slices(int m, int n, int k, int dtype);
+// imparo_gemm with the kernel named by the caller instead of chosen by the library: for tests and
+// measurements, so that every kernel can be met at any shape (the numbers are listed in gemm.hip).
+// Nothing in the library keeps the choice: it is this call's argument.
+int imparo_gemm_variant(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
+                        int m, int n, int k, int epilogue, int slices, int variant, imparo_stream stream);
 
 // Per (token, head): RMS norm over the head (weight null: none), NeoX rotation
-// with angles pos * inv_freq[i] over the first 2*n_freq dims (n_freq 0: none).
+// with angles pos * inv_freq[i] over the first 2*n_freq dims (n_freq 0: none): pair i is dims
+// (i, i + n_freq), or with `interleaved` dims (2i, 2i + 1).
 // qkv is float32 [n_tokens, (heads + 2*kv_heads) * head_dim]; q goes to q_out
 // [n_tokens, heads, head_dim], k and v into the paged cache at each token's
 // position: page = table[row_of_token[t] * table_stride + pos / page_size].
 // Cache layout [n_pages, kv_heads, page_size, head_dim]; with v_transposed the V
 // cache is [n_pages, kv_heads, head_dim, page_size]. write_kv 0 skips the cache.
 int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight, const float* k_weight, float eps,
-                              const float* inv_freq, int n_freq,
+                              const float* inv_freq, int n_freq, int interleaved,
                               const int32_t* positions, const int32_t* row_of_token,
                               const int32_t* block_table, int table_stride, int page_size,
                               void* q_out, void* k_cache, void* v_cache, int dtype, int write_kv,
@@ -76,6 +78,8 @@ int imparo_attention(const void* q, const void* k_cache, const void* v_cache, vo
 // range is split in pieces of 256 keys whose partial results go through
 // part_o [n_rows, heads, n_splits, head_dim] and part_ml [n_rows, heads,
 // n_splits, 2]; n_splits >= ceil(longest context / 256).
+int imparo_attention_decode_split(void);      // keys per split
+int imparo_attention_prefill_tile(void);      // queries per tile that n_tiles counts
 int imparo_attention_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
                             float* part_o, float* part_ml, const int32_t* rows, int n_rows,
                             const int32_t* seg_start, const int32_t* positions,
@@ -154,6 +158,12 @@ int imparo_sample_rows(const float* logits, const float* temperature, const floa
 
 // Fills n float32 values (or n int32 values of the same bits) without a memset node.
 int imparo_fill_f32(float* p, float value, int64_t n, imparo_stream stream);
+
+// The fixed-size state of one slot, every site in one launch: for site i, per_slot[i] float32
+// values at base[i] (a device address) + slot * per_slot[i] are set to value[i]. base, per_slot
+// and value are device arrays of n_sites entries that the caller built from tensors it owns.
+int imparo_fill_sites(const uint64_t* base, const int64_t* per_slot, const float* value, int n_sites, int slot,
+                      imparo_stream stream);
 
 #ifdef __cplusplus
 }

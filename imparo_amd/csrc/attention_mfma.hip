@@ -967,6 +967,12 @@ static int check_common(const void* q, const void* k_cache, const void* v_cache,
         default: return IMPARO_BAD_ARGUMENT;                                                                         \
     }
 
+// The two numbers of these kernels' geometry that a caller sizes things by: a decode row's keys are
+// split in runs of this many (the partial results' buffers hold one entry per run), and prompt
+// portions are counted in tiles of this many queries (n_tiles of imparo_attention_prefill).
+extern "C" int imparo_attention_decode_split() { return DEC_SPLIT; }
+extern "C" int imparo_attention_prefill_tile() { return 64; }
+
 static int attention_decode_launch(const void* q, const void* k_cache, const void* v_cache, void* out,
                                    float* part_o, float* part_ml, const int32_t* rows, int n_rows,
                                    const int32_t* seg_start, const int32_t* positions,

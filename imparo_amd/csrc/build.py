@@ -27,6 +27,27 @@ def sources() -> List[str]:
     return sorted(f for f in os.listdir(HERE) if f.endswith(".hip"))
 
 
+def _hash_of(paths: List[str]) -> str:
+    h = hashlib.sha256()
+    for path in sorted(paths):
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def source_hash() -> str:
+    """A hash of everything the kernel library is compiled from. The library
+    carries the hash of the sources it was built from (imparo_hip_source_hash),
+    so that a library older than its sources is noticed when it is loaded."""
+    return _hash_of([os.path.join(HERE, f) for f in os.listdir(HERE) if f.endswith((".hip", ".h"))])
+
+
+def host_source_hash() -> str:
+    src_dir = os.path.join(HERE, "host")
+    return _hash_of([os.path.join(src_dir, f) for f in os.listdir(src_dir) if f.endswith((".cpp", ".h"))])
+
+
 def _hipcc() -> str:
     for cand in (shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
         if cand and os.path.isfile(cand):
@@ -79,7 +100,8 @@ def build_host(verbose: bool = True) -> str:
     srcs = sorted(os.path.join(src_dir, f) for f in os.listdir(src_dir) if f.endswith(".cpp"))
     lib = os.path.join(out_dir, HOST_LIB_NAME)
     tmp = lib + f".tmp{os.getpid()}"
-    proc = subprocess.run([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-I", src_dir] + srcs + ["-o", tmp],
+    stamp = f'-DIMPARO_SOURCE_HASH="{host_source_hash()}"'
+    proc = subprocess.run([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", stamp, "-I", src_dir] + srcs + ["-o", tmp],
                           stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"building {HOST_LIB_NAME} failed:\n{proc.stderr}")
@@ -103,9 +125,11 @@ def build(verbose: bool = True) -> str:
     if verbose:
         _say(f"compiling {len(srcs)} sources for {ARCH} into {out_dir}")
 
+    stamp = f'-DIMPARO_SOURCE_HASH="{source_hash()}"'
+
     def compile_one(src: str) -> str:
         obj = os.path.join(obj_dir, src[:-4] + ".o")
-        cmd = [hipcc] + FLAGS + ["-c", os.path.join(HERE, src), "-o", obj]
+        cmd = [hipcc] + FLAGS + [stamp, "-c", os.path.join(HERE, src), "-o", obj]
         proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
         if proc.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{proc.stderr}")

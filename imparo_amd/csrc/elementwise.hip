@@ -186,51 +186,7 @@ extern "C" int imparo_rms_norm(float* x, const float* delta, int n_delta, int n_
     return launch_status();
 }
 
-// ---------------------------------------------------------------- SiLU gate
-template <typename TIn, typename TOut>
-__global__ void k_silu_mul(const TIn* __restrict__ gu, TOut* __restrict__ out, int64_t total, int hidden) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= total) return;
-    const int64_t t = i / hidden;
-    const int j = (int)(i - t * hidden);
-    const float g = load_f32<TIn>(gu, (size_t)t * 2 * hidden + j);
-    const float u = load_f32<TIn>(gu, (size_t)t * 2 * hidden + hidden + j);
-    store_f32<TOut>(out, (size_t)i, g / (1.0f + expf(-g)) * u);
-}
-
-extern "C" int imparo_silu_mul(const void* gu, int in_dtype, void* out, int out_dtype, int n_tokens, int hidden,
-                               imparo_stream stream) {
-    if (!gu || !out || n_tokens < 0 || hidden <= 0) return IMPARO_BAD_ARGUMENT;
-    if (n_tokens == 0) return IMPARO_OK;
-    hipStream_t s = (hipStream_t)stream;
-    const int64_t total = (int64_t)n_tokens * hidden;
-    const int threads = 256;
-    const unsigned blocks = (unsigned)((total + threads - 1) / threads);
-    if (in_dtype == IMPARO_F32 && out_dtype == IMPARO_F32)
-        k_silu_mul<float, float><<<blocks, threads, 0, s>>>((const float*)gu, (float*)out, total, hidden);
-    else if (in_dtype == IMPARO_F32 && out_dtype == IMPARO_BF16)
-        k_silu_mul<float, bf16_t><<<blocks, threads, 0, s>>>((const float*)gu, (bf16_t*)out, total, hidden);
-    else if (in_dtype == IMPARO_BF16 && out_dtype == IMPARO_BF16)
-        k_silu_mul<bf16_t, bf16_t><<<blocks, threads, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, total, hidden);
-    else
-        return IMPARO_BAD_ARGUMENT;
-    return launch_status();
-}
-
-// ---------------------------------------------------------------- bias, fill
-__global__ void k_add_bias(float* __restrict__ y, const float* __restrict__ bias, int64_t total, int n) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < total) y[i] += bias[i % n];
-}
-
-extern "C" int imparo_add_bias(float* y, const float* bias, int m, int n, imparo_stream stream) {
-    if (!y || !bias || m < 0 || n <= 0) return IMPARO_BAD_ARGUMENT;
-    if (m == 0) return IMPARO_OK;
-    const int64_t total = (int64_t)m * n;
-    k_add_bias<<<(unsigned)((total + 255) / 256), 256, 0, (hipStream_t)stream>>>(y, bias, total, n);
-    return launch_status();
-}
-
+// ---------------------------------------------------------------- fill
 __global__ void k_fill_f32(float* __restrict__ p, float value, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = value;
@@ -240,6 +196,27 @@ extern "C" int imparo_fill_f32(float* p, float value, int64_t n, imparo_stream s
     if (!p || n < 0) return IMPARO_BAD_ARGUMENT;
     if (n == 0) return IMPARO_OK;
     k_fill_f32<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(p, value, n);
+    return launch_status();
+}
+
+// Every fixed-state site's row of one slot in one launch: site i's row is per_slot[i] floats at
+// base[i] + slot * per_slot[i] and is filled with value[i]. grid (sites, blocks along the row).
+__global__ void k_fill_sites(const uint64_t* __restrict__ base, const int64_t* __restrict__ per_slot,
+                             const float* __restrict__ value, int slot) {
+    const int site = blockIdx.x;
+    const int64_t n = per_slot[site];
+    float* p = reinterpret_cast<float*>(base[site]) + (int64_t)slot * n;
+    const float v = value[site];
+    for (int64_t i = (int64_t)blockIdx.y * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.y * blockDim.x)
+        p[i] = v;
+}
+
+extern "C" int imparo_fill_sites(const uint64_t* base, const int64_t* per_slot, const float* value, int n_sites,
+                                 int slot, imparo_stream stream) {
+    if (n_sites < 0 || slot < 0 || (n_sites > 0 && (!base || !per_slot || !value))) return IMPARO_BAD_ARGUMENT;
+    if (n_sites == 0) return IMPARO_OK;
+    if (n_sites > 65535) return IMPARO_BAD_ARGUMENT;
+    k_fill_sites<<<dim3((unsigned)n_sites, 16), 256, 0, (hipStream_t)stream>>>(base, per_slot, value, slot);
     return launch_status();
 }
 

@@ -1165,12 +1165,8 @@ static int whole_slices(int slices, int k, int step) {
 // with few rows gives too few blocks to keep the memory system busy otherwise (one CU draws
 // about 50 GB/s at best, so it takes all of them): the measured optimum, with cold weights,
 // is about 256 blocks, with at least 512 of K per slice and at most 8 slices.
-static int g_force_few_row_kernel = 0;
-static int g_force_slices = 0;      // set by imparo_gemm_force_kernel, for measurements
-
 extern "C" int imparo_gemm_slices(int m, int n, int k, int dtype) {
     if (dtype != IMPARO_BF16) return 1;
-    if (g_force_slices) return g_force_slices;
     if (m > 64) {
         const DmaPlan plan = dma_plan(m, n, k, 0);
         if (plan.tn) return plan.slices;
@@ -1417,23 +1413,18 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
 }
 
 
-// For measurements and tests only: 0 lets the library choose the kernel, 1 forces the K-split
-// kernel, 2, 4 or 8 the shared-activation kernel with that many waves, 256 the 256x256 tile with
-// register staging, 258 / 263 / 262 the tile with loads straight into LDS at 256 rows by 256 / 192 /
-// 128, 358 / 352 the same at 128 rows by 256 / 128; plus 1000 times a number of K slices that
-// imparo_gemm then accepts whatever the shape.
-extern "C" void imparo_gemm_force_kernel(int which) {
-    g_force_slices = which / 1000;
-    g_force_few_row_kernel = which % 1000;
-}
-
-extern "C" int imparo_gemm(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
-                           int m, int n, int k, int epilogue, int slices, imparo_stream stream) {
+// `variant` 0 lets the library choose the kernel. The others are for measurements and tests only, so
+// that each kernel can be met at any shape: 1 the K-split kernel, 2, 4 or 8 the shared-activation
+// kernel with that many waves, 256 the 256x256 tile with register staging, 258 / 263 / 262 the tile
+// with loads straight into LDS at 256 rows by 256 / 192 / 128, 358 / 352 the same at 128 rows by
+// 256 / 128; with a variant, any number of K slices is taken.
+static int gemm_variant(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
+                        int m, int n, int k, int epilogue, int slices, int variant, imparo_stream stream) {
     if (!x || !w || !y || m < 0 || n <= 0 || k <= 0) return IMPARO_BAD_ARGUMENT;
     if (slices < 1) return IMPARO_BAD_ARGUMENT;
     // slices: only what imparo_gemm_slices allows, float32 out, no epilogue that is not linear
     const int slices_ok = imparo_gemm_slices(m, n, k, dtype);
-    if (slices > 1 && (slices != slices_ok || out_dtype != IMPARO_F32 || epilogue != EPI_NONE))
+    if (slices > 1 && ((slices != slices_ok && variant == 0) || out_dtype != IMPARO_F32 || epilogue != EPI_NONE))
         return IMPARO_BAD_ARGUMENT;
     if (epilogue != EPI_NONE && epilogue != EPI_SWIGLU) return IMPARO_BAD_ARGUMENT;
     if (epilogue == EPI_SWIGLU && (n % 2 != 0)) return IMPARO_BAD_ARGUMENT;
@@ -1465,9 +1456,19 @@ extern "C" int imparo_gemm(const void* x, const void* w, const float* bias, void
     if (k % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return IMPARO_BAD_ARGUMENT;
     if (out_dtype == IMPARO_F32)
         return launch_bf16<float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)y, m, n, k, epilogue,
-                                  g_force_few_row_kernel, slices, s);
+                                  variant, slices, s);
     if (out_dtype == IMPARO_BF16)
         return launch_bf16<bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)y, m, n, k, epilogue,
-                                   g_force_few_row_kernel, slices, s);
+                                   variant, slices, s);
     return IMPARO_BAD_ARGUMENT;
+}
+
+extern "C" int imparo_gemm(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
+                           int m, int n, int k, int epilogue, int slices, imparo_stream stream) {
+    return gemm_variant(x, w, bias, y, dtype, out_dtype, m, n, k, epilogue, slices, 0, stream);
+}
+
+extern "C" int imparo_gemm_variant(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
+                                   int m, int n, int k, int epilogue, int slices, int variant, imparo_stream stream) {
+    return gemm_variant(x, w, bias, y, dtype, out_dtype, m, n, k, epilogue, slices, variant, stream);
 }

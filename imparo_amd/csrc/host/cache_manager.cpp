@@ -78,10 +78,11 @@ struct ImparoCache {
     ImparoPool slots;
     std::unordered_map<int64_t, Request> live;
 
-    ImparoCache(int n_groups, const int32_t* w, int ps, int n_pages, int n_slots) : page_size(ps), slots(n_slots) {
+    ImparoCache(int n_groups, const int32_t* w, int ps, const int32_t* n_pages, int n_slots)
+        : page_size(ps), slots(n_slots) {
         for (int g = 0; g < n_groups; ++g) {
             windows.push_back(w ? w[g] : 0);
-            pools.emplace_back(n_pages);
+            pools.emplace_back(n_pages[g]);          // every group has a pool of its own size
         }
     }
     int first_needed_page(int g, int next_position) const {
@@ -97,7 +98,14 @@ struct ImparoCache {
     }
 };
 
+#ifndef IMPARO_SOURCE_HASH
+#define IMPARO_SOURCE_HASH "unknown"
+#endif
+
 extern "C" {
+
+// the hash of the sources this library was built from (given by the build)
+const char* imparo_host_source_hash() { return IMPARO_SOURCE_HASH; }
 
 ImparoPool* imparo_pool_new(int n_pages) { return n_pages < 0 ? nullptr : new ImparoPool(n_pages); }
 void imparo_pool_delete(ImparoPool* p) { delete p; }
@@ -111,8 +119,12 @@ int imparo_pool_is_free(const ImparoPool* p, int page) {
 }
 int imparo_pool_scramble(ImparoPool* p, uint64_t seed) { return p->scramble(seed); }
 
-ImparoCache* imparo_cache_new(int n_groups, const int32_t* windows, int page_size, int n_pages, int n_slots) {
-    if (n_groups < 0 || page_size <= 0 || (page_size & (page_size - 1)) || n_pages < 0 || n_slots < 0) return nullptr;
+ImparoCache* imparo_cache_new(int n_groups, const int32_t* windows, int page_size, const int32_t* n_pages,
+                              int n_slots) {
+    if (n_groups < 0 || page_size <= 0 || (page_size & (page_size - 1)) || n_slots < 0) return nullptr;
+    if (n_groups > 0 && !n_pages) return nullptr;
+    for (int g = 0; g < n_groups; ++g)
+        if (n_pages[g] < 0) return nullptr;
     return new ImparoCache(n_groups, windows, page_size, n_pages, n_slots);
 }
 void imparo_cache_delete(ImparoCache* c) { delete c; }
@@ -359,7 +371,7 @@ int64_t imparo_cache_pack(const ImparoCache* c, int n_rows, const int64_t* reqs,
                           int32_t* out, int64_t capacity, int32_t* layout) {
     const int R = n_rows, G = (int)c->pools.size();
     int64_t T = 0, W = 0;
-    int P = std::max(1, table_width), max_seg = 0, max_ctx = 0, n_single = 0, tiles = 0;
+    int P = std::max(1, table_width), max_seg = 0, max_ctx = 0, n_single = 0;
     std::vector<const Request*> rows((size_t)R);
     for (int r = 0; r < R; ++r) {
         auto it = c->live.find(reqs[r]);
@@ -369,7 +381,7 @@ int64_t imparo_cache_pack(const ImparoCache* c, int n_rows, const int64_t* reqs,
         W += n_want[r];
         max_seg = std::max(max_seg, n_tokens[r]);
         max_ctx = std::max(max_ctx, it->second.length + n_tokens[r]);
-        if (n_tokens[r] == 1) ++n_single; else tiles += (n_tokens[r] + 63) / 64;
+        if (n_tokens[r] == 1) ++n_single;
         if (table_width <= 0)
             for (int g = 0; g < G; ++g) P = std::max(P, (int)it->second.tables[(size_t)g].size());
     }
@@ -416,7 +428,7 @@ int64_t imparo_cache_pack(const ImparoCache* c, int n_rows, const int64_t* reqs,
             std::fill(dst + tab.size(), dst + P, -1);
         }
     if (layout) {
-        const int32_t v[11] = {(int32_t)T, R, (int32_t)W, G, P, n_single, R - n_single, tiles, max_seg, max_ctx,
+        const int32_t v[10] = {(int32_t)T, R, (int32_t)W, G, P, n_single, R - n_single, max_seg, max_ctx,
                                (int32_t)total};
         std::memcpy(layout, v, sizeof(v));
     }

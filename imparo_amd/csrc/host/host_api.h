@@ -41,8 +41,13 @@ int imparo_pool_high_water(const ImparoPool* p);
 int imparo_pool_is_free(const ImparoPool* p, int page);
 int imparo_pool_scramble(ImparoPool* p, uint64_t seed);   // only while every page is free
 
-// ---- the cache manager: n_groups paged groups (window 0 = keep every position), n_slots state slots
-ImparoCache* imparo_cache_new(int n_groups, const int32_t* windows, int page_size, int n_pages, int n_slots);
+// the hash of the sources this library was built from, as the build computed it
+const char* imparo_host_source_hash();
+
+// ---- the cache manager: n_groups paged groups (window 0 = keep every position), each with a pool
+// of n_pages[g] pages, and n_slots state slots
+ImparoCache* imparo_cache_new(int n_groups, const int32_t* windows, int page_size, const int32_t* n_pages,
+                              int n_slots);
 void imparo_cache_delete(ImparoCache* c);
 ImparoPool* imparo_cache_group_pool(ImparoCache* c, int group);
 ImparoPool* imparo_cache_slot_pool(ImparoCache* c);
@@ -84,7 +89,7 @@ int imparo_cache_end_step(ImparoCache* c, int n_rows, const int64_t* reqs, const
 // Layout (int32): tokens[T] | positions[T] | row_of_token[T] | seg_start[R] | seg_len[R] | slot[R] |
 // row lists[R] (rows with one token first, then the others) | want[W] | tables[G][R][P].
 // P = table_width, or the widest table of the batch if table_width is 0. `layout` receives
-// {T, R, W, G, P, n_single, n_multi, n_prefill_tiles, max_seg_len, max_context, total}.
+// {T, R, W, G, P, n_single, n_multi, max_seg_len, max_context, total}.
 // Returns the number of int32 written, or a negative code; lengths are those before the step.
 int64_t imparo_cache_pack(const ImparoCache* c, int n_rows, const int64_t* reqs, const int32_t* n_tokens,
                           const int32_t* tokens, const int32_t* n_want, const int32_t* want, int table_width,

@@ -16,11 +16,13 @@ __device__ __forceinline__ void rotation_of(int pos, float inv_freq, float& sn, 
 __device__ __forceinline__ float head_norm_scale(float sum_squares, int head_dim, float eps) {
     return 1.0f / sqrtf(sum_squares / (float)head_dim + eps);
 }
-// lane-owned pair (i, i + n_freq) of a row staged in LDS: reads both, then writes both
-__device__ __forceinline__ void rotate_pair(float* row, int i, int n_freq, float sn, float cs) {
-    const float x0 = row[i], x1 = row[i + n_freq];
-    row[i] = fmaf(x0, cs, -(x1 * sn));
-    row[i + n_freq] = fmaf(x0, sn, x1 * cs);
+// lane-owned pair i of a row staged in LDS: elements (i, i + n_freq), or with `interleaved`
+// (2i, 2i + 1); reads both, then writes both
+__device__ __forceinline__ void rotate_pair(float* row, int i, int n_freq, int interleaved, float sn, float cs) {
+    const int a = interleaved ? 2 * i : i, b = interleaved ? 2 * i + 1 : i + n_freq;
+    const float x0 = row[a], x1 = row[b];
+    row[a] = fmaf(x0, cs, -(x1 * sn));
+    row[b] = fmaf(x0, sn, x1 * cs);
 }
 
 // One wave per (token, unit), unit in [0, heads + 2*kv_heads): q heads, then k
@@ -30,7 +32,7 @@ __device__ __forceinline__ void rotate_pair(float* row, int i, int n_freq, float
 template <typename T>
 __global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float* __restrict__ q_weight,
                                      const float* __restrict__ k_weight, float eps,
-                                     const float* __restrict__ inv_freq, int n_freq,
+                                     const float* __restrict__ inv_freq, int n_freq, int interleaved,
                                      const int32_t* __restrict__ positions, const int32_t* __restrict__ row_of_token,
                                      const int32_t* __restrict__ block_table, int table_stride, int page_size,
                                      T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
@@ -88,7 +90,7 @@ __global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float*
                 if (i < n_freq) {
                     float sn, cs;
                     rotation_of(pos, freq[j], sn, cs);
-                    rotate_pair(row, i, n_freq, sn, cs);
+                    rotate_pair(row, i, n_freq, interleaved, sn, cs);
                 }
             }
         }
@@ -127,7 +129,7 @@ __global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float*
 template <typename T, int NPL, int UB>
 __global__ __launch_bounds__(ROPE_WAVES * WAVE) void k_qk_norm_rope_store_token(
     const float* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
-    const float* __restrict__ inv_freq, int n_freq, const int32_t* __restrict__ positions,
+    const float* __restrict__ inv_freq, int n_freq, int interleaved, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ row_of_token, const int32_t* __restrict__ block_table, int table_stride,
     int page_size, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int write_kv,
     int n_tokens, int heads, int kv_heads, int head_dim, int n_pages, int v_transposed) {
@@ -184,7 +186,7 @@ __global__ __launch_bounds__(ROPE_WAVES * WAVE) void k_qk_norm_rope_store_token(
 #pragma unroll
                 for (int j = 0; j < NPL; ++j) {
                     const int i = lane + j * WAVE;
-                    if (i < n_freq) rotate_pair(row, i, n_freq, sn_tab[i], cs_tab[i]);
+                    if (i < n_freq) rotate_pair(row, i, n_freq, interleaved, sn_tab[i], cs_tab[i]);
                 }
             } else {
 #pragma unroll
@@ -215,13 +217,13 @@ __global__ __launch_bounds__(ROPE_WAVES * WAVE) void k_qk_norm_rope_store_token(
 
 template <typename T>
 static void launch_rope_token(const float* qkv, const float* q_weight, const float* k_weight, float eps,
-                              const float* inv_freq, int n_freq, const int32_t* positions,
+                              const float* inv_freq, int n_freq, int interleaved, const int32_t* positions,
                               const int32_t* row_of_token, const int32_t* block_table, int table_stride,
                               int page_size, T* q_out, T* k_cache, T* v_cache, int write_kv, int n_tokens, int heads,
                               int kv_heads, int head_dim, int n_pages, int v_transposed, hipStream_t s) {
 #define ROPE_TOKEN(NPL, UB)                                                                                          \
     k_qk_norm_rope_store_token<T, NPL, UB><<<n_tokens, ROPE_WAVES * WAVE, 0, s>>>(                                   \
-        qkv, q_weight, k_weight, eps, inv_freq, n_freq, positions, row_of_token, block_table, table_stride,         \
+        qkv, q_weight, k_weight, eps, inv_freq, n_freq, interleaved, positions, row_of_token, block_table, table_stride,         \
         page_size, q_out, k_cache, v_cache, write_kv, n_tokens, heads, kv_heads, head_dim, n_pages, v_transposed)
     if (head_dim <= 64)
         ROPE_TOKEN(1, 4);
@@ -242,7 +244,7 @@ static void launch_rope_token(const float* qkv, const float* q_weight, const flo
 #endif
 
 extern "C" int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight, const float* k_weight, float eps,
-                                         const float* inv_freq, int n_freq,
+                                         const float* inv_freq, int n_freq, int interleaved,
                                          const int32_t* positions, const int32_t* row_of_token,
                                          const int32_t* block_table, int table_stride, int page_size,
                                          void* q_out, void* k_cache, void* v_cache, int dtype, int write_kv,
@@ -261,12 +263,12 @@ extern "C" int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight
     hipStream_t s = (hipStream_t)stream;
     if (n_tokens >= ROPE_TOKEN_KERNEL_FROM && (dtype == IMPARO_F32 || dtype == IMPARO_BF16)) {
         if (dtype == IMPARO_F32)
-            launch_rope_token<float>(qkv, q_weight, k_weight, eps, inv_freq, n_freq, positions, row_of_token,
+            launch_rope_token<float>(qkv, q_weight, k_weight, eps, inv_freq, n_freq, interleaved, positions, row_of_token,
                                      block_table, table_stride, page_size, (float*)q_out, (float*)k_cache,
                                      (float*)v_cache, write_kv, n_tokens, heads, kv_heads, head_dim, n_pages,
                                      v_transposed, s);
         else
-            launch_rope_token<bf16_t>(qkv, q_weight, k_weight, eps, inv_freq, n_freq, positions, row_of_token,
+            launch_rope_token<bf16_t>(qkv, q_weight, k_weight, eps, inv_freq, n_freq, interleaved, positions, row_of_token,
                                       block_table, table_stride, page_size, (bf16_t*)q_out, (bf16_t*)k_cache,
                                       (bf16_t*)v_cache, write_kv, n_tokens, heads, kv_heads, head_dim, n_pages,
                                       v_transposed, s);
@@ -274,12 +276,12 @@ extern "C" int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight
     }
     if (dtype == IMPARO_F32)
         k_qk_norm_rope_store<float><<<blocks, ROPE_WAVES * WAVE, 0, s>>>(
-            qkv, q_weight, k_weight, eps, inv_freq, n_freq, positions, row_of_token, block_table, table_stride,
+            qkv, q_weight, k_weight, eps, inv_freq, n_freq, interleaved, positions, row_of_token, block_table, table_stride,
             page_size, (float*)q_out, (float*)k_cache, (float*)v_cache, write_kv, n_tokens, heads, kv_heads,
             head_dim, n_pages, v_transposed);
     else if (dtype == IMPARO_BF16)
         k_qk_norm_rope_store<bf16_t><<<blocks, ROPE_WAVES * WAVE, 0, s>>>(
-            qkv, q_weight, k_weight, eps, inv_freq, n_freq, positions, row_of_token, block_table, table_stride,
+            qkv, q_weight, k_weight, eps, inv_freq, n_freq, interleaved, positions, row_of_token, block_table, table_stride,
             page_size, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, write_kv, n_tokens, heads, kv_heads,
             head_dim, n_pages, v_transposed);
     else

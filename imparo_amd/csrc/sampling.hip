@@ -159,3 +159,10 @@ extern "C" int imparo_sample_rows(const float* logits, const float* temperature,
     k_sample_rows<<<n_rows, threads, 0, (hipStream_t)stream>>>(logits, temperature, uniform, out, vocab);
     return launch_status();
 }
+
+// The hash of the sources this library was built from (given by the build), so that a
+// library older than its sources is noticed when it is loaded.
+#ifndef IMPARO_SOURCE_HASH
+#define IMPARO_SOURCE_HASH "unknown"
+#endif
+extern "C" const char* imparo_hip_source_hash() { return IMPARO_SOURCE_HASH; }

@@ -85,14 +85,14 @@ class _Upload:
 
 class _DecodeGraph:
     """A captured decode step for one batch shape: `rows` single-token requests
-    whose block tables are `table_width` pages wide. Its index arrays, its
-    scratch and its logits live at fixed addresses; a replay reads new indices
-    from the same place."""
+    whose block tables are `table_width` pages wide. Its index arrays live at an
+    address of its own; scratch and logits are the engine's (buffers never move,
+    and the capture keeps those it was recorded with alive)."""
 
     def __init__(self):
         self.graph = None
         self.meta: Optional[torch.Tensor] = None
-        self.workspace: Optional[Workspace] = None
+        self.pinned: list = []
         self.logits: Optional[torch.Tensor] = None
         self.last_used = 0
 
@@ -102,10 +102,24 @@ MAX_GRAPHS = 96      # captured batch shapes kept; beyond that the one unused fo
 
 
 class Engine:
-    def __init__(self, model_dir: str, dtype: str = "bfloat16", max_tokens: int = 8192, page_size: int = 64,
-                 max_requests: int = 64, device: str = "cuda:0", use_graphs: bool = True):
+    """`max_tokens`: the most tokens that live requests hold at any time, each
+    request's count rounded up to whole pages; the pools are made for that
+    many. Instead, `kv_budget_bytes` gives the memory the paged caches may
+    take and the pools are as large as fits (the reference sizes its pool
+    from a memory budget the same way and carries a cap in pages for tests,
+    /root/reference/crates/imparo-model/src/kv.rs:574-621), or `num_pages`
+    gives the pool size outright (one number, or one per cache group).
+    `max_step_tokens` bounds the tokens of one step; a larger batch is refused."""
+
+    def __init__(self, model_dir: str, dtype: str = "bfloat16", max_tokens: Optional[int] = None, page_size: int = 64,
+                 max_requests: int = 64, device: str = "cuda:0", use_graphs: bool = True,
+                 kv_budget_bytes: Optional[int] = None, num_pages=None, max_step_tokens: int = 8192):
         if dtype not in DTYPES:
             raise ValueError(f"dtype must be one of {sorted(DTYPES)}, got {dtype!r}")
+        if sum(x is not None for x in (max_tokens, kv_budget_bytes, num_pages)) > 1:
+            raise ValueError("give one of max_tokens, kv_budget_bytes and num_pages")
+        if max_step_tokens < 1:
+            raise ValueError(f"max_step_tokens must be at least 1, got {max_step_tokens}")
         library()                       # fail now, and loudly, if the kernels are missing
         if not torch.cuda.is_available():
             raise RuntimeError("imparo_amd runs on a GPU; none is visible to this process")
@@ -121,14 +135,16 @@ class Engine:
         self.config, self.plan = plan_from_config(self.config_json)
         declared = declared_tensors(self.plan)
         tensors = load_weights(model_dir, {k: d for k, (d, _) in declared.items()}, self.plan.restated_tensors)
-        self.model = Model(self.plan, tensors, self.device, self.dtype)
+        self.model = Model(self.plan, tensors, self.device, self.dtype, page_size)
         f = tensors.pop("__file__", None)
         del tensors
         if f is not None:
             f.close()
         self.page_size = page_size
-        n_pages = max(1, math.ceil(max_tokens / page_size))
-        self.cache = CacheManager(self.model.site_specs, page_size, n_pages, max_requests)
+        self.max_step_tokens = max_step_tokens
+        pool_sizes = self.pool_sizes(self.model.site_specs, page_size, self.dtype, max_tokens, kv_budget_bytes,
+                                     num_pages)
+        self.cache = CacheManager(self.model.site_specs, page_size, pool_sizes, max_requests)
         self.storage = CacheStorage(self.cache, self.dtype, self.device)
         self.workspace = Workspace(self.device)
         self._upload = _Upload(self.device)
@@ -141,6 +157,32 @@ class Engine:
         self.vocab_size = self.plan.vocab_size
         self.max_position = self.plan.max_position
         self.steps_run = 0
+
+    @staticmethod
+    def pool_sizes(site_specs, page_size: int, dtype: torch.dtype, max_tokens: Optional[int],
+                   kv_budget_bytes: Optional[int], num_pages) -> List[int]:
+        """Pages per cache group. From `num_pages` as given; from a budget in
+        bytes: every group the same number of pages, as many as the budget
+        pays for over all sites (a page of a group costs page_size x the bytes
+        its sites keep per position); else from `max_tokens` (default 8,192)."""
+        groups = CacheManager.groups_of(site_specs)
+        if num_pages is not None:
+            sizes = [int(num_pages)] * len(groups) if isinstance(num_pages, int) else [int(n) for n in num_pages]
+            if len(sizes) != len(groups) or any(n < 1 for n in sizes):
+                raise ValueError(f"num_pages {num_pages!r} does not give {len(groups)} cache groups a pool each")
+            return sizes
+        if kv_budget_bytes is not None:
+            element = 4 if dtype == torch.float32 else 2
+            per_page = sum(spec.bytes_per_position(element) * len(sites) * page_size for spec, sites in groups)
+            if per_page == 0:
+                return []
+            n = int(kv_budget_bytes) // per_page
+            if n < 1:
+                raise ValueError(f"a cache budget of {kv_budget_bytes} bytes does not pay for one page of "
+                                 f"{per_page} bytes over all sites")
+            return [n] * len(groups)
+        tokens = 8192 if max_tokens is None else max_tokens
+        return [max(1, math.ceil(tokens / page_size))] * len(groups)
 
     # ------------------------------------------------------------ requests
     def length(self, request: Hashable) -> int:
@@ -162,10 +204,16 @@ class Engine:
         """Runs one batch. Returns float32 logits [wanted, vocab] on the
         device, in the order of the entries and of each entry's `want`, or
         None when nothing is wanted. The tensor is the engine's: a later step
-        may write its own logits there, so use it (or copy it) before the next."""
+        may write its own logits there, so use it (or copy it) before the next.
+        A batch that is refused (StepError) changes nothing. A step that fails
+        once its kernels have started leaves no request of the batch live."""
         entries = list(entries)
         if not entries:
             return None
+        n_tokens = sum(len(e.tokens) for e in entries)
+        if n_tokens > self.max_step_tokens:
+            raise StepError(f"a step of {n_tokens} tokens passes this engine's bound of {self.max_step_tokens} "
+                            f"(max_step_tokens); cut the prompts into smaller portions")
         # the native side checks the batch, admits, and reserves pages and slots, all or nothing
         token_lists = [e.tokens for e in entries]
         on_device = [(row, e.tokens[0]) for row, e in enumerate(entries)
@@ -189,8 +237,9 @@ class Engine:
         if code:
             raise StepError(self._refusal(code, entries[row]))
         try:
-            for slot in batch.new_slots[batch.new_slots >= 0].tolist():
-                self.storage.zero_slot(slot)
+            with ops.on_current_stream():
+                for slot in batch.new_slots[batch.new_slots >= 0].tolist():
+                    self.storage.reset_slot(slot)
             if (self.use_graphs and self.model.graph_safe and batch.T == len(entries)
                     and bool((batch.n_want == 1).all())):
                 logits = self._decode_step(entries, batch)       # one token each, wanted
@@ -199,7 +248,13 @@ class Engine:
                 with ops.on_current_stream():
                     logits = self.model.forward(ctx, token_ids, want_rows)
         except BaseException:
+            # Pages and new admissions are rolled back. Fixed-size state is not a thing that can be
+            # rolled back (a conv history has been shifted by the layers that ran), so the requests
+            # of a step that failed after its first launch cannot go on: they are released, and a
+            # caller that wants them recomputes them from their tokens.
             self.cache.abort_step(batch)
+            for e in entries:
+                self.release(e.request)
             raise
         self.cache.end_step(batch)
         self.steps_run += 1
@@ -235,27 +290,26 @@ class Engine:
                 return self.model.forward(ctx, token_ids, want_rows)
         g = self._graphs.get(key)
         if g is None:
-            if len(self._graphs) >= MAX_GRAPHS:      # each holds a workspace and a logits buffer
+            if len(self._graphs) >= MAX_GRAPHS:      # each holds an executable graph and its index arrays
                 del self._graphs[min(self._graphs, key=lambda k: self._graphs[k].last_used)]
             g = self._graphs[key] = _DecodeGraph()
         g.last_used = self.steps_run
         if g.graph is None:
-            g.workspace = Workspace(self.device)
             # the capture fixes grid sizes: they are sized for the widest context the tables can hold
-            ctx, token_ids, want_rows = self._pack(batch, table_width=width, workspace=g.workspace, graph=g)
+            ctx, token_ids, want_rows = self._pack(batch, table_width=width, graph=g)
             if self._graph_pool is None:
                 self._graph_pool = torch.cuda.graph_pool_handle()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, pool=self._graph_pool), ops.on_current_stream():
                 g.logits = self.model.forward(ctx, token_ids, want_rows)
+            g.pinned = self.workspace.pin()          # the buffers whose addresses the graph holds
             g.graph = graph
         else:
-            self._pack(batch, table_width=width, workspace=g.workspace, graph=g)
+            self._pack(batch, table_width=width, graph=g)
         g.graph.replay()
         return g.logits
 
-    def _pack(self, batch, table_width: Optional[int] = None,
-              workspace: Optional[Workspace] = None, graph: Optional[_DecodeGraph] = None):
+    def _pack(self, batch, table_width: Optional[int] = None, graph: Optional[_DecodeGraph] = None):
         """Builds the step's index arrays, sends them to the device in one
         copy and wraps them in a StepContext. For a captured step the arrays go
         to the capture's own fixed buffer and sizes are the capture's bounds."""
@@ -287,12 +341,12 @@ class Engine:
             positions=dev[o_pos:o_pos + T], row_of_token=dev[o_row:o_row + T],
             seg_start=dev[o_start:o_start + R], seg_len=dev[o_len:o_len + R], slot=dev[o_slot:o_slot + R],
             block_tables=block_tables, page_size=self.page_size, dtype=self.dtype,
-            workspace=workspace or self.workspace, storage=self.storage, group_of_site=self.cache.group_of_site,
+            workspace=self.workspace, storage=self.storage, group_of_site=self.cache.group_of_site,
             max_seg_len=lay["max_seg_len"],
             max_context=lay["max_context"] if table_width is None else table_width * self.page_size,
-            decode_rows=dev[o_lists:o_lists + n_dec], n_decode_rows=n_dec,
-            prefill_rows=dev[o_lists + n_dec:o_lists + R], n_prefill_rows=lay["n_multi"],
-            n_prefill_tiles=lay["n_prefill_tiles"],
+            single_rows=dev[o_lists:o_lists + n_dec], n_single_rows=n_dec,
+            portion_rows=dev[o_lists + n_dec:o_lists + R], n_portion_rows=lay["n_multi"],
+            host_seg_len=batch.n_tok,
         )
         want_rows = dev[o_want:o_want + W] if W else None
         return ctx, dev[o_tok:o_tok + T], want_rows

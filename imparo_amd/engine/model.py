@@ -35,10 +35,8 @@ def declared_tensors(plan: ModelPlan) -> Declared:
 
     add(_declare("embedding", plan.embedding))
     for layer in plan.layers:
-        add(_declare("norm", layer.mixer_norm))
-        add(_declare("mixer", layer.mixer))
-        add(_declare("norm", layer.ffn_norm))
-        add(_declare("feed_forward", layer.ffn))
+        for role, spec in layer.parts.values():
+            add(_declare(role, spec))
     add(_declare("norm", plan.final_norm))
     add(_declare("head", plan.head))
     return out
@@ -46,7 +44,7 @@ def declared_tensors(plan: ModelPlan) -> Declared:
 
 class Model:
     def __init__(self, plan: ModelPlan, tensors: Dict[str, torch.Tensor], device: torch.device,
-                 dtype: torch.dtype):
+                 dtype: torch.dtype, page_size: int):
         plan.validate()
         self.plan = plan
         self.device = device
@@ -54,31 +52,30 @@ class Model:
         placed: Dict[str, torch.Tensor] = {}
         self.embedding = part_class("embedding", plan.embedding.kind)(plan.embedding, tensors, device, dtype, placed)
         self.blocks = []
+        built = []
         for layer in plan.layers:
-            mk = lambda role, spec: part_class(role, spec.kind)(spec, tensors, device, dtype)
-            block_cls = part_class("block", layer.arrangement)
-            self.blocks.append(block_cls(mk("norm", layer.mixer_norm), mk("mixer", layer.mixer),
-                                         mk("norm", layer.ffn_norm), mk("feed_forward", layer.ffn)))
+            parts = {name: part_class(role, spec.kind)(spec, tensors, device, dtype)
+                     for name, (role, spec) in layer.parts.items()}
+            built += list(parts.values())
+            self.blocks.append(part_class("block", layer.arrangement)(parts))
         self.final_norm = part_class("norm", plan.final_norm.kind)(plan.final_norm, tensors, device, dtype)
         self.head = part_class("head", plan.head.kind)(plan.head, tensors, device, dtype, placed)
         # a step can be captured into a graph only if every part says it launches kernels and nothing else
-        parts = [self.embedding, self.final_norm, self.head] + self.blocks
-        for b in self.blocks:
-            parts += [b.mixer_norm, b.mixer, b.ffn_norm, b.ffn] if hasattr(b, "mixer_norm") else []
-        self.graph_safe = all(getattr(p, "graph_safe", False) for p in parts)
+        self.graph_safe = all(getattr(p, "graph_safe", False)
+                              for p in [self.embedding, self.final_norm, self.head] + self.blocks + built)
         # cache sites: one per entry of the run order; None where the call borrows
         self.site_of_call: List[int] = []
         self.site_specs: List[StateSpec] = []
         for i, call in enumerate(plan.order):
-            mixer = self.blocks[call.layer].mixer
+            spec = self.blocks[call.layer].cache_spec(page_size)
             if call.cache_of is None:
                 self.site_of_call.append(i)
-                self.site_specs.append(mixer.cache_spec())
+                self.site_specs.append(spec)
             else:
                 self.site_of_call.append(call.cache_of)
                 self.site_specs.append(None)
                 owner = self.site_specs[call.cache_of]
-                if owner != mixer.cache_spec():
+                if owner != spec:
                     raise ValueError(f"run order entry {i} reads the cache of entry {call.cache_of}, "
                                      f"whose state has another shape")
 

@@ -333,13 +333,16 @@ class Scheduler:
 def generate(model, input_ids: Sequence[Sequence[int]], max_tokens: int = 16, temperature: float = 0.0,
              seed: int = 0, stop_token_ids: Optional[Sequence[int]] = None, dtype: str = "bfloat16",
              ctx: Optional[int] = None, parallel: int = 64, max_batch_tokens: int = 2048,
-             page_size: int = 64, overlap: bool = True) -> List[List[int]]:
+             page_size: int = 64, overlap: bool = True, num_pages=None,
+             kv_budget_bytes: Optional[int] = None) -> List[List[int]]:
     """Tokens in, tokens out. `model` is a model folder or an Engine; returns
     the generated ids of every prompt, in order. Request `i` samples with seed
     `seed + i`. `ctx` is the most tokens one request may hold (the reference's
     -c/--ctx), `parallel` the most requests that run at once (-np/--parallel).
     `overlap`: queue each step before the tokens of the step before are read
-    back (the same tokens come out; False waits after every step)."""
+    back (the same tokens come out; False waits after every step).
+    `num_pages` or `kv_budget_bytes` size the cache pools instead of `ctx` and
+    `parallel` (a smaller pool makes requests wait or be recomputed)."""
     from .engine import Engine
     from ..sampling.sampler import Sampler
     if isinstance(model, Engine):
@@ -349,8 +352,10 @@ def generate(model, input_ids: Sequence[Sequence[int]], max_tokens: int = 16, te
         per_request = ctx or longest
         n_live = min(parallel, len(input_ids))
         rounded = ((per_request + page_size - 1) // page_size + 1) * page_size
-        engine = Engine(model, dtype=dtype, max_tokens=rounded * n_live, page_size=page_size,
-                        max_requests=max(1, n_live))
+        sized = num_pages is not None or kv_budget_bytes is not None
+        engine = Engine(model, dtype=dtype, max_tokens=None if sized else rounded * n_live, page_size=page_size,
+                        max_requests=max(1, n_live), num_pages=num_pages, kv_budget_bytes=kv_budget_bytes,
+                        max_step_tokens=max(max_batch_tokens, 1))
     stops = tuple(stop_token_ids) if stop_token_ids is not None else tuple(engine.plan.stop_token_ids)
     sampler = Sampler(engine.device)
     sched = Scheduler(engine, sampler.pick, max_batch_tokens=max_batch_tokens,

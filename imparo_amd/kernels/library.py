@@ -24,22 +24,25 @@ _SIGNATURES = {
     "imparo_embed_gather": [P, I, P, P, I, I, I, P],
     "imparo_place_tokens": [P, P, P, P, I, I, P],
     "imparo_rms_norm": [P, P, I, I, P, P, P, I, I, I, F, I, P],
-    "imparo_silu_mul": [P, I, P, I, I, I, P],
-    "imparo_add_bias": [P, P, I, I, P],
     "imparo_gemm": [P, P, P, P, I, I, I, I, I, I, I, P],
     "imparo_gemm_slices": [I, I, I, I],
+    "imparo_gemm_variant": [P, P, P, P, I, I, I, I, I, I, I, I, P],
     "imparo_short_conv_decode": [P, P, P, P, P, P, I, I, I, I, I, P],
     "imparo_in_proj_conv_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
-    "imparo_qk_norm_rope_store": [P, P, P, F, P, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, P],
+    "imparo_qk_norm_rope_store": [P, P, P, F, P, I, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, P],
     "imparo_attention": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
     "imparo_attention_decode": [P, P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
     "imparo_attention_prefill": [P, P, P, P, P, P, I, P, I, I, P, P, P, P, I, I, I, I, I, I, F, I, P],
     "imparo_attention_prefill_splits": [I, I, I, I, I],
+    "imparo_attention_decode_split": [],
+    "imparo_attention_prefill_tile": [],
     "imparo_short_conv": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
     "imparo_short_conv_state": [P, P, P, P, P, I, I, I, I, I, P],
     "imparo_argmax_rows": [P, P, I, I, P],
     "imparo_sample_rows": [P, P, P, P, I, I, P],
     "imparo_fill_f32": [P, F, c_int64, P],
+    "imparo_fill_sites": [P, P, P, I, I, P],
+    "imparo_attention_decode_static": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
 }
 
 
@@ -56,14 +59,20 @@ def library() -> ctypes.CDLL:
             return _lib
         path = _build.library_path()
         if not os.path.isfile(path):
-            try:
-                path = _build.build(verbose=True)
-            except Exception as e:  # no silent fallback: say why there is no library
-                raise KernelLibraryError(f"the gfx950 kernel library is not built and building it failed: {e}") from e
+            path = _rebuild("is not built")
         try:
             lib = ctypes.CDLL(path)
         except OSError as e:
             raise KernelLibraryError(f"cannot load {path}: {e}") from e
+        built_from = _hash_in(lib, "imparo_hip_source_hash")
+        if built_from != _build.source_hash():
+            # older than its sources (or from before libraries carried a hash): never used silently
+            import _ctypes
+            _ctypes.dlclose(lib._handle)
+            path = _rebuild(f"at {path} was built from other sources ({built_from}) than those beside it")
+            lib = ctypes.CDLL(path)
+            if _hash_in(lib, "imparo_hip_source_hash") != _build.source_hash():
+                raise KernelLibraryError(f"{path} still does not match its sources after a rebuild")
         for name, argtypes in _SIGNATURES.items():
             try:
                 fn = getattr(lib, name)
@@ -74,6 +83,23 @@ def library() -> ctypes.CDLL:
             fn.restype = c_int
         _lib = lib
         return _lib
+
+
+def _hash_in(lib: ctypes.CDLL, name: str) -> str:
+    try:
+        fn = getattr(lib, name)
+    except AttributeError:
+        return "none"
+    fn.restype = ctypes.c_char_p
+    fn.argtypes = []
+    return fn().decode("ascii", "replace")
+
+
+def _rebuild(why: str) -> str:
+    try:
+        return _build.build(verbose=True)
+    except Exception as e:  # no silent fallback: say why there is no library
+        raise KernelLibraryError(f"the gfx950 kernel library {why} and building it failed: {e}") from e
 
 
 def loaded_path() -> str:

@@ -127,37 +127,18 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tenso
     return out
 
 
-def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    n, two_h = gu.shape
-    hidden = two_h // 2
-    if two_h != 2 * hidden:
-        raise KernelArgumentError("silu_mul: the input row must hold gate and up halves")
-    _check(library().imparo_silu_mul(_dev(gu, "silu_mul input"), _code(gu, "silu_mul input"),
-                                     _dev(out, "silu_mul output", None, (n, hidden)), _code(out, "silu_mul output"),
-                                     n, hidden, _stream()), "silu_mul")
-    return out
-
-
-def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
-    """y += bias on every row (the GEMM kernels add a bias themselves; this is
-    for other producers)."""
-    m, n = y.shape
-    _check(library().imparo_add_bias(_dev(y, "add_bias y", torch.float32), _dev(bias, "bias", torch.float32, (n,)),
-                                     m, n, _stream()), "add_bias")
-    return y
-
-
 def gemm_slices(m: int, n: int, k: int, dtype: torch.dtype) -> int:
     """Into how many slices of K this product may be cut when its consumer adds the slices (1: none)."""
     return int(library().imparo_gemm_slices(m, n, k, _CODES.get(dtype, -1)))
 
 
 def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
-         swiglu: bool = False) -> torch.Tensor:
+         swiglu: bool = False, variant: int = 0) -> torch.Tensor:
     """out[m, n] = x[m, k] . w[n, k]^T (+ bias[n]); x and w share a dtype; float32
     accumulate. With `swiglu` the rows of w alternate gate and up and out is
     [m, n/2] = silu(gate) * up. An `out` of shape [slices, m, n] (slices =
-    gemm_slices(...)) receives the sums over slices of K, to be added by the consumer."""
+    gemm_slices(...)) receives the sums over slices of K, to be added by the consumer.
+    `variant` other than 0 names the kernel (tests and measurements only; see imparo_gemm_variant)."""
     m, k = x.shape
     n, kw = w.shape
     if kw != k:
@@ -171,14 +152,17 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[tor
     slices = 1
     if out.dim() == 3:
         slices = out.shape[0]
-        if slices != gemm_slices(m, n, k, x.dtype) or swiglu or out.dtype != torch.float32:
+        if (slices != gemm_slices(m, n, k, x.dtype) and not variant) or swiglu or out.dtype != torch.float32:
             raise KernelArgumentError(f"gemm: this product cannot be cut into {slices} slices of K")
         _dev(out, "gemm out", torch.float32, (slices, m, n))
     else:
         _dev(out, "gemm out", None, (m, n // 2 if swiglu else n))
-    _check(library().imparo_gemm(_dev(x, "gemm x"), _dev(w, "gemm weight"), _dev(bias, "gemm bias", torch.float32, (n,)),
-                                 out.data_ptr(), _code(x, "gemm x"), _code(out, "gemm out"), m, n, k, int(swiglu),
-                                 slices, _stream()), "gemm")
+    args = (_dev(x, "gemm x"), _dev(w, "gemm weight"), _dev(bias, "gemm bias", torch.float32, (n,)),
+            out.data_ptr(), _code(x, "gemm x"), _code(out, "gemm out"), m, n, k, int(swiglu), slices)
+    if variant:
+        _check(library().imparo_gemm_variant(*args, int(variant), _stream()), "gemm")
+    else:
+        _check(library().imparo_gemm(*args, _stream()), "gemm")
     return out
 
 
@@ -186,7 +170,10 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_we
                        eps: float, inv_freq: Optional[torch.Tensor], positions: torch.Tensor,
                        row_of_token: torch.Tensor, block_table: Optional[torch.Tensor], page_size: int,
                        q_out: torch.Tensor, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                       heads: int, kv_heads: int, head_dim: int, v_transposed: bool = False) -> torch.Tensor:
+                       heads: int, kv_heads: int, head_dim: int, v_transposed: bool = False,
+                       interleaved: bool = False) -> torch.Tensor:
+    """`inv_freq` [n] turns pair i by position * inv_freq[i]: pair i is dims (i, i + n), or with
+    `interleaved` dims (2i, 2i + 1)."""
     n = qkv.shape[0]
     units = heads + 2 * kv_heads
     write_kv = k_cache is not None
@@ -205,7 +192,7 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_we
         _dev(qkv, "qkv", torch.float32, (n, units * head_dim)),
         _dev(q_weight, "q norm weight", torch.float32, (head_dim,)),
         _dev(k_weight, "k norm weight", torch.float32, (head_dim,)), float(eps),
-        _dev(inv_freq, "inverse frequencies", torch.float32), n_freq,
+        _dev(inv_freq, "inverse frequencies", torch.float32), n_freq, int(interleaved),
         _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
         _dev(block_table, "block table", torch.int32), table_stride, page_size,
         _dev(q_out, "q out", None, (n, heads, head_dim)), _dev(k_cache, "k cache"), _dev(v_cache, "v cache"),
@@ -238,7 +225,14 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out
     return out
 
 
-DECODE_SPLIT = 256
+def decode_split() -> int:
+    """Keys per split of the matrix-core decode kernel: its partial results hold one entry per split."""
+    return int(library().imparo_attention_decode_split())
+
+
+def prefill_tile() -> int:
+    """Queries per tile that `attention_prefill`'s n_tiles counts."""
+    return int(library().imparo_attention_prefill_tile())
 
 
 def mfma_attention_supported(dtype: torch.dtype, page_size: int, head_dim: int) -> bool:
@@ -266,7 +260,8 @@ def attention_decode(q, k_cache, v_cache, out, part_o, part_ml, rows, n_rows: in
     """Split-KV attention for rows that bring one token each. `rows` lists
     them (indices into seg_start); `max_context` bounds every row's position + 1."""
     n, heads, head_dim, n_pages, kv_heads, page_size = _check_mfma(q, k_cache, v_cache, out)
-    n_splits = max(1, (max_context + DECODE_SPLIT - 1) // DECODE_SPLIT)
+    split = decode_split()
+    n_splits = max(1, (max_context + split - 1) // split)
     if part_o.numel() < n_rows * heads * n_splits * head_dim or part_ml.numel() < n_rows * heads * n_splits * 2:
         raise KernelArgumentError("attention_decode: the scratch for partial results is too small")
     _check(library().imparo_attention_decode(
@@ -289,7 +284,7 @@ def attention_prefill(q, k_cache, v_cache, out, rows, n_rows: int, n_tiles: int,
                       block_table, scale: float, window: Optional[int], part_o: Optional[torch.Tensor] = None,
                       part_ml: Optional[torch.Tensor] = None, n_splits: int = 1) -> torch.Tensor:
     """Tiled attention for rows that bring a portion of a prompt. `n_tiles` is
-    the sum over the listed rows of ceil(seg_len / 64). With `n_splits` > 1
+    the sum over the listed rows of ceil(seg_len / prefill_tile()). With `n_splits` > 1
     (attention_prefill_splits) each block's keys are walked in that many parts,
     merged by a second launch: `part_o` [n, heads, n_splits, head_dim] and
     `part_ml` [n, heads, n_splits, 2] float32 hold the parts."""
@@ -399,3 +394,13 @@ def fill_f32(t: torch.Tensor, value: float) -> torch.Tensor:
     _check(library().imparo_fill_f32(_dev(t, "fill target", torch.float32), float(value), t.numel(), _stream()),
            "fill_f32")
     return t
+
+
+def fill_sites(base: torch.Tensor, per_slot: torch.Tensor, value: torch.Tensor, slot: int) -> None:
+    """Sets one slot's row of every fixed-state site in one launch: site i's row is per_slot[i]
+    float32 values at address base[i] + slot * per_slot[i] * 4 and becomes value[i] everywhere."""
+    n = base.shape[0]
+    _check(library().imparo_fill_sites(_dev(base, "site addresses", torch.int64, (n,)),
+                                       _dev(per_slot, "site row sizes", torch.int64, (n,)),
+                                       _dev(value, "site values", torch.float32, (n,)), n, int(slot), _stream()),
+           "fill_sites")

@@ -12,7 +12,7 @@ from typing import Dict, Optional
 
 import torch
 
-from ..cache.pages import PagedSpec
+from ..cache.pages import PagedSpec, kv_spec
 from ..config.plan import PartSpec
 from ..kernels import ops
 from ..weights.loader import TensorDecl
@@ -51,6 +51,8 @@ class Attention:
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
                  engine_dtype: torch.dtype):
         n = self._names(spec)
+        self.engine_dtype = engine_dtype
+        self.v_transposed = False        # decided with the cache's page size, in cache_spec
         self.width, self.heads, self.kv_heads, self.head_dim = (spec["width"], spec["heads"], spec["kv_heads"],
                                                                 spec["head_dim"])
         if self.head_dim % 16:
@@ -81,41 +83,56 @@ class Attention:
     def in_dtype(self) -> torch.dtype:
         return self.qkv.in_dtype
 
-    def cache_spec(self) -> PagedSpec:
-        return PagedSpec(self.kv_heads, self.head_dim, self.window)
+    def cache_spec(self, page_size: int) -> PagedSpec:
+        """Keys and values per position, laid out as this mixer's kernels read
+        them: where the matrix-core kernels apply (bfloat16, pages of at least
+        16, head sizes up to 128), V is kept transposed inside a page."""
+        self.v_transposed = ops.mfma_attention_supported(self.engine_dtype, page_size, self.head_dim)
+        return kv_spec(self.kv_heads, self.head_dim, self.window, self.v_transposed)
+
+    def _portion_tiles(self, ctx: StepContext) -> int:
+        """Tiles of queries that the portions of this batch make, as the prompt kernel counts them."""
+        key = ("attention portion tiles", ops.prefill_tile())
+        if key not in ctx.memo:
+            tile = ops.prefill_tile()
+            ctx.memo[key] = sum((int(n) + tile - 1) // tile for n in ctx.host_seg_len if n > 1)
+        return ctx.memo[key]
 
     def forward(self, ctx: StepContext, site: int, owns_cache: bool, h: torch.Tensor) -> torch.Tensor:
         T = h.shape[0]
-        qkv = self.qkv(ctx, h, torch.float32, "qkv")
+        qkv = self.qkv(ctx, h, torch.float32, "qkv", alias="mixer_in")
         k_cache, v_cache, table = ctx.kv(site)
-        vt = ctx.v_transposed(site)
+        vt = self.v_transposed
         q = ctx.workspace.get("q", (T, self.heads, self.head_dim), ctx.dtype)
         ops.qk_norm_rope_store(qkv, self.q_norm, self.k_norm, self.norm_eps, self.position.inv_freq,
                                ctx.positions, ctx.row_of_token, table if owns_cache else None, ctx.page_size,
                                q, k_cache if owns_cache else None, v_cache if owns_cache else None,
-                               self.heads, self.kv_heads, self.head_dim, v_transposed=vt)
-        o = ctx.workspace.get("attn_out", (T, self.heads * self.head_dim), ctx.dtype)
-        if vt and ctx.decode_rows is not None:
+                               self.heads, self.kv_heads, self.head_dim, v_transposed=vt,
+                               interleaved=bool(getattr(self.position, "interleaved", False)))
+        o = ctx.workspace.get("attn_out", (T, self.heads * self.head_dim), ctx.dtype, alias="mixer_mid")
+        if vt and ctx.single_rows is not None:
             # matrix-core kernels: single tokens split over their keys, portions tiled over their queries
-            if ctx.n_decode_rows:
-                n_splits = (ctx.max_context + ops.DECODE_SPLIT - 1) // ops.DECODE_SPLIT
-                part_o = ctx.workspace.get("attn_part_o", (ctx.n_decode_rows * self.heads * n_splits * self.head_dim,),
+            if ctx.n_single_rows:
+                split = ops.decode_split()
+                n_splits = (ctx.max_context + split - 1) // split
+                part_o = ctx.workspace.get("attn_part_o", (ctx.n_single_rows * self.heads * n_splits * self.head_dim,),
                                            torch.float32)
-                part_ml = ctx.workspace.get("attn_part_ml", (ctx.n_decode_rows * self.heads * n_splits * 2,),
+                part_ml = ctx.workspace.get("attn_part_ml", (ctx.n_single_rows * self.heads * n_splits * 2,),
                                             torch.float32)
-                ops.attention_decode(q, k_cache, v_cache, o, part_o, part_ml, ctx.decode_rows, ctx.n_decode_rows,
+                ops.attention_decode(q, k_cache, v_cache, o, part_o, part_ml, ctx.single_rows, ctx.n_single_rows,
                                      ctx.seg_start, ctx.positions, table, self.scale, self.window, ctx.max_context)
-            if ctx.n_prefill_rows:
+            if ctx.n_portion_rows:
                 # few queries over long contexts: each block's keys in parts, merged by a second launch
-                parts = ops.attention_prefill_splits(ctx.n_prefill_tiles, self.heads, self.kv_heads, self.head_dim,
+                n_tiles = self._portion_tiles(ctx)
+                parts = ops.attention_prefill_splits(n_tiles, self.heads, self.kv_heads, self.head_dim,
                                                      ctx.max_context)
                 part_o = part_ml = None
                 if parts > 1:
                     part_o = ctx.workspace.get("attn_prefill_part_o", (T * self.heads * parts * self.head_dim,),
                                                torch.float32)
                     part_ml = ctx.workspace.get("attn_prefill_part_ml", (T * self.heads * parts * 2,), torch.float32)
-                ops.attention_prefill(q, k_cache, v_cache, o, ctx.prefill_rows, ctx.n_prefill_rows,
-                                      ctx.n_prefill_tiles, ctx.seg_start, ctx.seg_len, ctx.positions, table,
+                ops.attention_prefill(q, k_cache, v_cache, o, ctx.portion_rows, ctx.n_portion_rows,
+                                      n_tiles, ctx.seg_start, ctx.seg_len, ctx.positions, table,
                                       self.scale, self.window, part_o, part_ml, parts)
         else:
             ops.attention(q, k_cache, v_cache, o, ctx.positions, ctx.row_of_token, table, self.scale, self.window,

@@ -6,8 +6,8 @@ beyond its row, or how the batch was cut.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
-from typing import Dict, Optional, Tuple
+from dataclasses import dataclass, field
+from typing import Dict, Optional, Sequence, Tuple
 
 import torch
 
@@ -20,22 +20,46 @@ Declared = Dict[str, Tuple[TensorDecl, str]]
 class Workspace:
     """Named scratch tensors that live across steps, so a step allocates
     nothing once sizes have been seen. Kernels of one step run in order on one
-    stream, so a name can be reused by every layer."""
+    stream, so a name can be reused by every layer.
+
+    Buffers never move: a name that needs more room gets a new buffer (at
+    least twice the old size) and the old one stays alive as long as a
+    captured step that was recorded with it does (`pin`), so every captured
+    shape can share this one workspace. Names that are never live at the same
+    time may share memory: `alias` names the group they share, which is as
+    large as its largest member (a layer's attention scratch and its conv
+    scratch; what a mixer used and what the feed-forward after it uses). The
+    reference plans its activation buffers the same way, in alias groups that
+    follow a block's order of work
+    (/root/reference/crates/imparo-model/src/lfm2/workflow_gpu.rs:110-183)."""
 
     def __init__(self, device: torch.device):
         self.device = device
-        self._buffers: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        self._buffers: Dict[str, torch.Tensor] = {}      # by name or alias group: raw bytes
 
-    def get(self, name: str, shape: Tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+    def get(self, name: str, shape: Tuple[int, ...], dtype: torch.dtype, alias: Optional[str] = None) -> torch.Tensor:
         n = 1
         for s in shape:
             n *= s
-        key = (name, dtype)
+        need = max(n, 1) * _ELEMENT_SIZE[dtype]
+        key = alias or name
         buf = self._buffers.get(key)
-        if buf is None or buf.numel() < n:
-            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+        if buf is None or buf.numel() < need:
+            grown = need if buf is None else max(need, 2 * buf.numel())
+            buf = torch.empty((grown + 255) // 256 * 256, dtype=torch.uint8, device=self.device)
             self._buffers[key] = buf
-        return buf[:n].view(shape)
+        return buf[:n * _ELEMENT_SIZE[dtype]].view(dtype).view(shape)
+
+    def pin(self) -> list:
+        """The buffers as they are now, to be kept by whoever recorded their addresses."""
+        return list(self._buffers.values())
+
+    def bytes(self) -> int:
+        return sum(b.numel() for b in self._buffers.values())
+
+
+_ELEMENT_SIZE = {torch.float32: 4, torch.bfloat16: 2, torch.int32: 4, torch.float16: 2, torch.int64: 8,
+                 torch.uint8: 1}
 
 
 @dataclass
@@ -46,6 +70,10 @@ class StepContext:
     sits at absolute position `positions[t]`; row r's tokens are
     [seg_start[r], seg_start[r] + seg_len[r]) and its fixed state lives in
     slot `slot[r]`; `block_tables[g]` is [rows, pages] for cache group g.
+    `single_rows` lists the rows that bring one token, `portion_rows` those
+    that bring more (indices into seg_start). `host_seg_len` is seg_len on the
+    host, for parts whose launches depend on it; a captured step has none
+    beyond "every row brings one token".
     """
     n_tokens: int
     n_rows: int
@@ -61,20 +89,21 @@ class StepContext:
     storage: "object"                   # imparo_amd.cache.storage.CacheStorage
     group_of_site: Dict[int, int]
     max_seg_len: int = 1                # host copy: longest segment of the batch
-    max_context: int = 0                # host copy: longest context after this step
-    # rows that bring one token / more than one, as index lists into seg_start
-    decode_rows: Optional[torch.Tensor] = None
-    n_decode_rows: int = 0
-    prefill_rows: Optional[torch.Tensor] = None
-    n_prefill_rows: int = 0
-    n_prefill_tiles: int = 0            # sum over prefill rows of ceil(seg_len / 64)
+    max_context: int = 0                # host copy: longest context after this step (a captured step: its bound)
+    single_rows: Optional[torch.Tensor] = None
+    n_single_rows: int = 0
+    portion_rows: Optional[torch.Tensor] = None
+    n_portion_rows: int = 0
+    host_seg_len: Optional[Sequence[int]] = None
+    memo: Dict[object, object] = field(default_factory=dict)   # what parts derive from the batch, once a step
+
+    def paged(self, site: int):
+        """The site's paged arrays by name, and the block table of its group."""
+        return self.storage.paged[site], self.block_tables[self.group_of_site[site]]
 
     def kv(self, site: int):
-        k, v = self.storage.kv[site]
-        return k, v, self.block_tables[self.group_of_site[site]]
-
-    def v_transposed(self, site: int) -> bool:
-        return bool(getattr(self.storage, "v_transposed", {}).get(site, False))
+        arrays, table = self.paged(site)
+        return arrays["k"], arrays["v"], table
 
     def fixed_state(self, site: int) -> torch.Tensor:
         return self.storage.fixed[site]

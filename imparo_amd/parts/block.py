@@ -6,17 +6,25 @@ delta is left pending on the residual stream so that the next norm, whichever
 block it belongs to, adds it while reading the row."""
 from __future__ import annotations
 
+from typing import Dict
 
 from .base import Residual, StepContext
 from .registry import register_part
 
 
 class PreNormBlock:
+    """Reads four parts by name: mixer_norm, mixer, ffn_norm, ffn."""
     role = "block"
     graph_safe = True     # launches kernels only: a step made of such parts can be captured
 
-    def __init__(self, mixer_norm, mixer, ffn_norm, ffn):
-        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+    def __init__(self, parts: Dict[str, object]):
+        self.parts = parts
+        self.mixer_norm, self.mixer = parts["mixer_norm"], parts["mixer"]
+        self.ffn_norm, self.ffn = parts["ffn_norm"], parts["ffn"]
+
+    def cache_spec(self, page_size: int):
+        """What a call of this block keeps between steps: its mixer's state."""
+        return self.mixer.cache_spec(page_size)
 
     def forward(self, ctx: StepContext, res: Residual, site: int, owns_cache: bool) -> None:
         h = self.mixer_norm.forward(ctx, res, self.mixer.in_dtype)

@@ -28,11 +28,12 @@ class Linear:
         return self.weight.dtype
 
     def __call__(self, ctx: StepContext, x: torch.Tensor, out_dtype: torch.dtype, name: str,
-                 swiglu: bool = False, sliced_ok: bool = False) -> torch.Tensor:
+                 swiglu: bool = False, sliced_ok: bool = False, alias: Optional[str] = None) -> torch.Tensor:
         """`swiglu`: the weight's rows alternate gate and up; the output is
         silu(gate) * up, half as wide. `sliced_ok`: the caller's consumer adds
         slices, so the result may come as [slices, rows, out] sums over parts
-        of K (few rows and a long K keep more of the chip busy that way)."""
+        of K (few rows and a long K keep more of the chip busy that way).
+        `alias`: the workspace group the output may share memory with."""
         width = self.out_features // 2 if swiglu else self.out_features
         m = x.shape[0]
         if sliced_ok and not swiglu and out_dtype == torch.float32:
@@ -40,7 +41,7 @@ class Linear:
             if slices > 1:
                 out = ctx.workspace.get(name + "_sliced", (slices, m, width), out_dtype)
                 return ops.gemm(x, self.weight, out, bias=self.bias)
-        out = ctx.workspace.get(name, (m, width), out_dtype)
+        out = ctx.workspace.get(name, (m, width), out_dtype, alias=alias)
         return ops.gemm(x, self.weight, out, bias=self.bias, swiglu=swiglu)
 
 

@@ -1,6 +1,7 @@
-"""Position encodings. A position part owns a table of inverse frequencies;
-the attention mixer hands it to the fused norm+rotation kernel together with
-each token's absolute position.
+"""Position encodings. A position part owns a table of inverse frequencies
+and says which dimensions make a pair (`interleaved` False: i with i +
+rotary_dim/2; True: 2i with 2i + 1); the attention mixer hands both to the
+fused norm+rotation kernel together with each token's absolute position.
 
 NeoX rotation: dimension i pairs with i + rotary_dim/2, inv_i =
 base^(-2i/rotary_dim), angle = position * inv_i
@@ -18,6 +19,7 @@ from .registry import register_part
 
 class RopeNeox:
     role = "position"
+    interleaved = False
 
     def __init__(self, spec: PartSpec, device: torch.device):
         self.rotary_dim = int(spec["rotary_dim"])
@@ -37,6 +39,8 @@ class RopeNeox:
 class NoPosition:
     """No rotation: keys are cached as the norm leaves them."""
     role = "position"
+
+    interleaved = False
 
     def __init__(self, spec: PartSpec, device: torch.device):
         self.rotary_dim = 0

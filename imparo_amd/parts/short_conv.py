@@ -59,20 +59,20 @@ class ShortConv:
     def in_dtype(self) -> torch.dtype:
         return self.in_proj.in_dtype
 
-    def cache_spec(self) -> FixedSpec:
+    def cache_spec(self, page_size: int) -> FixedSpec:
         return FixedSpec((self.taps - 1, self.width))
 
     def forward(self, ctx: StepContext, site: int, owns_cache: bool, h: torch.Tensor) -> torch.Tensor:
         if not owns_cache:
             raise ValueError("a short conv's state cannot be read from another layer")
         T = h.shape[0]
-        y = ctx.workspace.get("conv_out", (T, self.width), self.out_proj.in_dtype)
+        y = ctx.workspace.get("conv_out", (T, self.width), self.out_proj.in_dtype, alias="mixer_mid")
         if ctx.max_seg_len == 1 and ops.in_proj_conv_decode_supported(T, self.in_proj.weight):
             # a decode step's few rows: projection and conv in one launch
             ops.in_proj_conv_decode(h, self.in_proj.weight, self.in_proj.bias, self.conv_weight, self.conv_bias,
                                     ctx.fixed_state(site), ctx.slot, y)
             return self.out_proj(ctx, y, torch.float32, "mixer_out", sliced_ok=True)
-        bcx = self.in_proj(ctx, h, torch.float32, "bcx")
+        bcx = self.in_proj(ctx, h, torch.float32, "bcx", alias="mixer_in")
         ops.short_conv(bcx, self.conv_weight, self.conv_bias, ctx.fixed_state(site), ctx.row_of_token,
                        ctx.seg_start, ctx.seg_len, ctx.slot, y, single_tokens=ctx.max_seg_len == 1)
         # a delta for the residual stream: the next norm adds slices, so it may come sliced

@@ -93,12 +93,11 @@ def hand_context(segments: Sequence[Tuple[int, int]], page_size: int, n_pages: i
     class Storage:
         pass
     st = Storage()
-    st.kv, st.fixed, st.v_transposed = {}, {}, {}
+    st.paged, st.fixed = {}, {}
     for site, (hk, d) in (kv_sites or {}).items():
         v_shape = (n_pages, hk, d, page_size) if v_transposed else (n_pages, hk, page_size, d)
-        st.kv[site] = (torch.zeros(n_pages, hk, page_size, d, dtype=dtype, device=device),
-                       torch.zeros(v_shape, dtype=dtype, device=device))
-        st.v_transposed[site] = v_transposed
+        st.paged[site] = dict(k=torch.zeros(n_pages, hk, page_size, d, dtype=dtype, device=device),
+                              v=torch.zeros(v_shape, dtype=dtype, device=device))
     for site, shape in (fixed_sites or {}).items():
         st.fixed[site] = torch.zeros((n_slots,) + tuple(shape), dtype=torch.float32, device=device)
     R = len(segments)
@@ -127,11 +126,10 @@ def hand_context(segments: Sequence[Tuple[int, int]], page_size: int, n_pages: i
         seg_len=i32(length), slot=i32(slots if slots is not None else list(range(R))),
         block_tables={0: i32(tab)}, page_size=page_size, dtype=dtype, workspace=Workspace(device),
         storage=st, group_of_site={s: 0 for s in (kv_sites or {})},
-        max_seg_len=max(length), max_context=max(p0 + n for p0, n in segments))
+        max_seg_len=max(length), max_context=max(p0 + n for p0, n in segments), host_seg_len=list(length))
     dec = [r for r, n in enumerate(length) if n == 1]
     pre = [r for r, n in enumerate(length) if n > 1]
     lists = i32(dec + pre)
-    ctx.decode_rows, ctx.n_decode_rows = lists[:len(dec)], len(dec)
-    ctx.prefill_rows, ctx.n_prefill_rows = lists[len(dec):], len(pre)
-    ctx.n_prefill_tiles = sum((length[r] + 63) // 64 for r in pre)
+    ctx.single_rows, ctx.n_single_rows = lists[:len(dec)], len(dec)
+    ctx.portion_rows, ctx.n_portion_rows = lists[len(dec):], len(pre)
     return ctx

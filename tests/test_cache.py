@@ -4,7 +4,8 @@ import random
 
 import pytest
 
-from imparo_amd.cache import (PagePool, CacheManager, PagedSpec, FixedSpec, OutOfPages, CacheError)
+from imparo_amd.cache import (PagePool, CacheManager, PagedSpec, PagedArray, PAGE, FixedSpec, OutOfPages, CacheError,
+                              kv_spec)
 
 
 def test_lowest_free_page_always():
@@ -58,7 +59,7 @@ def test_scrambled_placement_is_a_permutation():
     assert p.alloc() == got[5]
 
 
-SITES = [FixedSpec((2, 8)), PagedSpec(2, 16), FixedSpec((2, 8)), PagedSpec(2, 16), PagedSpec(2, 16, window=10), None]
+SITES = [FixedSpec((2, 8)), kv_spec(2, 16), FixedSpec((2, 8)), kv_spec(2, 16), kv_spec(2, 16, window=10), None]
 
 
 def test_groups_follow_the_specs():
@@ -116,7 +117,7 @@ def test_slots_run_out():
 
 
 def test_a_window_gives_pages_back_as_it_passes_them():
-    m = CacheManager([PagedSpec(1, 16, window=10), PagedSpec(1, 16)], page_size=4, n_pages=64, n_slots=1)
+    m = CacheManager([kv_spec(1, 16, window=10), kv_spec(1, 16)], page_size=4, n_pages=64, n_slots=1)
     m.admit("a")
     for n in range(1, 41):
         m.reserve("a", n)
@@ -184,14 +185,14 @@ def test_random_orders_never_lose_or_share_a_page(seed):
 def test_pack_lays_out_a_step():
     """The native packer: tokens | positions | row_of_token | seg_start | seg_len | slot | row lists |
     want | tables, positions counted from each request's length before the step."""
-    m = CacheManager([PagedSpec(1, 16), FixedSpec((4,)), PagedSpec(1, 16, window=6)], page_size=4, n_pages=16, n_slots=4)
+    m = CacheManager([kv_spec(1, 16), FixedSpec((4,)), kv_spec(1, 16, window=6)], page_size=4, n_pages=16, n_slots=4)
     m.admit("a"), m.admit("b"), m.admit("c")
     m.reserve("a", 9), m.commit("a", 9)
     m.reserve("a", 10), m.reserve("b", 3), m.reserve("c", 1)
     arr, lay = m.pack(["a", "b", "c"], [[7], [1, 2, 3], [4]], [[0], [2, 0], []])
     T, R, W, G, P = (lay[k] for k in "TRWGP")
     assert (T, R, W, G) == (5, 3, 3, 2) and P == 3 and lay["n_single"] == 2 and lay["n_multi"] == 1
-    assert lay["max_seg_len"] == 3 and lay["max_context"] == 10 and lay["n_prefill_tiles"] == 1
+    assert lay["max_seg_len"] == 3 and lay["max_context"] == 10
     a = arr.tolist()
     assert a[0:5] == [7, 1, 2, 3, 4]                      # tokens
     assert a[5:10] == [9, 0, 1, 2, 0]                     # positions
@@ -218,7 +219,7 @@ def test_a_whole_step_is_booked_in_one_call():
     """begin_step admits, reserves and checks for the whole batch; end_step commits it. The
     result is what admit/reserve/commit give one request at a time."""
     from imparo_amd.cache import native as N
-    specs = [PagedSpec(1, 16), FixedSpec((4,)), PagedSpec(1, 16, window=6)]
+    specs = [kv_spec(1, 16), FixedSpec((4,)), kv_spec(1, 16, window=6)]
     m = CacheManager(specs, page_size=4, n_pages=16, n_slots=3)
     one = CacheManager(specs, page_size=4, n_pages=16, n_slots=3)
     steps = [(["a", "b"], [[1] * 9, [2] * 3]), (["b", "a", "c"], [[5], [6, 7], [8] * 5]), (["c", "a"], [[1], [2]])]
@@ -257,7 +258,7 @@ def test_a_whole_step_is_booked_in_one_call():
 
 
 def test_a_step_that_does_not_fit_changes_nothing():
-    m = CacheManager([PagedSpec(1, 16), PagedSpec(1, 16, window=6)], page_size=4, n_pages=6, n_slots=2)
+    m = CacheManager([kv_spec(1, 16), kv_spec(1, 16, window=6)], page_size=4, n_pages=6, n_slots=2)
     b = m.batch(["a"], [[1] * 10], [[9]])
     assert m.begin_step(b, 10, 64) == (0, -1)
     m.end_step(b)
@@ -277,3 +278,54 @@ def test_a_step_that_does_not_fit_changes_nothing():
     m.abort_step(b)
     assert snapshot(m, "abc") == before
     m.check()
+
+
+# ---- what a paged site keeps is the mixer's to declare; pools are sized per group
+def test_a_paged_spec_names_its_arrays_and_their_page_layout():
+    spec = kv_spec(2, 16, window=10, v_transposed=True)
+    assert [a.name for a in spec.arrays] == ["k", "v"]
+    assert spec.arrays[0].shape(5, 8) == (5, 2, 8, 16) and spec.arrays[1].shape(5, 8) == (5, 2, 16, 8)
+    assert spec.bytes_per_position(2) == 2 * 2 * 16 * 2
+    # a latent of 24 values a position in float32 beside a narrow key: no K/V pair of one shape
+    other = PagedSpec((PagedArray("latent", (PAGE, 24), float32=True), PagedArray("key", (1, PAGE, 8))))
+    assert other.bytes_per_position(2) == 24 * 4 + 8 * 2
+    assert other != spec and other == PagedSpec(other.arrays)
+    with pytest.raises(ValueError, match="twice"):
+        PagedSpec((PagedArray("a", (PAGE, 4)), PagedArray("a", (PAGE, 2))))
+    with pytest.raises(ValueError, match="positions"):
+        PagedSpec((PagedArray("a", (4, 4)),))
+
+
+def test_every_group_has_a_pool_of_its_own_size():
+    specs = [kv_spec(1, 16), FixedSpec((4,)), kv_spec(1, 16, window=6), kv_spec(1, 16)]
+    groups = CacheManager.groups_of(specs)
+    assert [(s.window, sites) for s, sites in groups] == [(None, [0, 3]), (6, [2])]
+    m = CacheManager(specs, page_size=4, n_pages=[10, 3], n_slots=2)
+    assert [g.pool.n_pages for g in m.groups] == [10, 3]
+    m.admit("a")
+    m.reserve("a", 11)                 # 3 pages in both groups
+    m.commit("a", 11)                  # the window's group gives one back
+    assert m.free_pages() == [7, 1]
+    with pytest.raises(OutOfPages):    # 5 more pages: the small pool cannot, and the large one keeps its pages
+        m.reserve("a", 31)
+    assert m.free_pages() == [7, 1]
+    m.check()
+    with pytest.raises(ValueError, match="pool sizes"):
+        CacheManager(specs, page_size=4, n_pages=[10], n_slots=2)
+
+
+def test_pool_sizes_from_a_budget_in_bytes():
+    from imparo_amd.engine import Engine
+    import torch
+    specs = [FixedSpec((2, 64)), kv_spec(8, 64), None, kv_spec(8, 64), kv_spec(8, 64, window=128)]
+    # a page of 64 positions: 2 * 8 * 64 values per position and site, 2 bytes each, three sites in two groups
+    per_page = 64 * (2 * 8 * 64 * 2) * 3
+    assert Engine.pool_sizes(specs, 64, torch.bfloat16, None, 10 * per_page + 5, None) == [10, 10]
+    assert Engine.pool_sizes(specs, 64, torch.float32, None, 10 * per_page, None) == [5, 5]
+    assert Engine.pool_sizes(specs, 64, torch.bfloat16, 1000, None, None) == [16, 16]
+    assert Engine.pool_sizes(specs, 64, torch.bfloat16, None, None, 7) == [7, 7]
+    assert Engine.pool_sizes(specs, 64, torch.bfloat16, None, None, [7, 3]) == [7, 3]
+    with pytest.raises(ValueError, match="one page"):
+        Engine.pool_sizes(specs, 64, torch.bfloat16, None, per_page - 1, None)
+    with pytest.raises(ValueError, match="num_pages"):
+        Engine.pool_sizes(specs, 64, torch.bfloat16, None, None, [7])

@@ -295,7 +295,7 @@ def test_tokens_fed_from_the_device(zoo, dtype):
             entries = [StepEntry(0, toks[0], [0]), StepEntry(1, toks[1], [0])]
             if s == 4:
                 entries.insert(1, StepEntry(2, prompts[2], [19]))
-            out.append(eng.step(entries))
+            out.append(eng.step(entries).clone())     # the logits tensor is the engine's: the next step writes there
         runs.append(torch.cat(out).cpu())
         if from_device:
             with pytest.raises(StepError, match="device token"):
@@ -308,6 +308,30 @@ def test_tokens_fed_from_the_device(zoo, dtype):
     assert torch.equal(runs[0], runs[1])
     ref = zoo[1]["B"](prompts[0] + nxt[0])
     check_logits(runs[0][0:1], ref[12:13], dtype, "first decoded row")
+
+
+def test_pool_sizing_and_the_bound_on_a_steps_tokens(zoo):
+    from imparo_amd.engine import Engine, StepEntry, StepError
+    vocab = vocab_of(zoo, "C")
+    # model C has two cache groups (all keys; a window): one number for both, or one each
+    eng = Engine(zoo[0]["C"], dtype="bfloat16", page_size=16, num_pages=[9, 4], max_requests=2, max_step_tokens=40)
+    assert [g.pool.n_pages for g in eng.cache.groups] == [9, 4]
+    toks = prompt_tokens(vocab, 60, 3)
+    with pytest.raises(StepError, match="max_step_tokens"):
+        eng.step([StepEntry("a", toks[:41], [])])
+    with pytest.raises(StepError, match="max_step_tokens"):
+        eng.step([StepEntry("a", toks[:30], []), StepEntry("b", toks[:11], [])])
+    assert not eng.is_live("a") and eng.free_pages() == [9, 4]
+    got = torch.cat([eng.step([StepEntry("a", toks[:40], list(range(40)))]).cpu(),
+                     eng.step([StepEntry("a", toks[40:], list(range(20)))]).cpu()])
+    check_logits(got, zoo[1]["C"](toks), "bfloat16", "two cache groups with pools of their own")
+    # a budget in bytes: pages of 16 positions x (5 kv heads x 16 x 2 arrays x 2 bytes) x 3 attention sites
+    per_page = 16 * (5 * 16 * 2 * 2) * 3
+    eng = Engine(zoo[0]["C"], dtype="bfloat16", page_size=16, kv_budget_bytes=12 * per_page + 100, max_requests=2)
+    assert [g.pool.n_pages for g in eng.cache.groups] == [12, 12]
+    assert sum(t.numel() * t.element_size() for a in eng.storage.paged.values() for t in a.values()) == 12 * per_page
+    with pytest.raises(ValueError, match="one of"):
+        Engine(zoo[0]["C"], max_tokens=64, num_pages=3)
 
 
 def test_refused_batches(zoo, engines):

@@ -160,33 +160,28 @@ def test_gemm_with_many_weight_rows(m, k):
 def test_gemm_with_large_tiles(m, n, k, tile):
     """Many rows: K a multiple of 128 goes to the kernel that loads straight into LDS, with a tile
     of 256 or 128 rows by 256, 192 or 128 weight rows, whichever its plan finds fastest (`tile`
-    other than 0 names one, through the library's switch for measurements, so that each is met);
+    other than 0 names one, an argument of the entry point for tests and measurements, so that each is met);
     another K to the tile kernels with register staging. Edges in both directions, an odd number
     of column pairs, a bias, both epilogues and output types."""
-    from imparo_amd.kernels import library
-    library().imparo_gemm_force_kernel(tile)
-    try:
-        _large_tile_case(m, n, k)
-    finally:
-        library().imparo_gemm_force_kernel(0)
+    _large_tile_case(m, n, k, tile)
 
 
-def _large_tile_case(m, n, k):
+def _large_tile_case(m, n, k, variant=0):
     x, w, b = rnd(m, k, seed=1, scale=0.5).to(torch.bfloat16), rnd(n, k, seed=2, scale=0.3).to(torch.bfloat16), rnd(n, seed=3)
     y = x.float() @ w.float().t() + b                       # float32 on the CPU: products exact, sums to 1e-6 sqrt(k)
     bound = 1e-6 * math.sqrt(k) * float(y.abs().max())
     out = torch.full((m, n), float("nan"), device=DEV)
-    ops().gemm(x.to(DEV), w.to(DEV), out, bias=b.to(DEV))
+    ops().gemm(x.to(DEV), w.to(DEV), out, bias=b.to(DEV), variant=variant)
     assert (out.cpu() - y).abs().max() <= 4 * bound
     outb = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
-    ops().gemm(x.to(DEV), w.to(DEV), outb, bias=b.to(DEV))
+    ops().gemm(x.to(DEV), w.to(DEV), outb, bias=b.to(DEV), variant=variant)
     assert torch.equal(outb.cpu(), out.cpu().to(torch.bfloat16))
     ref = torch.nn.functional.silu(y[:, 0::2].double()) * y[:, 1::2].double()
     out = torch.full((m, n // 2), float("nan"), device=DEV)
-    ops().gemm(x.to(DEV), w.to(DEV), out, bias=b.to(DEV), swiglu=True)
+    ops().gemm(x.to(DEV), w.to(DEV), out, bias=b.to(DEV), swiglu=True, variant=variant)
     torch.testing.assert_close(out.cpu().double(), ref, rtol=1e-5, atol=8 * bound)
     outb = torch.full((m, n // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
-    ops().gemm(x.to(DEV), w.to(DEV), outb, bias=b.to(DEV), swiglu=True)
+    ops().gemm(x.to(DEV), w.to(DEV), outb, bias=b.to(DEV), swiglu=True, variant=variant)
     assert torch.equal(outb.cpu(), out.cpu().to(torch.bfloat16))
 
 
@@ -244,21 +239,24 @@ def test_rms_norm(width):
     torch.testing.assert_close(out.cpu(), P.rms_norm((x + d)[[5, 0, 5]], w, 1e-5), rtol=2e-6, atol=2e-6)
 
 
-def test_embed_gather_and_silu_mul():
+def test_embed_gather():
     table = rnd(37, 24, seed=4)
     ids = torch.tensor([36, 0, 5, 5], dtype=torch.int32, device=DEV)
     for t in (table, table.to(torch.bfloat16)):
         out = torch.empty(4, 24, device=DEV)
         ops().embed_gather(t.to(DEV), ids, out)
         assert torch.equal(out.cpu(), t.float()[[36, 0, 5, 5]])
-    gu = rnd(5, 2 * 88, seed=5, scale=3.0)
-    out = torch.empty(5, 88, device=DEV)
-    ops().silu_mul(gu.to(DEV), out)
-    torch.testing.assert_close(out.cpu(), P.silu(gu[:, :88]) * gu[:, 88:], rtol=2e-6, atol=1e-6)
-    out = torch.empty(5, 88, dtype=torch.bfloat16, device=DEV)
-    ops().silu_mul(gu.to(DEV), out)
-    assert torch.equal(out.cpu(), (P.silu(gu[:, :88]) * gu[:, 88:]).to(torch.bfloat16)) or \
-        (out.cpu().float() - P.silu(gu[:, :88]) * gu[:, 88:]).abs().max() < 0.05
+
+
+def test_fill_sites_sets_one_slot_of_every_site():
+    sites = [torch.full((5, 2, 8), 7.0, device=DEV), torch.full((5, 3), 7.0, device=DEV),
+             torch.full((5, 4000), 7.0, device=DEV)]
+    base = torch.tensor([t.data_ptr() for t in sites], dtype=torch.int64, device=DEV)
+    per_slot = torch.tensor([t[0].numel() for t in sites], dtype=torch.int64, device=DEV)
+    value = torch.tensor([0.0, -1.5, 2.0], device=DEV)
+    ops().fill_sites(base, per_slot, value, 3)
+    for t, v in zip(sites, (0.0, -1.5, 2.0)):
+        assert bool((t[3] == v).all()) and bool((t[[0, 1, 2, 4]] == 7.0).all())
 
 
 # ---------------------------------------------------------------- norm + rotation + cache write
@@ -405,16 +403,16 @@ def _attention_case(H, Hk, D, page_size, window, dtype, sharpen=None, seed=0, ke
                         v_transposed=vt)
     else:
         n_splits = (ctx.max_context + 255) // 256
-        part_o = torch.full((ctx.n_decode_rows * H * n_splits * D,), float("nan"), device=DEV)
-        part_ml = torch.full((ctx.n_decode_rows * H * n_splits * 2,), float("nan"), device=DEV)
-        ops().attention_decode(q_all, k_cache, v_cache, out, part_o, part_ml, ctx.decode_rows, ctx.n_decode_rows,
+        part_o = torch.full((ctx.n_single_rows * H * n_splits * D,), float("nan"), device=DEV)
+        part_ml = torch.full((ctx.n_single_rows * H * n_splits * 2,), float("nan"), device=DEV)
+        ops().attention_decode(q_all, k_cache, v_cache, out, part_o, part_ml, ctx.single_rows, ctx.n_single_rows,
                                ctx.seg_start, ctx.positions, table, scale, window, ctx.max_context)
         parts_o = parts_ml = None
         if prefill_splits > 1:                 # NaN where no part writes: a part without keys must not be read
             parts_o = torch.full((ctx.n_tokens, H, prefill_splits, D), float("nan"), device=DEV)
             parts_ml = torch.full((ctx.n_tokens, H, prefill_splits, 2), float("nan"), device=DEV)
-        ops().attention_prefill(q_all, k_cache, v_cache, out, ctx.prefill_rows, ctx.n_prefill_rows,
-                                ctx.n_prefill_tiles, ctx.seg_start, ctx.seg_len, ctx.positions, table, scale, window,
+        ops().attention_prefill(q_all, k_cache, v_cache, out, ctx.portion_rows, ctx.n_portion_rows,
+                                sum((n + 63) // 64 for n in ctx.host_seg_len if n > 1), ctx.seg_start, ctx.seg_len, ctx.positions, table, scale, window,
                                 parts_o, parts_ml, prefill_splits)
     return out.cpu().float().reshape(-1, H, D), torch.cat(refs)
 

@@ -58,6 +58,10 @@ def test_attention_part(dtype, H, Hk, D, window, rot):
         v = (1 + 0.1 * rnd(*decl.shape, seed=i)) if init == "norm" else rnd(*decl.shape, seed=i, scale=0.15)
         t[name] = v.to(torch.bfloat16)
     part = cls(spec, t, DEV, dtype)
+    # the part says how its cache is laid out (V transposed in a page where its matrix-core kernels apply)
+    from imparo_amd.cache import kv_spec
+    vt = dtype == torch.bfloat16
+    assert part.cache_spec(16) == kv_spec(Hk, D, window, v_transposed=vt) and part.v_transposed == vt
     f = {k: v.float() for k, v in t.items()}
     lens = [23, 14]
     hs = [rnd(n, E, seed=50 + r).to(torch.bfloat16).float() for r, n in enumerate(lens)]
@@ -73,10 +77,10 @@ def test_attention_part(dtype, H, Hk, D, window, rot):
         o = P.attend(q, k, v, pos, 1.0 / math.sqrt(D), window)
         refs.append(P.linear(o.reshape(T, H * D), f["a.o_proj.weight"]))
     tables = [[5, 2], [0]]
-    ctx1 = hand_context([(0, 20), (0, 13)], 16, 8, dtype, DEV, kv_sites={3: (Hk, D)}, tables=tables)
+    ctx1 = hand_context([(0, 20), (0, 13)], 16, 8, dtype, DEV, kv_sites={3: (Hk, D)}, tables=tables, v_transposed=vt)
     x1 = torch.cat([hs[0][:20], hs[1][:13]]).to(part.in_dtype).to(DEV)
     out1 = part.forward(ctx1, 3, True, x1).cpu().clone()
-    ctx2 = hand_context([(20, 3), (13, 1)], 16, 8, dtype, DEV, kv_sites={3: (Hk, D)}, tables=tables)
+    ctx2 = hand_context([(20, 3), (13, 1)], 16, 8, dtype, DEV, kv_sites={3: (Hk, D)}, tables=tables, v_transposed=vt)
     ctx2.storage = ctx1.storage
     x2 = torch.cat([hs[0][20:], hs[1][13:]]).to(part.in_dtype).to(DEV)
     out2 = part.forward(ctx2, 3, True, x2).cpu()
@@ -84,8 +88,6 @@ def test_attention_part(dtype, H, Hk, D, window, rot):
     got1 = torch.cat([out1[20:], out2[3:]])
     torch.testing.assert_close(got0, refs[0], **tol(dtype))
     torch.testing.assert_close(got1, refs[1], **tol(dtype))
-    from imparo_amd.cache import PagedSpec
-    assert part.cache_spec() == PagedSpec(Hk, D, window)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -101,7 +103,7 @@ def test_short_conv_part(dtype, taps, bias):
     for i, (name, (decl, init)) in enumerate(sorted(cls.declare(spec).items())):
         t[name] = rnd(*decl.shape, seed=i, scale=0.3 if init == "conv" else 0.15).to(torch.bfloat16)
     part = cls(spec, t, DEV, dtype)
-    assert part.cache_spec() == FixedSpec((taps - 1, E))
+    assert part.cache_spec(16) == FixedSpec((taps - 1, E))
     f = {k: v.float() for k, v in t.items()}
     b = (lambda n: f[f"c.{n}.bias"]) if bias else (lambda n: None)
     h = rnd(17, E, seed=9).to(torch.bfloat16).float()

@@ -45,10 +45,12 @@ def test_embedding_norm_and_gate():
         out = torch.empty(7, width, device=DEV)
         ops().rms_norm(x.to(DEV), w.to(DEV), 1e-5, out)
         np.testing.assert_allclose(out.cpu().numpy(), R.rms_norm(x, w, 1e-5), rtol=2e-6, atol=2e-6)
-    gu = rnd(5, 2 * 88, seed=5, scale=3.0)
+    # the gate: the product's own epilogue (rows of the weight alternate gate and up)
+    x, w = rnd(5, 40, seed=5), rnd(2 * 88, 40, seed=6)
     out = torch.empty(5, 88, device=DEV)
-    ops().silu_mul(gu.to(DEV), out)
-    np.testing.assert_allclose(out.cpu().numpy(), R.swiglu(gu[:, :88], gu[:, 88:]), rtol=2e-6, atol=1e-6)
+    ops().gemm(x.to(DEV), w.to(DEV), out, swiglu=True)
+    gu = R.gemm(x, w)
+    np.testing.assert_allclose(out.cpu().numpy(), R.swiglu(gu[:, 0::2], gu[:, 1::2]), rtol=2e-6, atol=1e-6)
 
 
 @pytest.mark.parametrize("H,Hk,D,rot", [(3, 1, 48, 48), (6, 3, 64, 32), (5, 1, 128, 0)])

@@ -21,7 +21,7 @@ pytestmark = pytest.mark.gpu
 
 class LeakyMean:
     """The mixer interface: declare(spec), __init__(spec, tensors, device,
-    engine_dtype), in_dtype, cache_spec(), forward(ctx, site, owns_cache, h)."""
+    engine_dtype), in_dtype, cache_spec(page_size), forward(ctx, site, owns_cache, h)."""
     role = "mixer"
 
     @staticmethod
@@ -41,7 +41,7 @@ class LeakyMean:
     def in_dtype(self):
         return self.w.in_dtype
 
-    def cache_spec(self):
+    def cache_spec(self, page_size):
         from imparo_amd.cache import FixedSpec
         return FixedSpec((self.width,))
 
@@ -86,8 +86,8 @@ def toy(tmp_path_factory):
         plan = lfm2.build_plan(cfg)
         layers = list(plan.layers)
         for i in cfg.toy_layers:
-            layers[i] = dataclasses.replace(layers[i], mixer=PartSpec(
-                "test_leaky_mean", f"model.layers.{i}.toy", dict(width=cfg.hidden_size, decay=cfg.toy_decay)))
+            toy = PartSpec("test_leaky_mean", f"model.layers.{i}.toy", dict(width=cfg.hidden_size, decay=cfg.toy_decay))
+            layers[i] = layers[i].with_part("mixer", toy)
         return dataclasses.replace(plan, architecture="TestLeakyForCausalLM", layers=layers)
     register_architecture("TestLeakyForCausalLM", read, build)
     from tiny_configs import TINY_A

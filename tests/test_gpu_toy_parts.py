@@ -110,13 +110,13 @@ def toy(tmp_path_factory):
         layers = []
         for i, layer in enumerate(plan.layers):
             if i % 2 == 1:                       # odd layers route; the others keep their dense feed-forward
-                layer = dataclasses.replace(layer, ffn=PartSpec(
+                layer = layer.with_part("ffn", PartSpec(
                     "test_routed_toy", f"model.layers.{i}.moe",
                     dict(width=cfg.hidden_size, hidden=EXPERT_HIDDEN, experts=N_EXPERTS)))
             if layer.mixer.kind == "attention":
                 params = dict(layer.mixer.params)
                 params["position"] = PartSpec("test_partial_scaled_rope", "", dict(rotary_dim=ROTARY_DIM, base=ROTARY_BASE))
-                layer = dataclasses.replace(layer, mixer=PartSpec(layer.mixer.kind, layer.mixer.prefix, params))
+                layer = layer.with_part("mixer", PartSpec(layer.mixer.kind, layer.mixer.prefix, params))
             layers.append(layer)
         return dataclasses.replace(plan, architecture="TestRoutedForCausalLM", layers=layers)
     register_architecture("TestRoutedForCausalLM", read, build)

@@ -7,7 +7,7 @@ from typing import List, Sequence
 import numpy as np
 import pytest
 
-from imparo_amd.cache import CacheManager, PagedSpec, FixedSpec, OutOfPages
+from imparo_amd.cache import CacheManager, kv_spec, FixedSpec, OutOfPages
 from imparo_amd.engine.engine import DeviceToken
 from imparo_amd.engine.scheduler import Scheduler, Request
 from imparo_amd.sampling import SamplingParams, uniform_for
@@ -28,7 +28,7 @@ class FakeEngine:
 
     def __init__(self, n_pages, page_size=4, n_slots=4):
         self.page_size = page_size
-        self.cache = CacheManager([PagedSpec(1, 16), FixedSpec((2, 4))], page_size, n_pages, n_slots)
+        self.cache = CacheManager([kv_spec(1, 16), FixedSpec((2, 4))], page_size, n_pages, n_slots)
         self.history = {}
         self.steps = []          # [(request, n_tokens, wants)] per step
 
