@@ -10,7 +10,8 @@ GPU runs that next step).
 Default: batch 8, every request's context ending at 4096 tokens, random
 bfloat16 weights (seed 2), synthetic token ids uniform over the vocabulary.
 The JSON line also carries a 2,048-token prefill, the decode step's HBM
-roofline, and decode at batch 1 and 64.
+roofline, and decode at batch 1 and 64. Every figure is the median of three
+measurements taken in turn.
 """
 import argparse
 import json
@@ -91,10 +92,11 @@ def decode_run(engine, sampler, batch, context, steps, warmup, vocab, seed):
 
 
 def prefill_run(engine, tokens, vocab, reps, seed):
+    """Seconds of each of `reps` whole prompts of `tokens` tokens (one step each, fresh tokens each time)."""
     import torch
     from imparo_amd.engine import StepEntry
     g = torch.Generator().manual_seed(seed)
-    best = None
+    times = []
     for r in range(reps + 1):
         prompt = torch.randint(0, vocab, (tokens,), generator=g).tolist()
         torch.cuda.synchronize()
@@ -104,8 +106,19 @@ def prefill_run(engine, tokens, vocab, reps, seed):
         dt = time.perf_counter() - t0
         engine.release("p")
         if r > 0:                                      # the first run sizes the workspace
-            best = dt if best is None else min(best, dt)
-    return best
+            times.append(dt)
+    return times
+
+
+def median(xs):
+    xs = sorted(xs)
+    n = len(xs)
+    return xs[n // 2] if n % 2 else 0.5 * (xs[n // 2 - 1] + xs[n // 2])
+
+
+def percentile(xs, q):
+    xs = sorted(xs)
+    return xs[min(len(xs) - 1, int(q * len(xs)))]
 
 
 def shape(hidden, heads, block_ff_dim):
@@ -113,6 +126,66 @@ def shape(hidden, heads, block_ff_dim):
     cfg = dict(LFM2_1_2B)
     cfg.update(hidden_size=hidden, num_attention_heads=heads, block_ff_dim=block_ff_dim)
     return cfg
+
+
+class StepClock:
+    """Stands between the scheduler and the engine and notes, for every step, what it fed and a GPU
+    event at its start: the time from one step's event to the next is that step's time on the GPU
+    (the host runs a step ahead, so nothing waits for the notes)."""
+
+    def __init__(self, engine, weight_bytes, head_bytes, kv_bytes_per_token, flops_per_token):
+        self._engine = engine
+        self._held = {}                  # request -> tokens in the cache
+        self.notes = []                  # (event, decode rows, prompt tokens, bytes to read, flops)
+        self._sizes = (weight_bytes, head_bytes, kv_bytes_per_token, flops_per_token)
+
+    def __getattr__(self, name):
+        return getattr(self._engine, name)
+
+    def step(self, entries):
+        import torch
+        weight_bytes, head_bytes, kv_bytes, flops_per_token = self._sizes
+        rows = sum(1 for e in entries if len(e.tokens) == 1)
+        fed = sum(len(e.tokens) for e in entries)
+        for e in entries:
+            self._held[e.request] = self._held.get(e.request, 0) + len(e.tokens)
+        # every weight once (the head only if a row asks for logits), the cache of the requests in the step
+        to_read = (weight_bytes + (head_bytes if any(e.want for e in entries) else 0)
+                   + kv_bytes * sum(self._held[e.request] for e in entries))
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self.notes.append((ev, rows, fed - rows, to_read, flops_per_token * fed))
+        return self._engine.step(entries)
+
+    def release(self, request_id):
+        self._held.pop(request_id, None)
+        return self._engine.release(request_id)
+
+    def by_kind(self, hbm_peak_gbs, flops_peak):
+        """Step times by what a step fed: single tokens only, or portions of prompts as well."""
+        import torch
+        end = torch.cuda.Event(enable_timing=True)
+        end.record()
+        torch.cuda.synchronize()
+        events = [n[0] for n in self.notes] + [end]
+        kinds = {"decode_only": [], "mixed": []}
+        for i, (_, rows, prompt_tokens, to_read, flops) in enumerate(self.notes):
+            ms = events[i].elapsed_time(events[i + 1])
+            kinds["mixed" if prompt_tokens else "decode_only"].append((ms, rows, prompt_tokens, to_read, flops))
+        out = {}
+        for kind, steps in kinds.items():
+            if not steps:
+                continue
+            times = [t[0] for t in steps]
+            out[kind] = {
+                "steps": len(steps), "p50_ms": round(percentile(times, 0.5), 3), "p90_ms": round(percentile(times, 0.9), 3),
+                "max_ms": round(max(times), 3), "mean_rows": round(sum(t[1] for t in steps) / len(steps), 1),
+                "mean_prompt_tokens": round(sum(t[2] for t in steps) / len(steps), 1),
+                # what the step had to read / its time / the HBM peak; what it had to compute / its time / the MFMA peak
+                "hbm_frac_p50": round(percentile([t[3] / (t[0] * 1e-3) / 1e9 / hbm_peak_gbs for t in steps], 0.5), 4),
+                "mfma_frac_p50": round(percentile([t[4] / (t[0] * 1e-3) / flops_peak for t in steps], 0.5), 4),
+            }
+        return out
 
 
 def serving_workload(dtype):
@@ -125,9 +198,13 @@ def serving_workload(dtype):
     from imparo_amd.engine.scheduler import Scheduler
     from imparo_amd.sampling import Sampler, SamplingParams
     cfg = shape(1536, 24, 10240)
+    nums = model_numbers(cfg)
     tmp = tempfile.mkdtemp(prefix="imparo_bench_")
     write_random_model(cfg, 3, tmp)
-    engine = Engine(tmp, dtype=dtype, max_tokens=32 * (3072 + 512 + 64), page_size=64, max_requests=32)
+    elem = 2 if dtype == "bfloat16" else 4
+    engine = StepClock(Engine(tmp, dtype=dtype, max_tokens=32 * (3072 + 512 + 64), page_size=64, max_requests=32),
+                       nums["layer_params"] * elem, nums["head_params"] * elem, nums["kv_bytes_per_token"] * elem // 2,
+                       2.0 * nums["layer_params"])
     sampler = Sampler(engine.device)
     rng = np.random.default_rng(3)
     jobs = [(i, rng.integers(0, cfg["vocab_size"], size=int(rng.integers(64, 3073))).tolist(), int(rng.integers(32, 513)))
@@ -150,14 +227,17 @@ def serving_workload(dtype):
     n_prompt = sum(len(r.prompt) for r in done.values())
     n_out = sum(len(r.generated) for r in done.values())
     assert len(done) == 32 and all(r.finish_reason == "length" for r in done.values())
+    c = nums["cfg"]
     print(json.dumps({
         "metric": "continuous batching, LFM2-700M shape: generated tok/s over the whole run", "value": round(n_out / dt, 1),
         "unit": "tok/s", "n_gpus": 1, "seconds": round(dt, 3), "steps": steps, "prompt_tokens": n_prompt,
         "generated_tokens": n_out, "all_tokens_per_s": round((n_prompt + n_out) / dt, 1),
         "preemptions": sum(r.preemptions for r in done.values()), "dtype": "bf16" if dtype == "bfloat16" else "fp32",
         "data": "synthetic token ids, random weights (seed 3)",
+        "step_times": engine.by_kind(HBM_PEAK_GBS, MFMA_PEAK["bf16" if dtype == "bfloat16" else "fp32"]),
         "config": {"model": "LFM2-700M shape", "requests": 32, "waves": 4, "portion": 512, "max_batch_tokens": 2048,
-                   "hidden_size": 1536, "heads": 24, "kv_heads": 8, "ff_dim": 6912, "layers": 16}}), flush=True)
+                   "hidden_size": c.hidden_size, "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads,
+                   "ff_dim": c.ff_dim, "layers": c.num_hidden_layers}}), flush=True)
     return 0
 
 
@@ -262,18 +342,39 @@ def main() -> int:
     sampler = Sampler(engine.device)
     elem = 2 if args.dtype == "bfloat16" else 4
     if args.prefill_only:
-        pt = prefill_run(engine, 2048, c.vocab_size, 5, 3)
-        print(json.dumps({"prefill_ms": round(pt * 1e3, 3), "tokens": 2048}), flush=True)
+        pts = prefill_run(engine, 2048, c.vocab_size, 5, 3)
+        print(json.dumps({"prefill_ms": round(median(pts) * 1e3, 3), "tokens": 2048,
+                          "all_ms": [round(t * 1e3, 3) for t in pts]}), flush=True)
         return 0
-    print("[bench] decode ...", file=sys.stderr, flush=True)
-    dt = decode_run(engine, sampler, args.batch, args.context, args.steps, args.warmup, c.vocab_size, 2)
+
+    def step_bytes(batch, steps):
+        """Bytes one decode step has to read: every weight once, the cache of the live requests."""
+        mean_ctx = args.context - steps / 2
+        return ((nums["layer_params"] + nums["head_params"]) * elem
+                + batch * (mean_ctx * nums["kv_bytes_per_token"] * elem / 2 + nums["conv_state_bytes"]))
+
+    # Every figure is the median of PASSES measurements taken in turn (batch 8, batch 1, batch 64,
+    # prefill, and again), so that a slow moment of the machine does not fall on one of them alone.
+    # A decode measurement is W warmup steps and exactly K timed steps, each time on freshly filled contexts.
+    PASSES = 3
+    points_steps = max(8, args.steps // 2)
+    widths = [args.batch] + ([] if args.no_points else [b for b in (1, 64) if b != args.batch])
+    seconds = {b: [] for b in widths}
+    prefills = []
+    T = 2048
+    for p in range(PASSES):
+        for b in widths:
+            k = args.steps if b == args.batch else points_steps
+            w = args.warmup if b == args.batch else 4
+            print(f"[bench] pass {p + 1} of {PASSES}: decode at batch {b} ...", file=sys.stderr, flush=True)
+            seconds[b].append(decode_run(engine, sampler, b, args.context, k, w, c.vocab_size, 2 + 100 * p + b))
+        if not args.no_points:
+            print(f"[bench] pass {p + 1} of {PASSES}: prefill of {T} tokens ...", file=sys.stderr, flush=True)
+            prefills += prefill_run(engine, T, c.vocab_size, 2, 3 + p)
+    dt = median(seconds[args.batch])
     ms = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
-    # bytes one decode step has to read: every weight once, the cache of the live requests
-    mean_ctx = args.context - args.steps / 2
-    step_bytes = ((nums["layer_params"] + nums["head_params"]) * elem
-                  + args.batch * (mean_ctx * nums["kv_bytes_per_token"] * elem / 2 + nums["conv_state_bytes"]))
-    achieved = step_bytes / (dt / args.steps) / 1e9
+    achieved = step_bytes(args.batch, args.steps) / (dt / args.steps) / 1e9
     line = {
         "metric": f"decode tok/s (LFM2-1.2B shape, batch {args.batch}, context {args.context})",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -287,23 +388,24 @@ def main() -> int:
             "head_dim": c.head_dim, "ff_dim": c.ff_dim, "vocab_size": c.vocab_size, "conv_L_cache": c.conv_L_cache,
             "tie_embedding": c.tie_embedding, "page_size": engine.page_size, "decode_tokens": args.steps + args.warmup,
         },
+        "passes": PASSES, "ms_per_step_of_each_pass": [round(t / args.steps * 1e3, 4) for t in seconds[args.batch]],
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }
     if not args.no_points:
-        print("[bench] prefill of 2,048 tokens ...", file=sys.stderr, flush=True)
-        T = 2048
-        pt = prefill_run(engine, T, c.vocab_size, 3, 3)
+        pt = median(prefills)
         flops = 2.0 * T * nums["layer_params"] + 2.0 * nums["head_params"] + nums["attn_flops_per_pair"] * T * (T + 1) / 2
         peak = MFMA_PEAK["bf16" if args.dtype == "bfloat16" else "fp32"]
         line["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
-                           "frac": round(flops / pt / peak, 4)}
+                           "frac": round(flops / pt / peak, 4), "runs": len(prefills),
+                           "min_ms": round(min(prefills) * 1e3, 3), "max_ms": round(max(prefills) * 1e3, 3)}
         points = {}
         for b in (1, 64):
-            print(f"[bench] decode at batch {b} ...", file=sys.stderr, flush=True)
-            k = max(8, args.steps // 2)
-            d = decode_run(engine, sampler, b, args.context, k, 4, c.vocab_size, 10 + b)
+            k = args.steps if b == args.batch else points_steps
+            d = median(seconds[b])
             points[f"decode_b{b}"] = round(b * k / d, 1)
+            points[f"decode_b{b}_ms_per_step"] = round(d / k * 1e3, 4)
+            points[f"decode_b{b}_frac"] = round(step_bytes(b, k) / (d / k) / 1e9 / HBM_PEAK_GBS, 4)
         line["points"] = points
     print(json.dumps(line), flush=True)
     return 0
