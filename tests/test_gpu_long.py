@@ -1,6 +1,6 @@
-"""Long contexts and a serving workload, where the plain implementation cannot
-follow: the bfloat16 matrix-core path is held to the engine's own float32 path
-(itself held to the plain implementation at short lengths elsewhere), and
+"""Long contexts and a serving workload. Up to some 4,000 tokens both dtypes
+are held to the plain implementation; where it cannot follow (16,500 tokens)
+the bfloat16 matrix-core path is held to the engine's own float32 path, and
 continuous batching under page pressure is held to each request run alone."""
 import random
 
@@ -28,6 +28,26 @@ def long_model(tmp_path_factory):
     d = str(tmp_path_factory.mktemp("long"))
     write_random_model(LONG, 5, d)
     return d
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_four_thousand_tokens_against_the_plain_implementation(long_model, dtype):
+    """4,230 tokens: two portions of 2,048 (32 query tiles over up to 64 key tiles, the window of
+    700 giving pages back on the way), a short portion, then single tokens through captured steps
+    whose keys are walked in 17 splits. Every row of logits is compared."""
+    from plain_lfm2 import PlainLfm2
+    from imparo_amd.engine import StepEntry
+    N = 4196
+    toks = prompt_tokens(512, N + 34, 77)
+    eng = make_engine(long_model, dtype, page_size=64, max_tokens=N + 128, max_requests=2)
+    out = []
+    for lo, hi in ((0, 2048), (2048, 4096), (4096, N)):
+        out.append(eng.step([StepEntry("l", toks[lo:hi], list(range(hi - lo)))]).cpu())
+    for i in range(N, N + 34):
+        out.append(eng.step([StepEntry("l", toks[i:i + 1], [0])]).cpu().clone())
+    ref = PlainLfm2(long_model).logits(toks)
+    assert len(set(ref.argmax(-1).tolist())) >= 20        # the model's answers move with the context
+    check_logits(torch.cat(out), ref, dtype, f"4,230 tokens {dtype}")
 
 
 def test_long_context_bfloat16_against_float32(long_model):
