@@ -9,9 +9,31 @@
 // The arithmetic both kernels below share, written with explicit fused operations so that
 // the two compile to the same roundings: which of them a token meets depends on how many
 // tokens came with it, and its results must not.
+// The angle is position * inv_freq, the product taken in float64 and rounded to float32; its sine and
+// cosine to float32 accuracy. Angles reach 1e5 and more: the library's float32 routine then reduces the
+// argument with a long integer product, thousands of cycles in which a whole block waits for its table.
+// So the multiple of pi/2 comes off in float64 (two constants carry pi/2 to 107 bits; the product with a
+// count below 2^17 is exact enough by far) and the routine only sees what is left, at most pi/4.
 __device__ __forceinline__ void rotation_of(int pos, float inv_freq, float& sn, float& cs) {
     const float theta = (float)((double)pos * (double)inv_freq);
-    sincosf(theta, &sn, &cs);
+    const double t = (double)theta;
+    const double k = rint(t * 0.63661977236758134308);
+    double r = fma(-k, 1.57079632679489655800, t);
+    r = fma(-k, 6.12323399573676603587e-17, r);
+    float s, c;
+    sincosf((float)r, &s, &c);
+    const int quarter = (int)((long long)k & 3);
+    sn = (quarter & 1) ? c : s;
+    cs = (quarter & 1) ? s : c;
+    if (quarter == 1 || quarter == 2) cs = -cs;
+    if (quarter >= 2) sn = -sn;
+}
+// The sum over a wave's lanes, nearest lanes first (1, 2, 4, ... apart): the kernel below that gives a lane
+// four neighbouring elements adds them in this same order, inside the lane first.
+__device__ __forceinline__ float wave_sum_near_first(float v) {
+#pragma unroll
+    for (int off = 1; off < WAVE; off <<= 1) v += __shfl_xor(v, off, WAVE);
+    return v;
 }
 __device__ __forceinline__ float head_norm_scale(float sum_squares, int head_dim, float eps) {
     return 1.0f / sqrtf(sum_squares / (float)head_dim + eps);
@@ -73,7 +95,7 @@ __global__ void k_qk_norm_rope_store(const float* __restrict__ qkv, const float*
     if (!is_v) {
         float scale = 1.f;
         if (weight) {
-            ss = wave_sum(ss);
+            ss = wave_sum_near_first(ss);
             scale = head_norm_scale(ss, head_dim, eps);
         }
 #pragma unroll
@@ -174,7 +196,7 @@ __global__ __launch_bounds__(ROPE_WAVES * WAVE) void k_qk_norm_rope_store_token(
                     float ss = 0.f;
 #pragma unroll
                     for (int j = 0; j < NPL; ++j) ss = fmaf(a[b][j], a[b][j], ss);
-                    ss = wave_sum(ss);
+                    ss = wave_sum_near_first(ss);
                     scale = head_norm_scale(ss, head_dim, eps);
                 }
 #pragma unroll
@@ -215,6 +237,113 @@ __global__ __launch_bounds__(ROPE_WAVES * WAVE) void k_qk_norm_rope_store_token(
     }
 }
 
+// The same again for heads of 64 that are rotated whole (every LFM2 checkpoint): a lane takes four
+// neighbouring elements of a head, sixteen lanes a head, so a wave has four heads at a time and
+// nothing goes through LDS but the block's sines and cosines. The partner of an element is sixteen
+// lanes' worth away (i, i + 32: the lane 8 further in its group) or beside it in the lane (2i, 2i + 1).
+// Sums and products are taken in the order and with the roundings of the kernels above.
+// (e0^2 + e1^2) + (e2^2 + e3^2), every square and every sum rounded on its own: what four lanes with one
+// element each arrive at after two steps of the sum above. (The compiler would otherwise fuse a square
+// into the sum that follows it; the *_rn functions of the HIP headers are plain operators and do not stop it.)
+__device__ __forceinline__ float squares_of_four(const float (&e)[4]) {
+#pragma clang fp contract(off)
+    const float s0 = e[0] * e[0], s1 = e[1] * e[1], s2 = e[2] * e[2], s3 = e[3] * e[3];
+    const float a = s0 + s1, b = s2 + s3;
+    return a + b;
+}
+template <typename T> __device__ __forceinline__ void store4(T* dst, const float (&v)[4]);
+template <> __device__ __forceinline__ void store4<float>(float* dst, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+}
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* dst, const float (&v)[4]) {
+    union { bf16_t h[4]; uint2 u; } o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o.h[j] = f32_to_bf16(v[j]);
+    *reinterpret_cast<uint2*>(dst) = o.u;
+}
+
+template <typename T, int ROUNDS>
+__global__ __launch_bounds__(ROPE_WAVES * WAVE) void k_qk_norm_rope_store_token64(
+    const float* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
+    const float* __restrict__ inv_freq, int interleaved, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ row_of_token, const int32_t* __restrict__ block_table, int table_stride,
+    int page_size, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int write_kv,
+    int heads, int kv_heads, int n_pages, int v_transposed) {
+    constexpr int D = 64, HALF = 32;
+    __shared__ float sn_tab[HALF], cs_tab[HALF];
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x / WAVE;
+    const int l16 = lane & 15, sub = lane >> 4;
+    const int units = heads + 2 * kv_heads;
+    const int t = blockIdx.x;
+    const int pos = positions[t];
+    int page = -1;
+    if (write_kv) page = block_table[(size_t)row_of_token[t] * table_stride + pos / page_size];
+    if (threadIdx.x < HALF) rotation_of(pos, inv_freq[threadIdx.x], sn_tab[threadIdx.x], cs_tab[threadIdx.x]);
+    float wq[4], wk[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        wq[j] = q_weight ? q_weight[4 * l16 + j] : 1.f;
+        wk[j] = k_weight ? k_weight[4 * l16 + j] : 1.f;
+    }
+    const float* src = qkv + (size_t)t * units * D + 4 * l16;
+    // all of the wave's rows are asked for before the first is used
+    float4 rows[ROUNDS];
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+        const int u = (r * ROPE_WAVES + wave) * 4 + sub;
+        rows[r] = *reinterpret_cast<const float4*>(src + (size_t)min(u, units - 1) * D);
+    }
+    __syncthreads();
+    // element j of this lane: the pair it belongs to, and whether it is the pair's second element
+    float sn[4], cs[4];
+    bool second[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int pair = interleaved ? 2 * l16 + (j >> 1) : 4 * (l16 & 7) + j;
+        sn[j] = sn_tab[pair];
+        cs[j] = cs_tab[pair];
+        second[j] = interleaved ? (j & 1) : (l16 >= 8);
+    }
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+        const int u = (r * ROPE_WAVES + wave) * 4 + sub;
+        const bool is_q = u < heads;
+        const bool is_v = u >= heads + kv_heads;
+        const float e[4] = {rows[r].x, rows[r].y, rows[r].z, rows[r].w};
+        // (every lane takes part in the exchanges, also those of a value head or past the last unit)
+        float ss = squares_of_four(e);
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) ss += __shfl_xor(ss, off, WAVE);
+        const float scale = head_norm_scale(ss, D, eps);
+        float n[4], partner[4], o[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) n[j] = q_weight ? e[j] * scale * (is_q ? wq[j] : wk[j]) : e[j];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) partner[j] = interleaved ? n[j ^ 1] : __shfl_xor(n[j], 8, WAVE);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float x0 = second[j] ? partner[j] : n[j], x1 = second[j] ? n[j] : partner[j];
+            const float turned = second[j] ? fmaf(x0, sn[j], x1 * cs[j]) : fmaf(x0, cs[j], -(x1 * sn[j]));
+            o[j] = is_v ? e[j] : turned;
+        }
+        if (u >= units) continue;
+        if (is_q) {
+            store4<T>(q_out + ((size_t)t * heads + u) * D + 4 * l16, o);
+        } else if (write_kv && page >= 0 && page < n_pages) {        // never write outside the pool
+            const int kvh = is_v ? u - heads - kv_heads : u - heads;
+            if (is_v && v_transposed) {
+                T* dst = v_cache + (((size_t)page * kv_heads + kvh) * D + 4 * l16) * page_size + (pos % page_size);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) store_f32<T>(dst, (size_t)j * page_size, o[j]);
+            } else {
+                T* cache = is_v ? v_cache : k_cache;
+                store4<T>(cache + (((size_t)page * kv_heads + kvh) * page_size + (pos % page_size)) * D + 4 * l16, o);
+            }
+        }
+    }
+}
+
 template <typename T>
 static void launch_rope_token(const float* qkv, const float* q_weight, const float* k_weight, float eps,
                               const float* inv_freq, int n_freq, int interleaved, const int32_t* positions,
@@ -225,6 +354,24 @@ static void launch_rope_token(const float* qkv, const float* q_weight, const flo
     k_qk_norm_rope_store_token<T, NPL, UB><<<n_tokens, ROPE_WAVES * WAVE, 0, s>>>(                                   \
         qkv, q_weight, k_weight, eps, inv_freq, n_freq, interleaved, positions, row_of_token, block_table, table_stride,         \
         page_size, q_out, k_cache, v_cache, write_kv, n_tokens, heads, kv_heads, head_dim, n_pages, v_transposed)
+    const int units = heads + 2 * kv_heads;
+    // heads of 64 rotated whole, vectors aligned, up to 96 units a token: four elements a lane
+    const bool vectors = ((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)v_cache |
+                          (uintptr_t)q_weight | (uintptr_t)k_weight) % 16 == 0;
+    if (head_dim == 64 && n_freq == 32 && vectors && units <= 96) {
+#define ROPE_TOKEN64(ROUNDS)                                                                                        \
+    k_qk_norm_rope_store_token64<T, ROUNDS><<<n_tokens, ROPE_WAVES * WAVE, 0, s>>>(                                  \
+        qkv, q_weight, k_weight, eps, inv_freq, interleaved, positions, row_of_token, block_table, table_stride,     \
+        page_size, q_out, k_cache, v_cache, write_kv, heads, kv_heads, n_pages, v_transposed)
+        const int rounds = (units + 4 * ROPE_WAVES - 1) / (4 * ROPE_WAVES);
+        if (rounds <= 1) ROPE_TOKEN64(1);
+        else if (rounds == 2) ROPE_TOKEN64(2);
+        else if (rounds == 3) ROPE_TOKEN64(3);
+        else if (rounds == 4) ROPE_TOKEN64(4);
+        else ROPE_TOKEN64(6);
+#undef ROPE_TOKEN64
+        return;
+    }
     if (head_dim <= 64)
         ROPE_TOKEN(1, 4);
     else if (head_dim <= 128)

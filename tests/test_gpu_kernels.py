@@ -305,7 +305,8 @@ def test_qk_norm_rope_store(H, Hk, D, rot, page_size, vt):
         assert v_cache.cpu().float().permute(0, 2, 1, 3)[untouched].abs().sum() == 0
 
 
-@pytest.mark.parametrize("H,Hk,D,rot", [(4, 2, 16, 16), (5, 1, 64, 64), (6, 3, 96, 32), (3, 1, 144, 144), (2, 2, 272, 0)])
+@pytest.mark.parametrize("H,Hk,D,rot", [(4, 2, 16, 16), (5, 1, 64, 64), (32, 8, 64, 64), (9, 3, 64, 32), (6, 3, 96, 32),
+                                        (3, 1, 144, 144), (2, 2, 272, 0)])
 @pytest.mark.parametrize("vt", [False, True])
 def test_qk_norm_rope_store_many_tokens(H, Hk, D, rot, vt):
     """From 400 tokens on a launch takes the kernel with a block per token. A token's results are the
@@ -351,6 +352,63 @@ def test_qk_norm_rope_store_many_tokens(H, Hk, D, rot, vt):
             page = tables[r][pos // page_size]
             torch.testing.assert_close(kc[page, :, pos % page_size], k_ref[t], **tol)
             torch.testing.assert_close(vc[page, :, pos % page_size], v[t], **tol)
+
+
+@pytest.mark.parametrize("n_tokens", [5, 450])
+def test_rotation_at_far_positions(n_tokens):
+    """Angles of 1e5 radians and more (positions up to 127,999, a base of 10 so that the slow pairs turn
+    too): sines and cosines keep float32 accuracy after the argument's reduction. A wrong multiple of
+    pi/2, or a quarter turn taken the wrong way, would show as errors of order one."""
+    H, Hk, D = 3, 1, 64
+    g = torch.Generator().manual_seed(5)
+    positions = torch.randint(90000, 128000, (n_tokens,), generator=g).to(torch.int32)
+    positions[0], positions[1] = 127999, 0
+    qkv = rnd(n_tokens, (H + 2 * Hk) * D, seed=9)
+    i = np.arange(D // 2, dtype=np.float32)
+    inv_np = np.power(np.float32(10.0), (np.float32(-2.0) * i / np.float32(D))).astype(np.float32)
+    q_out = torch.empty(n_tokens, H, D, device=DEV)
+    ops().qk_norm_rope_store(qkv.to(DEV), None, None, 1e-6, torch.from_numpy(inv_np).to(DEV), positions.to(DEV),
+                             torch.zeros(n_tokens, dtype=torch.int32, device=DEV), None, 16, q_out, None, None, H, Hk, D)
+    theta = (positions.numpy().astype(np.float64)[:, None] * inv_np.astype(np.float64)).astype(np.float32).astype(np.float64)
+    cos, sin = torch.from_numpy(np.cos(theta)).unsqueeze(1), torch.from_numpy(np.sin(theta)).unsqueeze(1)
+    x = qkv[:, :H * D].reshape(n_tokens, H, D).double()
+    ref = torch.cat([x[..., :32] * cos - x[..., 32:] * sin, x[..., :32] * sin + x[..., 32:] * cos], dim=-1)
+    assert theta.max() > 1e5
+    torch.testing.assert_close(q_out.cpu().double(), ref, rtol=0, atol=2e-6)
+
+
+@pytest.mark.parametrize("H,Hk,D", [(7, 2, 64), (3, 1, 32)])
+def test_rotation_of_neighbouring_pairs_many_tokens(H, Hk, D):
+    """Pairs (2i, 2i + 1) instead of (i, i + half): the kernel with a block per token (heads of 64 take
+    four elements a lane there) gives the bits of the kernel with a wave per head, and the rotation
+    is the one written out here."""
+    segments, page_size, n_pages = [(3, 411)], 16, 30
+    qkv = rnd(411, (H + 2 * Hk) * D, seed=D + 1).to(DEV)
+    qw, kw = (1 + 0.1 * rnd(D, seed=1)).to(DEV), (1 + 0.1 * rnd(D, seed=2)).to(DEV)
+    i = np.arange(D // 2, dtype=np.float32)
+    inv_np = np.power(np.float32(1e4), (np.float32(-2.0) * i / np.float32(D))).astype(np.float32)
+    inv = torch.from_numpy(inv_np).to(DEV)
+    results = []
+    for step in (411, 9):
+        ctx = hand_context(segments, page_size, n_pages, torch.float32, DEV, kv_sites={0: (Hk, D)})
+        k_cache, v_cache, table = ctx.kv(0)
+        q_out = torch.empty(411, H, D, device=DEV)
+        for t0 in range(0, 411, step):
+            t1 = min(411, t0 + step)
+            ops().qk_norm_rope_store(qkv[t0:t1], qw, kw, 1e-6, inv, ctx.positions[t0:t1], ctx.row_of_token[t0:t1],
+                                     table, page_size, q_out[t0:t1], k_cache, v_cache, H, Hk, D, interleaved=True)
+        results.append((q_out.cpu(), k_cache.cpu().clone(), v_cache.cpu().clone()))
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    positions = np.asarray(ctx.positions.cpu().tolist(), dtype=np.float64)
+    theta = torch.from_numpy((positions[:, None] * inv_np.astype(np.float64)).astype(np.float32))
+    cos, sin = theta.cos().unsqueeze(1), theta.sin().unsqueeze(1)
+    x = P.rms_norm(qkv.cpu()[:, :H * D].reshape(411, H, D), qw.cpu(), 1e-6)
+    ref = x.clone()
+    ref[..., 0::2] = x[..., 0::2] * cos - x[..., 1::2] * sin
+    ref[..., 1::2] = x[..., 0::2] * sin + x[..., 1::2] * cos
+    torch.testing.assert_close(results[0][0], ref, rtol=1e-5, atol=1e-5)
+    assert (ref - x).abs().max() > 0.5          # it did turn
 
 
 # ---------------------------------------------------------------- attention
