@@ -1,6 +1,6 @@
 """Configurations at the edges of what the kernels take, end to end against the plain
 implementation: 13 heads of 16 without groups, a vocabulary and a feed-forward width that are no
-multiple of 8, 5 and 8 conv taps, head sizes of 80, 160 and 256 (the last two beyond the
+multiple of 8, 5 and 8 conv taps, head sizes of 48, 80, 96, 128, 160 and 256 (the last two beyond the
 matrix-core attention kernels), a window that is no multiple of a page. Each runs a random
 schedule of mixed batches (portions of up to 200 tokens beside single tokens, pages used again,
 only some places wanted), in float32 and in bfloat16."""
@@ -31,6 +31,14 @@ ODD = {
                         num_attention_heads=3, num_key_value_heads=1, block_ff_dim=72, conv_L_cache=8, conv_bias=True),
     "heads_of_256": _cfg(vocab_size=130, hidden_size=512, num_hidden_layers=2, layer_types=["full_attention", "conv"],
                          num_attention_heads=2, num_key_value_heads=2, block_ff_dim=64, conv_L_cache=3),
+    "heads_of_128_in_groups": _cfg(vocab_size=300, hidden_size=512, num_hidden_layers=2,
+                                   layer_types=["full_attention", "conv"], num_attention_heads=4,
+                                   num_key_value_heads=2, block_ff_dim=96, conv_L_cache=3),
+    "heads_of_96": _cfg(vocab_size=150, hidden_size=288, num_hidden_layers=2, layer_types=["conv", "full_attention"],
+                        num_attention_heads=3, num_key_value_heads=3, block_ff_dim=80, conv_L_cache=3),
+    "six_heads_of_48": _cfg(vocab_size=99, hidden_size=288, num_hidden_layers=2,
+                            layer_types=["full_attention", "full_attention"], num_attention_heads=6,
+                            num_key_value_heads=2, block_ff_dim=120, conv_L_cache=3),
     "heads_of_160_window_33": _cfg(vocab_size=130, hidden_size=320, num_hidden_layers=2,
                                    layer_types=["sliding_attention", "full_attention"], num_attention_heads=2,
                                    num_key_value_heads=1, block_ff_dim=64, conv_L_cache=3, sliding_window=33),
