@@ -87,6 +87,25 @@ int imparo_attention_decode(const void* q, const void* k_cache, const void* v_ca
                             int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
                             int n_splits, imparo_stream stream);
 
+// The same for a step whose rows' keys and values are not in the cache yet: qkv is the fused
+// projection's float32 rows [tokens, (heads + 2 kv_heads) x head_dim] (q heads, k heads, v heads). The
+// launch norms each head of q and k (weights [head_dim], or both null: no norm), rotates them
+// (inv_freq [n_freq] with 2 n_freq = head_dim, pairs (i, i + n_freq) or with `interleaved`
+// (2i, 2i + 1); n_freq 0: no rotation), attends over the cached keys before each row's position and
+// the new key, and with write_kv puts the new key and value into their page (V pages transposed).
+// It replaces imparo_qk_norm_rope_store + imparo_attention_decode for such a step, in one launch less.
+// Head sizes 64 and 128 (imparo_attention_decode_qkv_takes); a layer that reads another layer's cache
+// finds the row's key there already and takes the two-launch form.
+int imparo_attention_decode_qkv_takes(int head_dim, int n_freq);
+int imparo_attention_decode_qkv_pays(int n_rows);       // few rows: the one launch is the faster way
+int imparo_attention_decode_qkv(const float* qkv, const float* q_weight, const float* k_weight, float eps,
+                                const float* inv_freq, int n_freq, int interleaved, void* k_cache, void* v_cache,
+                                int write_kv, void* out, float* part_o, float* part_ml, const int32_t* rows,
+                                int n_rows, const int32_t* seg_start, const int32_t* positions,
+                                const int32_t* block_table, int table_stride, int page_size, int heads,
+                                int kv_heads, int head_dim, int n_pages, float scale, int window, int n_splits,
+                                imparo_stream stream);
+
 // imparo_attention_decode for callers that cannot allocate device memory: code under HIP graph
 // capture, tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the
 // reference. The splits' partial results go through a buffer of IMPARO_STATIC_SCRATCH_BYTES that the

@@ -189,17 +189,110 @@ __device__ __forceinline__ void decode_tile(DecodeState<ND>& st, const DecodeTil
 // and are merged in wave order; one partial (max, sum, O) per split goes to
 // scratch for the merge kernel. With a single split the block writes the
 // normalised result itself and no merge follows.
+// FROM_QKV: the step's rows come as the fused projection's float32 rows [token, (heads + 2 kv_heads) x D]
+// instead of finished queries, and their keys and values are not in the cache yet. Every block norms and
+// rotates its own queries (the work of one wave over 16 heads; the sines and cosines once a block in
+// LDS); the block whose split holds the row's own position also norms and rotates the new key, weighs
+// it and the new value in from registers (the cached keys end one position earlier), and, for a layer
+// that owns its cache, writes both into their page: the launch that would do all this ahead of the
+// attention is gone. Head sizes of 64 and 128 rotated whole, where both elements of a pair (i, i + D/2)
+// or (2i, 2i + 1) sit in one lane.
+struct FromQkv {
+    const float* qkv;
+    const float* q_weight;      // per-head norm weights [D], or null: no norm
+    const float* k_weight;
+    const float* inv_freq;      // [D / 2], or null: no rotation
+    bf16_t* k_out;              // the caches again, to write: null for a layer that reads another's cache
+    bf16_t* v_out;
+    float eps;
+    int interleaved;
+};
+
+// One head's 8 x NK elements of a lane (dims dk*32 + 8*g + j): asked for early (`head_elements`, with the
+// norm's weights), then normed, rotated and rounded to bfloat16 (`normed_rotated`) once the block's sines
+// and cosines are there. All lanes with the same lane % 16 share a head: the sum of squares crosses
+// lanes 16 and 32 apart. The norm's weights are read from LDS.
 template <int ND>
-__global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_decode(
+struct HeadElements {
+    float e[(ND + 1) / 2][8];
+};
+template <int ND>
+__device__ __forceinline__ void head_elements(HeadElements<ND>& h, const float* src, int g) {
+    constexpr int NK = (ND + 1) / 2;
+#pragma unroll
+    for (int dk = 0; dk < NK; ++dk) {
+        const float4 a = *reinterpret_cast<const float4*>(src + dk * 32 + 8 * g);
+        const float4 b = *reinterpret_cast<const float4*>(src + dk * 32 + 8 * g + 4);
+        h.e[dk][0] = a.x, h.e[dk][1] = a.y, h.e[dk][2] = a.z, h.e[dk][3] = a.w;
+        h.e[dk][4] = b.x, h.e[dk][5] = b.y, h.e[dk][6] = b.z, h.e[dk][7] = b.w;
+    }
+}
+template <int ND>
+__device__ __forceinline__ void normed_rotated(Frag8 (&out)[(ND + 1) / 2], HeadElements<ND>& h, const float* weight,
+                                               float eps, bool rotate, int interleaved, const float* sn_tab,
+                                               const float* cs_tab, bool valid, int g) {
+    constexpr int D = ND * 16, NK = (ND + 1) / 2;
+    static_assert(D % 64 == 0, "pairs inside a lane");
+    auto& e = h.e;
+    if (weight) {                      // (in LDS)
+        float ss = 0.f;
+#pragma unroll
+        for (int dk = 0; dk < NK; ++dk)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ss = fmaf(e[dk][j], e[dk][j], ss);
+        ss += __shfl_xor(ss, 16, WAVE);
+        ss += __shfl_xor(ss, 32, WAVE);
+        const float scale = head_norm_scale(ss, D, eps);
+#pragma unroll
+        for (int dk = 0; dk < NK; ++dk)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) e[dk][j] = e[dk][j] * scale * weight[dk * 32 + 8 * g + j];
+    }
+    if (rotate) {
+        if (interleaved) {
+#pragma unroll
+            for (int dk = 0; dk < NK; ++dk)
+#pragma unroll
+                for (int j = 0; j < 8; j += 2) {
+                    const int i = dk * 16 + 4 * g + j / 2;
+                    const float x0 = e[dk][j], x1 = e[dk][j + 1], sn = sn_tab[i], cs = cs_tab[i];
+                    e[dk][j] = fmaf(x0, cs, -(x1 * sn));
+                    e[dk][j + 1] = fmaf(x0, sn, x1 * cs);
+                }
+        } else {
+#pragma unroll
+            for (int dk = 0; dk < NK / 2; ++dk)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int i = dk * 32 + 8 * g + j;
+                    const float x0 = e[dk][j], x1 = e[dk + NK / 2][j], sn = sn_tab[i], cs = cs_tab[i];
+                    e[dk][j] = fmaf(x0, cs, -(x1 * sn));
+                    e[dk + NK / 2][j] = fmaf(x0, sn, x1 * cs);
+                }
+        }
+    }
+#pragma unroll
+    for (int dk = 0; dk < NK; ++dk) {
+        out[dk].u = make_uint4(f32x2_to_bf16x2(e[dk][0], e[dk][1]), f32x2_to_bf16x2(e[dk][2], e[dk][3]),
+                               f32x2_to_bf16x2(e[dk][4], e[dk][5]), f32x2_to_bf16x2(e[dk][6], e[dk][7]));
+        out[dk].u = zero_unless(valid, out[dk].u);
+    }
+}
+
+template <int ND, bool FROM_QKV>
+__global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 4 : 2) void k_attn_decode(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out,
     const int32_t* __restrict__ rows, const int32_t* __restrict__ seg_start, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int n_pages,
-    float scale, int window, int n_splits) {
+    float scale, int window, int n_splits, FromQkv fq) {
     constexpr int D = ND * 16, NK = (ND + 1) / 2;
     constexpr int TILES = DEC_SPLIT / (MFMA_WAVES * 32);   // tiles a wave takes at most
     __shared__ float sm[MFMA_WAVES][16], sl[MFMA_WAVES][16];
     __shared__ float so[MFMA_WAVES][16][D + 1];
+    __shared__ float sn_tab[FROM_QKV ? D / 2 : 1], cs_tab[FROM_QKV ? D / 2 : 1];
+    __shared__ __attribute__((aligned(16))) float qw_tab[FROM_QKV ? D : 1], kw_tab[FROM_QKV ? D : 1];
+    __shared__ __attribute__((aligned(16))) float k_raw[FROM_QKV ? D : 1], v_raw[FROM_QKV ? D : 1];
     const int split = blockIdx.x, ri = blockIdx.z;
     const int G = heads / kv_heads, passes = (G + 15) / 16;
     const int kvh = blockIdx.y / passes, pass = blockIdx.y % passes;
@@ -207,40 +300,118 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_decode(
     const int t = seg_start[row];
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+    const int last = FROM_QKV ? pos - 1 : pos;              // the last key that is in the cache
     const int k_begin = max(split * DEC_SPLIT, lo & ~31);
-    const int k_end = min((split + 1) * DEC_SPLIT, pos + 1);
-    if (k_begin >= k_end) return;
+    const int k_end = min((split + 1) * DEC_SPLIT, last + 1);
+    const bool own = FROM_QKV && split == pos / DEC_SPLIT;  // this block weighs the row's own key in
+    if (k_begin >= k_end && !own) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int hq = pass * 16 + c;               // query head inside the group
     const bool qvalid = hq < G;
     const int head = kvh * G + min(hq, G - 1);
     DecodeState<ND> st;
-    {
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) st.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    st.m = -INFINITY;
+    st.l = 0.f;
+    Paged kv{k_cache, v_cache, block_table + (size_t)row * table_stride, page_size, kv_heads, kvh, n_pages,
+             __ffs(page_size) - 1};
+    const int hi_q = qvalid ? last : -1;
+    // (a block with the row's own key only: one clamped tile is loaded and none is used)
+    const int lo_c = min(lo, max(last, 0)), last_c = max(last, 0);
+    DecodeTile<ND> regs[TILES];
+#pragma unroll
+    for (int j = 0; j < TILES; ++j)             // past the split's end: clamped addresses, never used
+        decode_load<ND>(regs[j], kv, k_begin + (wave + j * MFMA_WAVES) * 32, lo_c, last_c, lane);
+    if (!FROM_QKV) {
         const bf16_t* qrow = q + ((size_t)t * heads + head) * D;
 #pragma unroll
         for (int dk = 0; dk < NK; ++dk) {
             const int d = dk * 32 + 8 * g;
             st.q[dk].u = zero_unless(qvalid && d < D, *reinterpret_cast<const uint4*>(qrow + min(d, D - 8)));
         }
-#pragma unroll
-        for (int dt = 0; dt < ND; ++dt) st.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        st.m = -INFINITY;
-        st.l = 0.f;
     }
-    Paged kv{k_cache, v_cache, block_table + (size_t)row * table_stride, page_size, kv_heads, kvh, n_pages,
-             __ffs(page_size) - 1};
-    const int hi_q = qvalid ? pos : -1;
-    DecodeTile<ND> regs[TILES];
-#pragma unroll
-    for (int j = 0; j < TILES; ++j)             // past the split's end: clamped addresses, never used
-        decode_load<ND>(regs[j], kv, k_begin + (wave + j * MFMA_WAVES) * 32, lo, pos, lane);
+    const int units = heads + 2 * kv_heads;
+    if constexpr (FROM_QKV) {
+        // The tiles' loads are on their way; so is the query's row, before anything waits. Meanwhile the
+        // block's sines and cosines are worked out and the norms' weights go to LDS.
+        HeadElements<ND> qh;
+        head_elements<ND>(qh, fq.qkv + ((size_t)t * units + head) * D, g);
+        if (fq.inv_freq && (int)threadIdx.x < D / 2)
+            rotation_of(pos, fq.inv_freq[threadIdx.x], sn_tab[threadIdx.x], cs_tab[threadIdx.x]);
+        if (fq.q_weight && (int)threadIdx.x >= 128 && (int)threadIdx.x < 128 + D / 2) {     // (another wave's lanes)
+            const int i = (int)threadIdx.x - 128;
+            qw_tab[2 * i] = fq.q_weight[2 * i], qw_tab[2 * i + 1] = fq.q_weight[2 * i + 1];
+            kw_tab[2 * i] = fq.k_weight[2 * i], kw_tab[2 * i + 1] = fq.k_weight[2 * i + 1];
+        }
+        if (own && wave == 1 && lane < D / 2) {      // the row's new key and value wait in LDS for the first wave
+            const int u = lane < D / 4 ? heads + kvh : heads + kv_heads + kvh, at = 4 * (lane % (D / 4));
+            const float4 x = *reinterpret_cast<const float4*>(fq.qkv + ((size_t)t * units + u) * D + at);
+            *reinterpret_cast<float4*>((lane < D / 4 ? k_raw : v_raw) + at) = x;
+        }
+        __syncthreads();
+        normed_rotated<ND>(st.q, qh, fq.q_weight ? qw_tab : nullptr, fq.eps, fq.inv_freq != nullptr, fq.interleaved,
+                           sn_tab, cs_tab, qvalid, g);
+    }
 #pragma unroll
     for (int j = 0; j < TILES; ++j) {
         const int kb = k_begin + (wave + j * MFMA_WAVES) * 32;
         if (kb < k_end) {
-            const bool full = kb >= lo && kb + 31 <= pos;
-            decode_tile<ND>(st, regs[j], kb, lo, hi_q, lo, pos, full, scale, lane);
+            const bool full = kb >= lo && kb + 31 <= last;
+            decode_tile<ND>(st, regs[j], kb, lo, hi_q, lo, last, full, scale, lane);
+        }
+    }
+    if constexpr (FROM_QKV) {
+        if (own && wave == 0) {
+            // the row's own key and value, from the projection's row: every lane holds the key's dims
+            // dk*32 + 8*g + j (the same for all 16 heads) and the value's dims dt*16 + 4*g + i
+            Frag8 kf[NK];
+            HeadElements<ND> kh;
+            head_elements<ND>(kh, k_raw, g);
+            float4 vnew[ND];
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) vnew[dt] = *reinterpret_cast<const float4*>(v_raw + dt * 16 + 4 * g);
+            normed_rotated<ND>(kf, kh, fq.k_weight ? kw_tab : nullptr, fq.eps, fq.inv_freq != nullptr, fq.interleaved,
+                               sn_tab, cs_tab, true, g);
+            bf16_t vb[ND][4];
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) {
+                const float4 v4 = vnew[dt];
+                vb[dt][0] = f32_to_bf16(v4.x), vb[dt][1] = f32_to_bf16(v4.y);
+                vb[dt][2] = f32_to_bf16(v4.z), vb[dt][3] = f32_to_bf16(v4.w);
+            }
+            float dot = 0.f;
+#pragma unroll
+            for (int dk = 0; dk < NK; ++dk)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) dot = fmaf((float)st.q[dk].v[j], (float)kf[dk].v[j], dot);
+            dot += __shfl_xor(dot, 16, WAVE);
+            dot += __shfl_xor(dot, 32, WAVE);
+            if (qvalid) {
+                const float sc = dot * scale;
+                const float m_new = fmaxf(st.m, sc);
+                const float corr = (st.m == -INFINITY) ? 0.f : __expf(st.m - m_new);
+                const float p = bf16_to_f32(f32_to_bf16(__expf(sc - m_new)));    // rounded as the tiles' weights are
+                st.l = st.l * corr + p;
+                st.m = m_new;
+#pragma unroll
+                for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) st.o[dt][i] = fmaf(p, bf16_to_f32(vb[dt][i]), st.o[dt][i] * corr);
+            }
+            const int page = kv.table[pos >> kv.page_shift];
+            if (fq.k_out && pass == 0 && c == 0 && page >= 0 && page < n_pages) {      // never outside the pool
+                const int slot = pos & (page_size - 1);
+                bf16_t* kdst = fq.k_out + (((size_t)page * kv_heads + kvh) * page_size + slot) * D + 8 * g;
+#pragma unroll
+                for (int dk = 0; dk < NK; ++dk) *reinterpret_cast<uint4*>(kdst + dk * 32) = kf[dk].u;
+                bf16_t* vdst = fq.v_out + ((size_t)page * kv_heads + kvh) * page_size * D + slot;
+#pragma unroll
+                for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) vdst[(size_t)(dt * 16 + 4 * g + i) * page_size] = vb[dt][i];
+            }
         }
     }
     if (g == 0) {
@@ -978,12 +1149,24 @@ static int attention_decode_launch(const void* q, const void* k_cache, const voi
                                    const int32_t* seg_start, const int32_t* positions,
                                    const int32_t* block_table, int table_stride, int page_size,
                                    int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
-                                   int n_splits, hipStream_t s) {
+                                   int n_splits, hipStream_t s, const FromQkv* from_qkv = nullptr) {
     const int G = heads / kv_heads;
     dim3 grid(n_splits, kv_heads * ((G + 15) / 16), n_rows);
-    DISPATCH_ND(head_dim / 16, (k_attn_decode<ND><<<grid, MFMA_WAVES * 64, 0, s>>>(
-        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, part_o, part_ml, (bf16_t*)out, rows, seg_start,
-        positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, n_splits)));
+    if (from_qkv) {
+#define DECODE_FROM_QKV(ND)                                                                                          \
+    k_attn_decode<ND, true><<<grid, MFMA_WAVES * 64, 0, s>>>(                                                        \
+        nullptr, (const bf16_t*)k_cache, (const bf16_t*)v_cache, part_o, part_ml, (bf16_t*)out, rows, seg_start,     \
+        positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, n_splits, *from_qkv)
+        if (head_dim == 64) DECODE_FROM_QKV(4);
+        else if (head_dim == 128) DECODE_FROM_QKV(8);
+        else return IMPARO_BAD_ARGUMENT;
+#undef DECODE_FROM_QKV
+    } else {
+        DISPATCH_ND(head_dim / 16, (k_attn_decode<ND, false><<<grid, MFMA_WAVES * 64, 0, s>>>(
+            (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, part_o, part_ml, (bf16_t*)out, rows,
+            seg_start, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window,
+            n_splits, FromQkv{})));
+    }
     if (launch_status()) return IMPARO_LAUNCH_FAILED;
     if (n_splits == 1) return IMPARO_OK;
     k_attn_decode_merge<<<n_rows * heads, 64, 0, s>>>(part_o, part_ml, (bf16_t*)out, rows, seg_start, positions, heads,
@@ -1006,6 +1189,39 @@ extern "C" int imparo_attention_decode(const void* q, const void* k_cache, const
     return attention_decode_launch(q, k_cache, v_cache, out, part_o, part_ml, rows, n_rows, seg_start, positions,
                                    block_table, table_stride, page_size, heads, kv_heads, head_dim, n_pages, scale,
                                    window, n_splits, (hipStream_t)stream);
+}
+
+// Which head sizes and rotations imparo_attention_decode_qkv takes: 64 or 128, rotated whole or not at all.
+extern "C" int imparo_attention_decode_qkv_takes(int head_dim, int n_freq) {
+    return (head_dim == 64 || head_dim == 128) && (n_freq == 0 || 2 * n_freq == head_dim);
+}
+// ... and for how many rows it is the faster way: every block of a row's splits makes the row's queries
+// again, which a launch of its own does once (measured at 4,096 keys: 18.9 against 16.7 + 4.6 us for 8
+// rows, 6 us a layer slower for 64).
+extern "C" int imparo_attention_decode_qkv_pays(int n_rows) { return n_rows <= 16; }
+
+extern "C" int imparo_attention_decode_qkv(const float* qkv, const float* q_weight, const float* k_weight, float eps,
+                                           const float* inv_freq, int n_freq, int interleaved, void* k_cache,
+                                           void* v_cache, int write_kv, void* out, float* part_o, float* part_ml,
+                                           const int32_t* rows, int n_rows, const int32_t* seg_start,
+                                           const int32_t* positions, const int32_t* block_table, int table_stride,
+                                           int page_size, int heads, int kv_heads, int head_dim, int n_pages,
+                                           float scale, int window, int n_splits, imparo_stream stream) {
+    const int bad = check_common(qkv, k_cache, v_cache, out, rows, seg_start, positions, block_table, table_stride,
+                                 page_size, heads, kv_heads, head_dim, n_pages, window);
+    if (bad) return bad;
+    if (!part_o || !part_ml || n_rows < 0 || n_splits <= 0 || n_splits > 65535) return IMPARO_BAD_ARGUMENT;
+    if (!imparo_attention_decode_qkv_takes(head_dim, n_freq) || (n_freq > 0 && !inv_freq)) return IMPARO_BAD_ARGUMENT;
+    if ((q_weight == nullptr) != (k_weight == nullptr) || (q_weight && !(eps > 0.f))) return IMPARO_BAD_ARGUMENT;
+    if (((uintptr_t)qkv | (uintptr_t)q_weight | (uintptr_t)k_weight | (uintptr_t)k_cache) % 16 != 0)
+        return IMPARO_BAD_ARGUMENT;
+    if (n_rows == 0) return IMPARO_OK;
+    if (n_rows > 65535) return IMPARO_BAD_ARGUMENT;
+    const FromQkv fq{qkv, q_weight, k_weight, n_freq > 0 ? inv_freq : nullptr, write_kv ? (bf16_t*)k_cache : nullptr,
+                     write_kv ? (bf16_t*)v_cache : nullptr, eps, interleaved};
+    return attention_decode_launch(nullptr, k_cache, v_cache, out, part_o, part_ml, rows, n_rows, seg_start, positions,
+                                   block_table, table_stride, page_size, heads, kv_heads, head_dim, n_pages, scale,
+                                   window, n_splits, (hipStream_t)stream, &fq);
 }
 
 // ---------------------------------------------------------------- decode without a workspace argument

@@ -70,6 +70,41 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
     return total;
 }
 
+// ---- what every kernel that norms and rotates a head shares, so that all of them round alike
+// The angle is position * inv_freq, the product taken in float64 and rounded to float32; its sine and
+// cosine to float32 accuracy. Angles reach 1e5 and more, where a float32 library routine reduces the
+// argument with a long integer product (thousands of cycles in which a whole block waits for its table,
+// and the routine's code for that case weighs on the small angles too). So everything is done here, in
+// float64: the multiple of pi/2 comes off (two constants carry pi/2 to 107 bits; the product with a count
+// below 2^17 is exact enough by far), and what is left, at most pi/4, goes into the two power series, cut
+// where the next term is below 2e-9 (sine, after x^9) and 2e-10 (cosine, after x^10).
+__device__ __forceinline__ void rotation_of(int pos, float inv_freq, float& sn, float& cs) {
+    const float theta = (float)((double)pos * (double)inv_freq);
+    const double t = (double)theta;
+    const double k = rint(t * 0.63661977236758134308);
+    double r = fma(-k, 1.57079632679489655800, t);
+    r = fma(-k, 6.12323399573676603587e-17, r);
+    const double z = r * r;
+    double s = fma(z, 1.0 / 362880.0, -1.0 / 5040.0);
+    s = fma(z, s, 1.0 / 120.0);
+    s = fma(z, s, -1.0 / 6.0);
+    s = fma(z * r, s, r);
+    double c = fma(z, -1.0 / 3628800.0, 1.0 / 40320.0);
+    c = fma(z, c, -1.0 / 720.0);
+    c = fma(z, c, 1.0 / 24.0);
+    c = fma(z, c, -0.5);
+    c = fma(z, c, 1.0);
+    const int quarter = (int)((long long)k & 3);
+    const float sf = (float)s, cf = (float)c;
+    sn = (quarter & 1) ? cf : sf;
+    cs = (quarter & 1) ? sf : cf;
+    if (quarter == 1 || quarter == 2) cs = -cs;
+    if (quarter >= 2) sn = -sn;
+}
+__device__ __forceinline__ float head_norm_scale(float sum_squares, int head_dim, float eps) {
+    return 1.0f / sqrtf(sum_squares / (float)head_dim + eps);
+}
+
 // Orders LDS traffic between the lanes of one wave: what any lane wrote before
 // is visible to every lane after.
 __device__ __forceinline__ void wave_lds_sync() {

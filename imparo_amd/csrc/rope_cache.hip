@@ -9,34 +9,12 @@
 // The arithmetic both kernels below share, written with explicit fused operations so that
 // the two compile to the same roundings: which of them a token meets depends on how many
 // tokens came with it, and its results must not.
-// The angle is position * inv_freq, the product taken in float64 and rounded to float32; its sine and
-// cosine to float32 accuracy. Angles reach 1e5 and more: the library's float32 routine then reduces the
-// argument with a long integer product, thousands of cycles in which a whole block waits for its table.
-// So the multiple of pi/2 comes off in float64 (two constants carry pi/2 to 107 bits; the product with a
-// count below 2^17 is exact enough by far) and the routine only sees what is left, at most pi/4.
-__device__ __forceinline__ void rotation_of(int pos, float inv_freq, float& sn, float& cs) {
-    const float theta = (float)((double)pos * (double)inv_freq);
-    const double t = (double)theta;
-    const double k = rint(t * 0.63661977236758134308);
-    double r = fma(-k, 1.57079632679489655800, t);
-    r = fma(-k, 6.12323399573676603587e-17, r);
-    float s, c;
-    sincosf((float)r, &s, &c);
-    const int quarter = (int)((long long)k & 3);
-    sn = (quarter & 1) ? c : s;
-    cs = (quarter & 1) ? s : c;
-    if (quarter == 1 || quarter == 2) cs = -cs;
-    if (quarter >= 2) sn = -sn;
-}
 // The sum over a wave's lanes, nearest lanes first (1, 2, 4, ... apart): the kernel below that gives a lane
 // four neighbouring elements adds them in this same order, inside the lane first.
 __device__ __forceinline__ float wave_sum_near_first(float v) {
 #pragma unroll
     for (int off = 1; off < WAVE; off <<= 1) v += __shfl_xor(v, off, WAVE);
     return v;
-}
-__device__ __forceinline__ float head_norm_scale(float sum_squares, int head_dim, float eps) {
-    return 1.0f / sqrtf(sum_squares / (float)head_dim + eps);
 }
 // lane-owned pair i of a row staged in LDS: elements (i, i + n_freq), or with `interleaved`
 // (2i, 2i + 1); reads both, then writes both

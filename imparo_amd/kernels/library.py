@@ -32,6 +32,11 @@ _SIGNATURES = {
     "imparo_qk_norm_rope_store": [P, P, P, F, P, I, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, P],
     "imparo_attention": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
     "imparo_attention_decode": [P, P, P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
+    # qkv, q_w, k_w, eps, inv_freq, n_freq, interleaved, k_cache, v_cache, write_kv, out, part_o, part_ml, rows, n_rows,
+    # seg_start, positions, table, stride, page, heads, kv_heads, head_dim, n_pages, scale, window, n_splits, stream
+    "imparo_attention_decode_qkv": [P, P, P, F, P, I, I, P, P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
+    "imparo_attention_decode_qkv_takes": [I, I],
+    "imparo_attention_decode_qkv_pays": [I],
     "imparo_attention_prefill": [P, P, P, P, P, P, I, P, I, I, P, P, P, P, I, I, I, I, I, I, F, I, P],
     "imparo_attention_prefill_splits": [I, I, I, I, I],
     "imparo_attention_decode_split": [],

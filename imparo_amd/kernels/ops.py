@@ -274,6 +274,50 @@ def attention_decode(q, k_cache, v_cache, out, part_o, part_ml, rows, n_rows: in
     return out
 
 
+def attention_decode_qkv_takes(head_dim: int, n_freq: int) -> bool:
+    """Whether attention_decode_qkv takes heads of this size with this many rotated pairs."""
+    return bool(library().imparo_attention_decode_qkv_takes(int(head_dim), int(n_freq)))
+
+
+def attention_decode_qkv_pays(n_rows: int) -> bool:
+    """Whether the one launch is the faster way for a step of this many rows."""
+    return bool(library().imparo_attention_decode_qkv_pays(int(n_rows)))
+
+
+def attention_decode_qkv(qkv, q_weight, k_weight, eps: float, inv_freq, k_cache, v_cache, out, part_o, part_ml,
+                         rows, n_rows: int, seg_start, positions, block_table, heads: int, scale: float,
+                         window: Optional[int], max_context: int, interleaved: bool = False,
+                         write_kv: bool = True) -> torch.Tensor:
+    """qk_norm_rope_store and attention_decode in one launch less, for a step whose rows all bring one
+    token: `qkv` is the fused projection's float32 rows; the new keys and values are weighed in from
+    registers and, with `write_kv`, written into their pages (V pages transposed)."""
+    n_pages, kv_heads, page_size, head_dim = k_cache.shape
+    n = qkv.shape[0]
+    _dev(qkv, "qkv", torch.float32, (n, (heads + 2 * kv_heads) * head_dim))
+    _dev(out, "attention out", torch.bfloat16)
+    if out.numel() != n * heads * head_dim:
+        raise KernelArgumentError("attention_decode_qkv: the output does not match the rows")
+    if k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16 or tuple(v_cache.shape) != (n_pages, kv_heads, head_dim, page_size):
+        raise KernelArgumentError("attention_decode_qkv: bfloat16 caches, V pages transposed")
+    n_freq = 0 if inv_freq is None else inv_freq.shape[0]
+    if not attention_decode_qkv_takes(head_dim, n_freq):
+        raise KernelArgumentError(f"attention_decode_qkv: heads of {head_dim} with {n_freq} rotated pairs are not taken")
+    split = decode_split()
+    n_splits = max(1, (max_context + split - 1) // split)
+    if part_o.numel() < n_rows * heads * n_splits * head_dim or part_ml.numel() < n_rows * heads * n_splits * 2:
+        raise KernelArgumentError("attention_decode_qkv: the scratch for partial results is too small")
+    _check(library().imparo_attention_decode_qkv(
+        qkv.data_ptr(), _dev(q_weight, "q norm weight", torch.float32, (head_dim,)),
+        _dev(k_weight, "k norm weight", torch.float32, (head_dim,)), float(eps),
+        _dev(inv_freq, "inv_freq", torch.float32), n_freq, int(bool(interleaved)), k_cache.data_ptr(),
+        v_cache.data_ptr(), int(bool(write_kv)), out.data_ptr(), _dev(part_o, "partial outputs", torch.float32),
+        _dev(part_ml, "partial sums", torch.float32), _dev(rows, "decode rows", torch.int32), n_rows,
+        _dev(seg_start, "seg_start", torch.int32), _dev(positions, "positions", torch.int32, (n,)),
+        _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size, heads, kv_heads, head_dim,
+        n_pages, float(scale), int(window or 0), n_splits, _stream()), "attention_decode_qkv")
+    return out
+
+
 def attention_prefill_splits(n_tiles: int, heads: int, kv_heads: int, head_dim: int, max_context: int) -> int:
     """Into how many parts the keys of a launch of prompt portions are cut (1: none): few queries
     over long contexts would leave most of the chip idle."""

@@ -98,27 +98,44 @@ class Attention:
             ctx.memo[key] = sum((int(n) + tile - 1) // tile for n in ctx.host_seg_len if n > 1)
         return ctx.memo[key]
 
+    def _decode_parts(self, ctx: StepContext):
+        """Room for the partial results of the single-token rows' splits."""
+        split = ops.decode_split()
+        n_splits = (ctx.max_context + split - 1) // split
+        part_o = ctx.workspace.get("attn_part_o", (ctx.n_single_rows * self.heads * n_splits * self.head_dim,),
+                                   torch.float32)
+        part_ml = ctx.workspace.get("attn_part_ml", (ctx.n_single_rows * self.heads * n_splits * 2,), torch.float32)
+        return part_o, part_ml
+
     def forward(self, ctx: StepContext, site: int, owns_cache: bool, h: torch.Tensor) -> torch.Tensor:
         T = h.shape[0]
         qkv = self.qkv(ctx, h, torch.float32, "qkv", alias="mixer_in")
         k_cache, v_cache, table = ctx.kv(site)
         vt = self.v_transposed
+        inv_freq = self.position.inv_freq
+        interleaved = bool(getattr(self.position, "interleaved", False))
+        if (vt and owns_cache and ctx.single_rows is not None and ctx.n_single_rows == T and not ctx.n_portion_rows
+                and ops.attention_decode_qkv_pays(T)
+                and ops.attention_decode_qkv_takes(self.head_dim, 0 if inv_freq is None else inv_freq.shape[0])):
+            # every row brings one token: head norm, rotation and the write of the new key and value ride
+            # in the attention launch (the new key is weighed in from registers)
+            o = ctx.workspace.get("attn_out", (T, self.heads * self.head_dim), ctx.dtype, alias="mixer_mid")
+            part_o, part_ml = self._decode_parts(ctx)
+            ops.attention_decode_qkv(qkv, self.q_norm, self.k_norm, self.norm_eps, inv_freq, k_cache, v_cache, o,
+                                     part_o, part_ml, ctx.single_rows, ctx.n_single_rows, ctx.seg_start,
+                                     ctx.positions, table, self.heads, self.scale, self.window, ctx.max_context,
+                                     interleaved=interleaved)
+            return self.out(ctx, o, torch.float32, "mixer_out", sliced_ok=True)
         q = ctx.workspace.get("q", (T, self.heads, self.head_dim), ctx.dtype)
-        ops.qk_norm_rope_store(qkv, self.q_norm, self.k_norm, self.norm_eps, self.position.inv_freq,
+        ops.qk_norm_rope_store(qkv, self.q_norm, self.k_norm, self.norm_eps, inv_freq,
                                ctx.positions, ctx.row_of_token, table if owns_cache else None, ctx.page_size,
                                q, k_cache if owns_cache else None, v_cache if owns_cache else None,
-                               self.heads, self.kv_heads, self.head_dim, v_transposed=vt,
-                               interleaved=bool(getattr(self.position, "interleaved", False)))
+                               self.heads, self.kv_heads, self.head_dim, v_transposed=vt, interleaved=interleaved)
         o = ctx.workspace.get("attn_out", (T, self.heads * self.head_dim), ctx.dtype, alias="mixer_mid")
         if vt and ctx.single_rows is not None:
             # matrix-core kernels: single tokens split over their keys, portions tiled over their queries
             if ctx.n_single_rows:
-                split = ops.decode_split()
-                n_splits = (ctx.max_context + split - 1) // split
-                part_o = ctx.workspace.get("attn_part_o", (ctx.n_single_rows * self.heads * n_splits * self.head_dim,),
-                                           torch.float32)
-                part_ml = ctx.workspace.get("attn_part_ml", (ctx.n_single_rows * self.heads * n_splits * 2,),
-                                            torch.float32)
+                part_o, part_ml = self._decode_parts(ctx)
                 ops.attention_decode(q, k_cache, v_cache, o, part_o, part_ml, ctx.single_rows, ctx.n_single_rows,
                                      ctx.seg_start, ctx.positions, table, self.scale, self.window, ctx.max_context)
             if ctx.n_portion_rows:

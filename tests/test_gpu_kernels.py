@@ -540,6 +540,103 @@ def test_matrix_core_attention_with_32_queries_a_wave(H, Hk, D, ctx, q):
     torch.testing.assert_close(wide, narrow, rtol=2 ** -7, atol=2 ** -7)
 
 
+@pytest.mark.parametrize("H,Hk,D", [(8, 2, 64), (5, 5, 64), (40, 2, 64), (4, 1, 128)])
+@pytest.mark.parametrize("page_size,window,interleaved,normed,rotated", [
+    (16, None, False, True, True), (64, None, False, True, True), (64, 100, True, True, True),
+    (32, 1, False, True, True), (16, None, False, False, True), (64, 300, False, True, False)])
+def test_decode_attention_from_the_projection_rows(H, Hk, D, page_size, window, interleaved, normed, rotated):
+    """Rows of one token whose keys and values are not in the cache yet: one launch norms and rotates
+    q and k, attends over the cached keys and the new one, and writes the new key and value into their
+    page. Held to the plain functions, and to the two launches it replaces. The new position's slot
+    holds NaN beforehand (so does every slot beyond the contexts): reading it before it is written,
+    or instead of the registers, would poison the output."""
+    ctx_lens = (1, 70, 256, 257, 700, 513, 33, 512)
+    n_pages = sum((c + page_size - 1) // page_size for c in ctx_lens) + 3
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(3)).tolist()
+    tables, nxt = [], 0
+    for c in ctx_lens:
+        k = (c + page_size - 1) // page_size
+        tables.append(perm[nxt:nxt + k])
+        nxt += k
+    ctx = hand_context([(c - 1, 1) for c in ctx_lens], page_size, n_pages, torch.bfloat16, DEV, kv_sites={0: (Hk, D)},
+                       tables=tables, v_transposed=True)
+    k_cache, v_cache, table = ctx.kv(0)
+    k_cache.fill_(float("nan"))
+    v_cache.fill_(float("nan"))
+    R = len(ctx_lens)
+    qkv = rnd(R, (H + 2 * Hk) * D, seed=11)
+    qw, kw = 1 + 0.1 * rnd(D, seed=1), 1 + 0.1 * rnd(D, seed=2)
+    base = 1e4
+    i = np.arange(D // 2, dtype=np.float32)
+    inv_np = np.power(np.float32(base), (np.float32(-2.0) * i / np.float32(D))).astype(np.float32)
+
+    def turned(x, pos, weight):              # x [heads, D] at one position
+        if normed:
+            x = P.rms_norm(x, weight, 1e-5)
+        if not rotated:
+            return x
+        theta = torch.from_numpy((np.float64(pos) * inv_np.astype(np.float64)).astype(np.float32))
+        cos, sin = theta.cos(), theta.sin()
+        out = x.clone()
+        if interleaved:
+            out[..., 0::2] = x[..., 0::2] * cos - x[..., 1::2] * sin
+            out[..., 1::2] = x[..., 0::2] * sin + x[..., 1::2] * cos
+        else:
+            h = D // 2
+            out[..., :h] = x[..., :h] * cos - x[..., h:] * sin
+            out[..., h:] = x[..., :h] * sin + x[..., h:] * cos
+        return out
+
+    bf = lambda t: t.to(torch.bfloat16).float()
+    refs, new_k, new_v = [], [], []
+    for r, c in enumerate(ctx_lens):
+        k, v = bf(rnd(c, Hk, D, seed=20 + r)), bf(rnd(c, Hk, D, seed=40 + r))
+        for p in range(c - 1):
+            page = tables[r][p // page_size]
+            k_cache[page, :, p % page_size] = k[p].to(torch.bfloat16).to(DEV)
+            v_cache[page, :, :, p % page_size] = v[p].to(torch.bfloat16).to(DEV)
+        q_r = qkv[r, :H * D].reshape(H, D)
+        k[c - 1] = bf(turned(qkv[r, H * D:(H + Hk) * D].reshape(Hk, D), c - 1, kw))
+        v[c - 1] = bf(qkv[r, (H + Hk) * D:].reshape(Hk, D))
+        q = torch.zeros(c, H, D)
+        q[c - 1] = bf(turned(q_r, c - 1, qw))
+        refs.append(torch.as_tensor(P.attend(q, k, v, range(c), 1.0 / math.sqrt(D), window))[c - 1])
+        new_k.append(k[c - 1])
+        new_v.append(v[c - 1])
+    ref = torch.stack(refs)
+    scale = 1.0 / math.sqrt(D)
+    n_splits = (ctx.max_context + 255) // 256
+    qw_d, kw_d = (qw.to(DEV), kw.to(DEV)) if normed else (None, None)
+    inv_d = torch.from_numpy(inv_np).to(DEV) if rotated else None
+    # the two launches, on a copy of the caches
+    k2, v2 = k_cache.clone(), v_cache.clone()
+    q2 = torch.empty(R, H, D, dtype=torch.bfloat16, device=DEV)
+    ops().qk_norm_rope_store(qkv.to(DEV), qw_d, kw_d, 1e-5, inv_d, ctx.positions, ctx.row_of_token, table, page_size,
+                             q2, k2, v2, H, Hk, D, v_transposed=True, interleaved=interleaved)
+    two = torch.full((R, H * D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    part_o = torch.full((R * H * n_splits * D,), float("nan"), device=DEV)
+    part_ml = torch.full((R * H * n_splits * 2,), float("nan"), device=DEV)
+    ops().attention_decode(q2, k2, v2, two, part_o, part_ml, ctx.single_rows, ctx.n_single_rows, ctx.seg_start,
+                           ctx.positions, table, scale, window, ctx.max_context)
+    # the one launch
+    one = torch.full((R, H * D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    part_o.fill_(float("nan"))
+    part_ml.fill_(float("nan"))
+    ops().attention_decode_qkv(qkv.to(DEV), qw_d, kw_d, 1e-5, inv_d, k_cache, v_cache, one, part_o, part_ml,
+                               ctx.single_rows, ctx.n_single_rows, ctx.seg_start, ctx.positions, table, H, scale,
+                               window, ctx.max_context, interleaved=interleaved)
+    one_f, two_f = one.cpu().float().reshape(R, H, D), two.cpu().float().reshape(R, H, D)
+    torch.testing.assert_close(one_f, ref, rtol=2 ** -6, atol=2 ** -6)
+    torch.testing.assert_close(one_f, two_f, rtol=2 ** -6, atol=2 ** -6)
+    # the new keys and values are in their pages, as the other launch leaves them up to one rounding, and nothing else is
+    for r, c in enumerate(ctx_lens):
+        page, slot = tables[r][(c - 1) // page_size], (c - 1) % page_size
+        torch.testing.assert_close(k_cache[page, :, slot].cpu().float(), new_k[r], rtol=2 ** -7, atol=2 ** -7)
+        assert torch.equal(v_cache[page, :, :, slot].cpu().float(), new_v[r])
+    assert torch.equal(torch.isnan(k_cache), torch.isnan(k2)) and torch.equal(torch.isnan(v_cache), torch.isnan(v2))
+    assert int((~torch.isnan(k_cache[:, 0, :, 0])).sum()) == sum(ctx_lens)
+
+
 def test_matrix_core_attention_refuses_other_sizes():
     from imparo_amd.kernels import KernelArgumentError
     assert not ops().mfma_attention_supported(torch.bfloat16, 8, 64)
