@@ -140,6 +140,7 @@ def cmd_generate(a) -> int:
     prompts = [_ids(p) for p in a.input_ids]
     t0 = time.time()
     out = generate(a.model, prompts, max_tokens=a.max_tokens, temperature=a.temperature, seed=a.seed,
+                   stop_token_ids=None if a.stop_token_ids is None else _ids(a.stop_token_ids),
                    dtype=a.dtype, ctx=a.ctx, parallel=a.parallel, max_batch_tokens=a.max_batch_tokens,
                    page_size=a.page_size, num_pages=a.num_pages,
                    kv_budget_bytes=None if a.kv_gb is None else int(a.kv_gb * (1 << 30)))
@@ -194,6 +195,8 @@ def main(argv=None) -> int:
     g.add_argument("--max-tokens", type=int, default=16)
     g.add_argument("--temperature", type=float, default=0.0)
     g.add_argument("--seed", type=int, default=0)
+    g.add_argument("--stop-token-ids", default=None,
+                   help='ids that end a reply unsent, e.g. "7,2" ("" for none; default: the model\'s eos_token_id)')
     g.add_argument("--max-batch-tokens", type=int, default=2048, help="token budget of one step")
     g.set_defaults(fn=cmd_generate)
 

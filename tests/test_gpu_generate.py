@@ -162,6 +162,14 @@ def test_command_line(loud_model_dirs, loud_plain_models, tmp_path):
                        capture_output=True, text=True, env=env, timeout=240)
     assert r.returncode == 0, r.stderr
     assert json.loads(r.stdout.splitlines()[0])["output_ids"] == want
+    # a stop id given on the command line ends the reply before it; a small pool (--num-pages) changes nothing
+    stop = next(t for i, t in enumerate(want) if i >= 2 and t not in want[:i])
+    r = subprocess.run([sys.executable, "-m", "imparo_amd", "generate", "-m", model_dirs["A"], "--dtype", "float32",
+                        "--input-ids", " ".join(map(str, p)), "--max-tokens", "6", "--stop-token-ids", f"{stop},255",
+                        "--page-size", "8", "--num-pages", "3"],
+                       capture_output=True, text=True, env=env, timeout=240)
+    assert r.returncode == 0, r.stderr
+    assert json.loads(r.stdout.splitlines()[0])["output_ids"] == want[:want.index(stop)]
     r = subprocess.run([sys.executable, "-m", "imparo_amd", "forward", "--dtype", "float32", "--decode", "5",
                         "--split", "0,4", "--scramble-kv", "--page-size", "8", model_dirs["A"]] + list(map(str, p)),
                        capture_output=True, text=True, env=env, timeout=240)
