@@ -763,7 +763,11 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
 // (Two blocks per CU for head sizes up to 64: within 256 registers a wave the compiler keeps the
 // products' results in vector registers, where the softmax wants them, not in the accumulator file.)
 // HALVES: 2 for 32 queries a wave; 1 for 16, twice the waves, when a launch has too few to fill the SIMDs twice.
-template <int ND, int HALVES>
+// PAGE_TILE: pages of at least 64 positions, so that a tile of 64 keys lies in one page. One look at the
+// block table a tile then serves every thread, and what a thread reads of a tile is at a fixed place
+// inside the page: a quarter of the instructions of the general staging, which was a quarter to a
+// third of the kernel's time.
+template <int ND, int HALVES, bool PAGE_TILE>
 __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefill_x32(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int32_t* __restrict__ rows, int n_rows,
@@ -828,7 +832,14 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     bool qvalid[HALVES];
     Frag8 qf[HALVES][NK];
     f32x4 o[HALVES][ND];
-    float m_run[HALVES], l_run[HALVES];
+    float m_run[HALVES];
+    // The sums of the weights come out of the matrix pipe too: one more product per group of 32 keys whose
+    // "values" are all ones leaves each query's sum in every row of its column. It sums the weights as the
+    // value products use them, rounded to bfloat16, and takes 32 additions and two exchanges a tile off
+    // the vector ALUs, which are what bounds this kernel.
+    f32x4 l_acc[HALVES];
+    Frag8 ones;
+    ones.u = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);
 #pragma unroll
     for (int h = 0; h < HALVES; ++h) {
         const int qi = q_first + 16 * h + c;
@@ -843,7 +854,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt) o[h][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
         m_run[h] = -INFINITY;
-        l_run[h] = 0.f;
+        l_acc[h] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     const float scale_log2 = scale * 1.44269504088896340736f;
 
@@ -862,8 +873,24 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     u32x4 kr_a[K_PER], vr_a[V_PER], kr_b[K_PER], vr_b[V_PER];
     int kpage[K_PER], vpage[V_PER];
     const int kb_last = blk_last & ~(PX_KEYS - 1);
+    // PAGE_TILE: where in a page this thread's pieces of a tile lie that starts at the page's first position
+    unsigned k_at[K_PER], v_at[V_PER];
+#pragma unroll
+    for (int j = 0; j < K_PER; ++j) {
+        const int pc = tid + j * 256;
+        k_at[j] = (unsigned)(kvh * page_size + pc / (D / 8)) * D + (pc % (D / 8)) * 8;
+    }
+#pragma unroll
+    for (int j = 0; j < V_PER; ++j) {
+        const int pc = tid + j * 256;
+        v_at[j] = (unsigned)(kvh * D + pc / (PX_KEYS / 8)) * page_size + (pc % (PX_KEYS / 8)) * 8;
+    }
     auto load_pages = [&](int kb) __attribute__((always_inline)) {
         kb = min(kb, kb_last);
+        if constexpr (PAGE_TILE) {
+            kpage[0] = table[kb >> page_shift];       // the tile's page: it holds a live key, so it is there
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < K_PER; ++j) {
             const int pc = tid + j * 256;
@@ -879,6 +906,17 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     };
     auto load_data = [&](int kb, u32x4 (&kr)[K_PER], u32x4 (&vr)[V_PER]) __attribute__((always_inline)) {
         kb = min(kb, kb_last);
+        if constexpr (PAGE_TILE) {
+            // (keys of the page outside the live range are read too: what they hold is masked, and zeroed
+            // where it would be multiplied)
+            const size_t base = (size_t)min(max(kpage[0], 0), n_pages - 1) * page_elems;
+            const unsigned first = (unsigned)(kb & (page_size - 1));
+#pragma unroll
+            for (int j = 0; j < K_PER; ++j) kr[j] = *reinterpret_cast<const u32x4*>(k_cache + base + k_at[j] + first * D);
+#pragma unroll
+            for (int j = 0; j < V_PER; ++j) vr[j] = *reinterpret_cast<const u32x4*>(v_cache + base + v_at[j] + first);
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < K_PER; ++j) {
             const int pc = tid + j * 256;
@@ -976,7 +1014,6 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
                 mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
                 const float m_new = fmaxf(m_run[h], mx);
                 const float m_sub = (m_new == -INFINITY) ? 0.f : m_new * scale_log2;   // exp2(-inf - 0) = 0: masked keys
-                float psum = 0.f;
 #pragma unroll
                 for (int s16 = 0; s16 < 4; ++s16) {
                     uint32_t pk[2];
@@ -985,7 +1022,6 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
                         const float p0 = __builtin_amdgcn_exp2f(fmaf(sc[h][s16][i], scale_log2, -m_sub));
                         const float p1 = __builtin_amdgcn_exp2f(fmaf(sc[h][s16][i + 1], scale_log2, -m_sub));
                         pk[i >> 1] = f32x2_to_bf16x2(p0, p1);
-                        psum += p0 + p1;
                     }
                     // K-slots 4 t + i of group G, s16 = 2 G + t
                     if (s16 & 1) {
@@ -996,18 +1032,18 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
                         pb[h][s16 >> 1].u.y = pk[1];
                     }
                 }
-                psum += __shfl_xor(psum, 16, WAVE);
-                psum += __shfl_xor(psum, 32, WAVE);
                 // the old sums shrink by exp2((old max - new max) * scale): by 1, and nothing to do, for
                 // every query whose maximum stood (the whole wave mostly, once the walk is under way)
                 if (__any(m_new != m_run[h])) {
                     const float corr = (m_run[h] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_run[h] - m_new) * scale_log2);
-                    l_run[h] *= corr;
+                    l_acc[h] = l_acc[h] * corr;
 #pragma unroll
                     for (int dt = 0; dt < ND; ++dt) o[h][dt] = o[h][dt] * corr;
                 }
-                l_run[h] += psum;
                 m_run[h] = m_new;
+#pragma unroll
+                for (int G = 0; G < 2; ++G)
+                    l_acc[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pb[h][G].v, l_acc[h], 0, 0, 0);
             }
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt) {
@@ -1046,7 +1082,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
             const size_t slot = ((size_t)(t0 + q_first + 16 * h + c) * heads + head) * n_splits + split;
             if (g == 0) {
                 part_ml[slot * 2] = m_run[h];               // of unscaled scores; -inf: no key, weight zero
-                part_ml[slot * 2 + 1] = l_run[h];
+                part_ml[slot * 2 + 1] = l_acc[h][0];
             }
             float* dst = part_o + slot * D + 4 * g;
 #pragma unroll
@@ -1058,7 +1094,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
 #pragma unroll
     for (int h = 0; h < HALVES; ++h) {
         if (!qvalid[h]) continue;
-        const float inv = l_run[h] > 0.f ? 1.0f / l_run[h] : 0.f;
+        const float inv = l_acc[h][0] > 0.f ? 1.0f / l_acc[h][0] : 0.f;
         bf16_t* dst = out + ((size_t)(t0 + q_first + 16 * h + c) * heads + head) * D + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt) {
@@ -1346,17 +1382,16 @@ extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, cons
         const int hpb = p.hpb;
         const bool wide = p.wide;
         dim3 grid32((unsigned)(n_tiles * (p.qt < 64 ? 64 / p.qt : 1)), heads / hpb, n_splits);
+#define PREFILL_X32_GO(ND, HALVES, PAGE_TILE)                                                                       \
+    k_attn_prefill_x32<ND, HALVES, PAGE_TILE><<<grid32, MFMA_WAVES * 64, 0, s>>>(                                    \
+        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, rows, n_rows, seg_start,     \
+        seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, hpb,      \
+        part_o, part_ml)
 #define PREFILL_X32(ND)                                                                                              \
-    if (wide)                                                                                                        \
-        k_attn_prefill_x32<ND, 2><<<grid32, MFMA_WAVES * 64, 0, s>>>(                                                \
-            (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, rows, n_rows, seg_start, \
-            seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, hpb,  \
-            part_o, part_ml);                                                                                        \
-    else                                                                                                             \
-        k_attn_prefill_x32<ND, 1><<<grid32, MFMA_WAVES * 64, 0, s>>>(                                                \
-            (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, rows, n_rows, seg_start, \
-            seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window, hpb,  \
-            part_o, part_ml)
+    if (wide && page_size >= PX_KEYS) PREFILL_X32_GO(ND, 2, true);                                                   \
+    else if (wide) PREFILL_X32_GO(ND, 2, false);                                                                     \
+    else if (page_size >= PX_KEYS) PREFILL_X32_GO(ND, 1, true);                                                      \
+    else PREFILL_X32_GO(ND, 1, false)
         switch (head_dim / 32) {
             case 1: PREFILL_X32(2); break;
             case 2: PREFILL_X32(4); break;
@@ -1364,6 +1399,7 @@ extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, cons
             default: PREFILL_X32(8);
         }
 #undef PREFILL_X32
+#undef PREFILL_X32_GO
         if (launch_status()) return IMPARO_LAUNCH_FAILED;
         if (n_splits == 1) return IMPARO_OK;
         // a block of four waves per token and four heads; tokens past the portions' last find none and leave
