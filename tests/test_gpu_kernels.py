@@ -525,7 +525,10 @@ def test_matrix_core_attention_with_the_keys_in_parts(H, Hk, D, page_size, windo
     assert ops().attention_prefill_splits(8, 16, 8, 64, 3000) == 2           # at least 1024 keys to a part
     assert ops().attention_prefill_splits(8, 16, 8, 64, 1500) == 1           # a short context is walked whole
     assert ops().attention_prefill_splits(32, 16, 8, 64, 30000) == 2         # 512 blocks
-    assert ops().attention_prefill_splits(32, 32, 8, 64, 30000) == 1         # 512 blocks of 32 queries a wave: enough
+    assert ops().attention_prefill_splits(32, 32, 8, 64, 30000) == 3         # 512 blocks of 32 queries a wave: two rounds of 768
+    assert ops().attention_prefill_splits(32, 32, 8, 64, 9000) == 1          # ... over a long context only
+    assert ops().attention_prefill_splits(64, 32, 8, 64, 30000) == 2         # 1,024 such blocks
+    assert ops().attention_prefill_splits(128, 32, 8, 64, 30000) == 1        # 2,048: enough
     assert ops().attention_prefill_splits(8, 16, 8, 80, 30000) == 1          # (the kernel for other head sizes has none)
 
 
