@@ -361,11 +361,11 @@ static void launch_rope_token(const float* qkv, const float* q_weight, const flo
 #undef ROPE_TOKEN
 }
 
-// From this many tokens on a launch takes the kernel with a block per token: its table of sines
-// and cosines costs each block a fixed 10 us or so, which the kernel with a wave per head passes
-// at about 400 tokens (40 heads of 64: 8 us at 256 tokens, 13 at 512, 43 at 2,048 against 22)
+// From this many tokens on a launch takes the kernel with a block per token (48 heads of 64, a wave per
+// head against a block per token: 3.8 against 4.1 us at 16 tokens, 4.2 against 4.3 at 64, 5.3 against 4.5
+// at 128, 8.5 against 4.9 at 256, 15 us at 2,048)
 #ifndef ROPE_TOKEN_KERNEL_FROM
-#define ROPE_TOKEN_KERNEL_FROM 400
+#define ROPE_TOKEN_KERNEL_FROM 96
 #endif
 
 extern "C" int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight, const float* k_weight, float eps,

@@ -309,7 +309,7 @@ def test_qk_norm_rope_store(H, Hk, D, rot, page_size, vt):
                                         (3, 1, 144, 144), (2, 2, 272, 0)])
 @pytest.mark.parametrize("vt", [False, True])
 def test_qk_norm_rope_store_many_tokens(H, Hk, D, rot, vt):
-    """From 400 tokens on a launch takes the kernel with a block per token. A token's results are the
+    """From 96 tokens on a launch takes the kernel with a block per token. A token's results are the
     same bits whichever kernel it met (the same tokens again, a few at a time), and right."""
     segments, page_size, n_pages = [(0, 270), (5, 141)], 16, 30
     tables = [[3, 1, 7, 9, 11, 29, 28, 13, 15, 17, 19, 21, 23, 25, 27, 5, 6], [0, 2, 4, 8, 10, 12, 14, 16, 18, 20]]
