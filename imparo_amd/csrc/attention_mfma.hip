@@ -964,12 +964,10 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
         }
     };
 
-    // One tile: LDS buffer `buf` holds it, `have` the next tile's data (asked for a tile ago), `fill`
-    // takes the loads of the tile after that; then `have` goes to the other LDS buffer.
-    auto tile_step = [&](int kb, int buf, u32x4 (&kr_have)[K_PER], u32x4 (&vr_have)[V_PER], u32x4 (&kr_fill)[K_PER],
-                         u32x4 (&vr_fill)[V_PER]) __attribute__((always_inline)) {
-        load_data(kb + 2 * PX_KEYS, kr_fill, vr_fill);      // with the pages asked for a tile ago
-        load_pages(kb + 3 * PX_KEYS);
+    // One tile: LDS buffer `buf` holds it and `have` the next tile's data, asked for two tiles ago, which goes
+    // to the other LDS buffer once this tile is done; the set is then free and takes the loads of the tile
+    // three further on (the other set holds the tile in between).
+    auto tile_step = [&](int kb, int buf, u32x4 (&kr_have)[K_PER], u32x4 (&vr_have)[V_PER]) __attribute__((always_inline)) {
         // this wave's part of the tile: keys lo_all .. pos_last
         if (wave_on && kb <= pos_last && kb + PX_KEYS - 1 >= lo_all) {
             const bool full = kb >= lo_max && kb + PX_KEYS - 1 <= pos_first && kb >= blk_lo && kb + PX_KEYS - 1 <= blk_last;
@@ -1059,6 +1057,8 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
             }
         }
         stage_store(min(kb + PX_KEYS, kb_last), buf ^ 1, kr_have, vr_have);
+        load_data(kb + 3 * PX_KEYS, kr_have, vr_have);      // with the pages asked for a tile ago
+        load_pages(kb + 4 * PX_KEYS);
         __syncthreads();
     };
     const int kb_first = blk_lo & ~(PX_KEYS - 1);
@@ -1068,11 +1068,13 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     load_data(kb_first + PX_KEYS, kr_b, vr_b);
     load_pages(kb_first + 2 * PX_KEYS);
     stage_store(kb_first, 0, kr_a, vr_a);
+    load_data(kb_first + 2 * PX_KEYS, kr_a, vr_a);
+    load_pages(kb_first + 3 * PX_KEYS);
     __syncthreads();
     for (int kb = kb_first; kb <= blk_last; kb += 2 * PX_KEYS) {
-        tile_step(kb, 0, kr_b, vr_b, kr_a, vr_a);
+        tile_step(kb, 0, kr_b, vr_b);
         if (kb + PX_KEYS > blk_last) break;
-        tile_step(kb + PX_KEYS, 1, kr_a, vr_a, kr_b, vr_b);
+        tile_step(kb + PX_KEYS, 1, kr_a, vr_a);
     }
     if (!wave_on) return;
     if (n_splits > 1) {
