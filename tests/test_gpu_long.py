@@ -50,6 +50,36 @@ def test_four_thousand_tokens_against_the_plain_implementation(long_model, dtype
     check_logits(torch.cat(out), ref, dtype, f"4,230 tokens {dtype}")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_borrowed_cache_at_head_size_64(long_model, tmp_path, dtype):
+    """A run order in which attention layer 1 runs twice, the second time on the first call's keys and
+    values, decoded token by token. In bfloat16 with heads of 64 the call that owns the cache writes the
+    new key inside its attention launch; the call that borrows must find it there and may not weigh in
+    a key of its own."""
+    import dataclasses, json, os, shutil
+    from plain_lfm2 import PlainLfm2
+    from imparo_amd.config import register_architecture, Lfm2Config, LayerCall, lfm2
+    from gpu_helpers import step_all
+    order = [(0, None), (1, None), (1, 1), (2, None), (3, None)]
+
+    def build(cfg):
+        plan = lfm2.build_plan(cfg)
+        return dataclasses.replace(plan, architecture="TestLfm2Borrowing", order=[LayerCall(l, c) for l, c in order])
+    register_architecture("TestLfm2Borrowing", Lfm2Config.from_dict, build)
+    d = str(tmp_path / "borrowing")
+    shutil.copytree(long_model, d)
+    cfg = json.load(open(os.path.join(d, "config.json")))
+    cfg["architectures"] = ["TestLfm2Borrowing"]
+    json.dump(cfg, open(os.path.join(d, "config.json"), "w"))
+    toks = prompt_tokens(512, 130, 12)
+    plain = PlainLfm2(long_model)
+    ref = plain.logits(toks, order)
+    assert not torch.allclose(ref, plain.logits(toks), atol=1e-3)        # the second call matters
+    eng = make_engine(d, dtype, page_size=64, max_tokens=512, max_requests=2)
+    got = step_all(eng, "b", toks, [61] + [1] * 40 + [9] + [1] * 20)
+    check_logits(got, ref, dtype, f"borrowed cache {dtype}")
+
+
 def test_long_context_bfloat16_against_float32(long_model):
     """16,500 tokens in portions of 2,048 (tiles of 64 queries over hundreds of
     key tiles, a window of 700 that gives pages back), two short portions (their
