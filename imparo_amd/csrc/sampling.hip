@@ -38,18 +38,26 @@ __device__ __forceinline__ Best row_best(const float* __restrict__ row, int voca
     if ((vocab & 3) == 0 && (((uintptr_t)row) & 15) == 0) {
         // four values a load, four loads in flight; a thread meets its indices in ascending
         // order, so "greater than" alone keeps the smallest index at the maximum
+        // (sixteen loads in flight: a row of 65,536 on 1,024 threads is one trip to memory, not four;
+        // no load sits under a branch: past the end the row's last piece is read again and not counted)
         const float4* row4 = reinterpret_cast<const float4*>(row);
         const int n4 = vocab >> 2;
-#pragma unroll 4
-        for (int i = threadIdx.x; i < n4; i += blockDim.x) {
-            const float4 v = row4[i];
-            const float vs[4] = {v.x, v.y, v.z, v.w};
+        constexpr int DEEP = 16;
+        for (int first = threadIdx.x; first < n4; first += DEEP * (int)blockDim.x) {
+            float4 v[DEEP];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if (vs[j] > b.v || (vs[j] == b.v && 4 * i + j < b.i)) {
-                    b.v = vs[j];
-                    b.i = 4 * i + j;
-                }
+            for (int k = 0; k < DEEP; ++k) v[k] = row4[min(first + k * (int)blockDim.x, n4 - 1)];
+#pragma unroll
+            for (int k = 0; k < DEEP; ++k) {
+                const int i = first + k * (int)blockDim.x;
+                const float vs[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (i < n4 && (vs[j] > b.v || (vs[j] == b.v && 4 * i + j < b.i))) {
+                        b.v = vs[j];
+                        b.i = 4 * i + j;
+                    }
+            }
         }
     } else {
         for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
