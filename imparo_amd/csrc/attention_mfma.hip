@@ -1108,8 +1108,13 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     }
 }
 
-// One wave per (token, head) of the launch's portion rows merges the splits of the kernel above, in
-// split order: weights exp2((max_s - max) * scale * log2 e), as the kernel itself weighs its tiles.
+// Merges the parts of the kernel above for the launch's portion rows, in the order of the parts: weights
+// exp2((max_s - max) * scale * log2 e), as the kernel itself weighs its tiles. A lane holds four
+// neighbouring elements of a head, so head_dim / 4 lanes hold a head and a wave several heads; GROUP parts
+// at a time, every load of a group asked for before the first is used and none under a branch (past the
+// last part the last is read again and weighs nothing): a wave that fetches part after part makes one trip
+// to memory after the other, and the kernel is nothing but those trips.
+template <int GROUP>
 __global__ void k_attn_prefill_merge(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                      bf16_t* __restrict__ out, const int32_t* __restrict__ rows, int n_rows,
                                      const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len,
@@ -1124,30 +1129,49 @@ __global__ void k_attn_prefill_merge(const float* __restrict__ part_o, const flo
         tok -= seg_len[r];
     }
     if (t < 0) return;
-    const int lane = threadIdx.x & 63, head = blockIdx.y * (blockDim.x / 64) + (threadIdx.x >> 6);
-    if (head >= heads) return;
+    const int lanes_a_head = head_dim / 4, heads_a_wave = 64 / lanes_a_head;
+    const int lane = threadIdx.x & 63, wave = blockIdx.y * (blockDim.x / 64) + (threadIdx.x >> 6);
+    const int sub = lane / lanes_a_head, d = (lane % lanes_a_head) * 4;
+    const int head = wave * heads_a_wave + sub;
+    if (sub >= heads_a_wave || head >= heads) return;
     const size_t base = ((size_t)t * heads + head) * n_splits;
     const float scale_log2 = scale * 1.44269504088896340736f;
     float ms = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) ms = fmaxf(ms, part_ml[(base + s) * 2]);
-    float acc[2] = {0.f, 0.f}, ls = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-        const float m = part_ml[(base + s) * 2];
-        if (m == -INFINITY) continue;                    // no key in that part: its output was never a sum
-        const float wgt = __builtin_amdgcn_exp2f((m - ms) * scale_log2);
-        ls += part_ml[(base + s) * 2 + 1] * wgt;
+    for (int s0 = 0; s0 < n_splits; s0 += GROUP) {
+        float2 ml[GROUP];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int d = lane + j * 64;
-            if (d < head_dim) acc[j] += part_o[(base + s) * head_dim + d] * wgt;
+        for (int j = 0; j < GROUP; ++j)
+            ml[j] = *reinterpret_cast<const float2*>(part_ml + (base + min(s0 + j, n_splits - 1)) * 2);
+#pragma unroll
+        for (int j = 0; j < GROUP; ++j) ms = fmaxf(ms, ml[j].x);
+    }
+    float acc[4] = {0.f, 0.f, 0.f, 0.f}, ls = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += GROUP) {
+        float2 ml[GROUP];
+        float4 o[GROUP];
+#pragma unroll
+        for (int j = 0; j < GROUP; ++j) {
+            const size_t at = base + min(s0 + j, n_splits - 1);
+            ml[j] = *reinterpret_cast<const float2*>(part_ml + at * 2);
+            o[j] = *reinterpret_cast<const float4*>(part_o + at * head_dim + d);
+        }
+#pragma unroll
+        for (int j = 0; j < GROUP; ++j) {                // in the order of the parts
+            // a part without keys has maximum -inf and an output that was never a sum: weight zero, never multiplied
+            const bool counts = s0 + j < n_splits && ml[j].x != -INFINITY;
+            const float wgt = counts ? __builtin_amdgcn_exp2f((ml[j].x - ms) * scale_log2) : 0.f;
+            ls += counts ? ml[j].y * wgt : 0.f;
+            acc[0] += counts ? o[j].x * wgt : 0.f;
+            acc[1] += counts ? o[j].y * wgt : 0.f;
+            acc[2] += counts ? o[j].z * wgt : 0.f;
+            acc[3] += counts ? o[j].w * wgt : 0.f;
         }
     }
     const float inv = ls > 0.f ? 1.0f / ls : 0.f;
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int d = lane + j * 64;
-        if (d < head_dim) out[((size_t)t * heads + head) * head_dim + d] = f32_to_bf16(acc[j] * inv);
-    }
+    uint2 packed;
+    packed.x = (uint32_t)f32_to_bf16(acc[0] * inv) | ((uint32_t)f32_to_bf16(acc[1] * inv) << 16);
+    packed.y = (uint32_t)f32_to_bf16(acc[2] * inv) | ((uint32_t)f32_to_bf16(acc[3] * inv) << 16);
+    *reinterpret_cast<uint2*>(out + ((size_t)t * heads + head) * head_dim + d) = packed;
 }
 
 // ---------------------------------------------------------------- entry points
@@ -1386,6 +1410,9 @@ extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, cons
     if (!seg_len || n_rows < 0 || n_tiles < 0 || heads > 65535) return IMPARO_BAD_ARGUMENT;
     if (n_splits < 1 || n_splits > 64 || (n_splits > 1 && (!part_o || !part_ml || head_dim % 32 != 0)))
         return IMPARO_BAD_ARGUMENT;
+    // the merge moves four elements of a head in one access
+    if (n_splits > 1 && (((uintptr_t)part_o & 15) || ((uintptr_t)part_ml & 7) || ((uintptr_t)out & 7)))
+        return IMPARO_BAD_ARGUMENT;
     if (n_rows == 0 || n_tiles == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;
     if (head_dim % 32 == 0) {
@@ -1413,10 +1440,17 @@ extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, cons
 #undef PREFILL_X32_GO
         if (launch_status()) return IMPARO_LAUNCH_FAILED;
         if (n_splits == 1) return IMPARO_OK;
-        // a block of four waves per token and four heads; tokens past the portions' last find none and leave
-        dim3 merge_grid((unsigned)n_tiles * 64, (unsigned)((heads + 3) / 4));
-        k_attn_prefill_merge<<<merge_grid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, rows, n_rows, seg_start, seg_len,
-                                                       heads, head_dim, n_splits, scale);
+        // a block of four waves per token, each wave as many heads as its lanes hold; tokens past the portions'
+        // last find none and leave
+        const int heads_a_block = 4 * (64 / (head_dim / 4));
+        dim3 merge_grid((unsigned)n_tiles * 64, (unsigned)((heads + heads_a_block - 1) / heads_a_block));
+#define MERGE(GROUP)                                                                                              \
+    k_attn_prefill_merge<GROUP><<<merge_grid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, rows, n_rows, seg_start, \
+                                                           seg_len, heads, head_dim, n_splits, scale)
+        if (n_splits <= 2) MERGE(2);
+        else if (n_splits <= 4) MERGE(4);
+        else MERGE(8);
+#undef MERGE
         return launch_status();
     }
     dim3 grid(n_tiles, heads);

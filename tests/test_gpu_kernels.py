@@ -514,7 +514,7 @@ def test_matrix_core_attention(H, Hk, D, page_size, window):
 
 @pytest.mark.parametrize("H,Hk,D", [(6, 3, 64), (40, 2, 32), (12, 3, 96), (8, 1, 128)])
 @pytest.mark.parametrize("page_size,window", [(16, None), (32, 19), (128, 300)])
-@pytest.mark.parametrize("parts", [3, 8])
+@pytest.mark.parametrize("parts", [2, 3, 8])
 def test_matrix_core_attention_with_the_keys_in_parts(H, Hk, D, page_size, window, parts):
     """Prompt portions whose blocks walk their keys in parts, merged by a second launch (few queries
     over long contexts); short contexts leave some parts without keys."""
