@@ -565,10 +565,25 @@ __device__ __forceinline__ void load_to_lds(const bf16_t* src, bf16_t* dst_wave_
                                      (void __attribute__((address_space(3)))*)dst_wave_uniform, 16, 0, 0);
 }
 
+// The same load written out, for the kernel that keeps the loads of several K-steps in flight. The compiler
+// answers a fragment read from LDS that follows any load into LDS it knows of with a wait for every load
+// (it counts such a load as one that may come back out of order), which empties the pipeline; a load it
+// does not know of it does not wait for, and the kernel waits itself, by count. `lds_byte` is the same
+// for the whole wave.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void load_to_lds_uncounted(const bf16_t* src, unsigned lds_byte) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(src), "s"(lds_byte)
+                 : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
 // TMI, TN: MFMA tiles of 32x32 down a wave's part of the activation rows and across its part of
 // the weight rows; NWM, NWN: waves down and across (eight in all). The launcher's plan chooses
 // the tile so that the blocks come out in whole rounds of the CUs.
-template <typename TOut, int TMI, int TN, int NWN, int NWM = 2>
+template <typename TOut, int TMI, int TN, int NWN, int NWM = 2, int STAGES = 2>
 __global__ __launch_bounds__(64 * NWM * NWN) void k_gemm_bf16_dma(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                              const float* __restrict__ bias, TOut* __restrict__ Y,
                                                              int M, int N, int K_all, int k_per, int tiles_m,
@@ -582,6 +597,10 @@ __global__ __launch_bounds__(64 * NWM * NWN) void k_gemm_bf16_dma(const bf16_t* 
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "the waves share the tile's rows evenly");
     __shared__ __attribute__((aligned(1024))) bf16_t stage0[(BM + BN) * DM_BK];   // X rows, then W rows
     __shared__ __attribute__((aligned(1024))) bf16_t stage1[(BM + BN) * DM_BK];
+    // four stages (a block alone on its CU): the loads of three K-steps in flight while one is multiplied
+    static_assert(STAGES == 2 || STAGES == 4, "two stages or four");
+    __shared__ __attribute__((aligned(1024))) bf16_t stage2[STAGES == 4 ? (BM + BN) * DM_BK : 8];
+    __shared__ __attribute__((aligned(1024))) bf16_t stage3[STAGES == 4 ? (BM + BN) * DM_BK : 8];
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + N_XCD - 1) / N_XCD;
     const int logical = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;
@@ -616,6 +635,15 @@ __global__ __launch_bounds__(64 * NWM * NWN) void k_gemm_bf16_dma(const bf16_t* 
     auto load_step = [&](bf16_t* stage, int kt) __attribute__((always_inline)) {
         const bf16_t* xk = X + (size_t)kt * DM_BK;
         const bf16_t* wk = W + (size_t)kt * DM_BK;
+        if (STAGES == 4) {
+            const unsigned to = __builtin_amdgcn_readfirstlane(
+                (unsigned)(size_t)(__attribute__((address_space(3))) bf16_t*)stage + wave * 8 * DM_BK * 2);
+#pragma unroll
+            for (int j = 0; j < LX; ++j) load_to_lds_uncounted(xk + off_x[j], to + j * 8 * NW * DM_BK * 2);
+#pragma unroll
+            for (int j = 0; j < LW; ++j) load_to_lds_uncounted(wk + off_w[j], to + (BM + j * 8 * NW) * DM_BK * 2);
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < LX; ++j) load_to_lds(xk + off_x[j], stage + (j * 8 * NW + wave * 8) * DM_BK);
 #pragma unroll
@@ -651,8 +679,8 @@ __global__ __launch_bounds__(64 * NWM * NWN) void k_gemm_bf16_dma(const bf16_t* 
     const int nk = K / DM_BK;
     Frag8 fa0[TMI], fb0[TN], fa1[TMI], fb1[TN];
     // K-step kt from `cur`: on entry set 0 holds its first sub-step and the loads of step kt+1
-    // into `next` are in flight; on exit set 0 holds the first sub-step of kt+1 and the loads
-    // of kt+2 into `cur` are in flight
+    // into `next` are in flight (and with four stages those of kt+2 and kt+3); on exit set 0 holds
+    // the first sub-step of kt+1 and the loads of kt+STAGES into `cur` are in flight
     auto k_step = [&](bf16_t* cur, bf16_t* next, int kt) __attribute__((always_inline)) {
         // (the scheduling barriers keep each sub-step's reads and products where they are written:
         // left alone, the compiler sinks the loads of the next step to just before the wait for them)
@@ -665,9 +693,15 @@ __global__ __launch_bounds__(64 * NWM * NWN) void k_gemm_bf16_dma(const bf16_t* 
         read(cur, 3, fa1, fb1);
         multiply(fa0, fb0);
         __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();               // this wave's part of `next` has landed and `cur` is read; so for every wave
+        // this wave's part of `next` has landed and `cur` is read; after the barrier, so for every wave
+        if (STAGES == 4) {             // the loads of the two steps after `next` stay in flight: a bare barrier
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * (LX + LW)) : "memory");
+            __builtin_amdgcn_s_barrier();
+        } else {
+            __syncthreads();
+        }
         read(next, 0, fa0, fb0);
-        load_step(cur, min(kt + 2, nk - 1));      // past the end: the last step again, into a stage nobody reads any more
+        load_step(cur, min(kt + STAGES, nk - 1));   // past the end: the last step again, into a stage nobody reads any more
         multiply(fa1, fb1);
 #pragma unroll
         for (int q = 0; q < TMI * TN; ++q) {        // one product, (one fragment read,) one load or two
@@ -680,13 +714,30 @@ __global__ __launch_bounds__(64 * NWM * NWN) void k_gemm_bf16_dma(const bf16_t* 
         }
         __builtin_amdgcn_sched_barrier(0);
     };
-    load_step(stage0, 0);
-    __syncthreads();
-    load_step(stage1, 1);
-    read(stage0, 0, fa0, fb0);
-    for (int kt = 0; kt < nk; kt += 2) {               // an even number of K-steps: one loop, one way round it
-        k_step(stage0, stage1, kt);
-        k_step(stage1, stage0, kt + 1);
+    if (STAGES == 4) {
+        load_step(stage0, 0);
+        load_step(stage1, 1);
+        load_step(stage2, 2);
+        load_step(stage3, 3);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (LX + LW)) : "memory");
+        __builtin_amdgcn_s_barrier();
+        read(stage0, 0, fa0, fb0);
+        for (int kt = 0; kt < nk; kt += 4) {           // K-steps in fours: one loop, one way round it
+            k_step(stage0, stage1, kt);
+            k_step(stage1, stage2, kt + 1);
+            k_step(stage2, stage3, kt + 2);
+            k_step(stage3, stage0, kt + 3);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the loads past the end: nothing may land in what the tile leaves through
+    } else {
+        load_step(stage0, 0);
+        __syncthreads();
+        load_step(stage1, 1);
+        read(stage0, 0, fa0, fb0);
+        for (int kt = 0; kt < nk; kt += 2) {           // an even number of K-steps: one loop, one way round it
+            k_step(stage0, stage1, kt);
+            k_step(stage1, stage0, kt + 1);
+        }
     }
     // The tile leaves through LDS, a wave's 32 rows x 128 columns at a time (one row of its MFMA
     // tiles): the wave writes the accumulators as the matrix pipe left them, reads whole rows
@@ -756,27 +807,31 @@ static bool dma_tile_takes(int m, int n, int k) {
 }
 
 // Which tile (bm = 256 or 128 activation rows, tn = 4, 3, 2 for 256, 192, 128 weight rows; 192 with
-// bm 256 only) and how many slices of K suit a product of many rows; tn = 0: none (a K the kernel
-// does not take). A model of the time, fitted to this machine (it picks the fastest or one within
-// a few percent of it on every shape measured, 128 to 4,096 rows):
-//   - a block alone on its CU takes 0.11 us + 0.0155 us per MFMA of a SIMD for a K-step of 64
-//     (bm * bn / 1024 of them), and 5 us + 0.03 us per such MFMA for its beginning and end;
-//   - two blocks fit a CU where their stages take 80 KB or less each (the 128x128 tile), and a
-//     step then takes what the products of both take;
-//   - the more CUs are busy the slower each runs (clocks, L2): up to 45% with all 256, and more
-//     with small tiles, which read more operand bytes per product;
+// bm 256 only), on how many stages, and how many slices of K suit a product of many rows; tn = 0:
+// none (a K the kernel does not take). A model of the time, fitted to this machine over 128 to 8,192
+// rows and seven weight shapes, every tile and 1 to 8 slices measured (what it picks is within 1 % of
+// the fastest on average and within 7 % on every shape whose consumer can add slices):
+//   - a K-step of 64 takes a block alone on its CU the first figure below with few CUs busy and the
+//     second with all 256 (clocks, L2), in between in proportion:
+//         128x128 0.46 .. 0.78 us    128x256 0.70 .. 1.08    256x128 0.66 .. 1.08
+//         256x192 0.89 .. 1.30       256x256 1.03 .. 1.58
+//   - two blocks fit a CU where their stages take 80 KB or less each (the 128x128 tile on two
+//     stages); a step of both then takes 1.09 us, and with two on some CUs only, in between;
+//   - the 128x128 tile can instead keep four stages (one block a CU, three steps' loads in flight):
+//     0.33 .. 0.53 us a step, which pays where the tiles are one round of the CUs or less;
 //   - with one or two tiles down the rows (a decode batch of 65 to 256 rows) every block meets its
-//     weights first, and cold: a K-step then takes 1 us whatever the tile (measured: 32 us for 32
-//     steps at 128 rows), so such products gain most from many slices (up to 8);
+//     weights first, and cold: a step then takes 0.55 us at least on two stages and 0.36 on four;
+//   - a block's beginning and end take 4.3 us + 0.116 us per MFMA of a SIMD in a K-step
+//     (bm * bn / 1024 of them);
 //   - blocks run in rounds of what fits the chip at once; the operands have to come from memory
-//     once (5.5 TB/s) and the results have to go there (5 TB/s); a slice beyond the first costs
-//     its consumer one more pass over rows x width of float32.
+//     once (5.5 TB/s) and the results have to go there (7.6 TB/s); a slice beyond the first costs
+//     its consumer one more pass over rows x width of float32 (5 TB/s).
 // `fixed_slices` > 0: the caller has decided (1: its consumer cannot add slices).
 struct DmaPlan {
-    int bm, tn, slices;
+    int bm, tn, slices, stages;
 };
 static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
-    DmaPlan best{0, 0, fixed_slices > 0 ? fixed_slices : 1};
+    DmaPlan best{0, 0, fixed_slices > 0 ? fixed_slices : 1, 2};
     if (m <= 64 || !dma_tile_takes(m, n, k)) return best;
     double best_cost = 0.0;
     for (int slices : {1, 2, 3, 4, 6, 8}) {                 // (3 and 6: a K of 27 or 9 times 256 has no other cut)
@@ -787,24 +842,31 @@ static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
             for (int tn = 4; tn >= 2; --tn) {
                 if (tn == 3 && bm != 256) continue;
                 const int bn = 64 * tn;
-                const long long blocks = (long long)tiles_m * ((n + bn - 1) / bn) * slices;
-                const int at_once = 256 * ((bm + bn) * DM_BK * 2 * 2 <= 80 * 1024 ? 2 : 1);
-                const long long rounds = (blocks + at_once - 1) / at_once;
-                const long long per_round = (blocks + rounds - 1) / rounds;
-                const double cus = (double)std::min<long long>(256, per_round);
-                const double per_cu = (double)((per_round + (long long)cus - 1) / (long long)cus);
-                const double mfmas = bm * bn / 1024.0;
-                const double small = 1.0 + 0.1 * (256.0 / bm - 1.0) + 0.1 * (256.0 / bn - 1.0);
-                double step = std::max(0.11 + 0.0155 * mfmas, per_cu * 0.0155 * mfmas) *
-                              (1.0 + 0.45 * cus / 256.0 * small);
-                if (tiles_m <= 2) step = std::max(step, 1.0);     // nobody has read these weights before: memory is far
-                const double ends = 5.0 + 0.03 * mfmas;
-                const double from_memory = ((double)m + n) * k * 2.0 / 5.5e6;
-                const double cost = std::max(rounds * (k / slices / DM_BK * step + ends), from_memory + ends) +
-                                    (double)slices * m * n * 4.0 / 5e6 + (slices - 1) * ((double)m * n * 4.0 / 5e6);
-                if (best.tn == 0 || cost < best_cost) {
-                    best = DmaPlan{bm, tn, slices};
-                    best_cost = cost;
+                for (int stages = 2; stages <= 4; stages += 2) {
+                    // four stages: the 128x128 tile, K-steps in fours
+                    if (stages == 4 && (bm != 128 || tn != 2 || (k / slices) % (4 * DM_BK) != 0)) continue;
+                    const long long blocks = (long long)tiles_m * ((n + bn - 1) / bn) * slices;
+                    const int at_once = 256 * ((bm + bn) * DM_BK * 2 * stages <= 80 * 1024 ? 2 : 1);
+                    const long long rounds = (blocks + at_once - 1) / at_once;
+                    const long long per_round = (blocks + rounds - 1) / rounds;
+                    const double cus = (double)std::min<long long>(256, per_round);
+                    double few, all;
+                    if (bm == 128 && tn == 2) few = stages == 4 ? 0.33 : 0.46, all = stages == 4 ? 0.53 : 0.78;
+                    else if (bm == 128) few = 0.70, all = 1.08;
+                    else if (tn == 2) few = 0.66, all = 1.08;
+                    else if (tn == 3) few = 0.89, all = 1.30;
+                    else few = 1.03, all = 1.58;
+                    double step = per_round > 256 ? all + (1.09 - all) * (per_round - 256) / 256.0    // some CUs, or all, with two
+                                                  : few + (all - few) * cus / 256.0;
+                    if (tiles_m <= 2) step = std::max(step, stages == 4 ? 0.36 : 0.55);
+                    const double ends = 4.3 + 0.116 * (bm * bn / 1024.0);
+                    const double from_memory = ((double)m + n) * k * 2.0 / 5.5e6;
+                    const double cost = std::max(rounds * (k / slices / DM_BK * step + ends), from_memory + ends) +
+                                        (double)slices * m * n * 4.0 / 7.6e6 + (slices - 1) * ((double)m * n * 4.0 / 5e6);
+                    if (best.tn == 0 || cost < best_cost) {
+                        best = DmaPlan{bm, tn, slices, stages};
+                        best_cost = cost;
+                    }
                 }
             }
         }
@@ -816,7 +878,7 @@ static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
 // bm: 256 or 128 activation rows to a tile; tn: 4, 3 (bm 256 only) or 2 for 256, 192 or 128 weight rows.
 template <typename TOut>
 static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
-                      int bm, int tn, int slices, hipStream_t s) {
+                      int bm, int tn, int slices, hipStream_t s, int stages = 2) {
     const int tiles_m = (m + bm - 1) / bm, tiles_n = (n + 64 * tn - 1) / (64 * tn);
     const long long total = (long long)tiles_m * tiles_n;
     const dim3 grid((unsigned)(((total + N_XCD - 1) / N_XCD) * N_XCD), (unsigned)slices);
@@ -825,6 +887,8 @@ static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TOut*
                                                                    tiles_n, epilogue)
     if (bm == 128 && tn == 4)
         DMA_GO(2, 2, 4);
+    else if (bm == 128 && stages == 4)
+        k_gemm_bf16_dma<TOut, 2, 1, 4, 2, 4><<<grid, 512, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
     else if (bm == 128)
         DMA_GO(2, 1, 4);
     else if (tn == 4)     // 256 wide: eight waves
@@ -1390,7 +1454,8 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
         // `force` (for measurements) 256: the 256x256 tile with register staging
         if (force == 0) {
             const DmaPlan plan = dma_plan(m, n, k, slices);
-            if (plan.tn) return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, plan.bm, plan.tn, slices, s);
+            if (plan.tn)
+                return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, plan.bm, plan.tn, slices, s, plan.stages);
         }
         if (slices == 1 && (force == 256 || (force == 0 && big_tile_pays(m, n, k))))
             return launch_big<TOut, 2, 4, 4, 2>(x, w, bias, y, m, n, k, epilogue, s);
@@ -1398,9 +1463,11 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
         if ((force == 258 || force == 262 || force == 263) && k % slices == 0 && dma_tile_takes(m, n, k / slices) &&
             dma_tile_takes(m, n, k))
             return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, 256, force == 258 ? 4 : force - 260, slices, s);
-        // 358, 352: 128 activation rows to a tile, 256 and 128 wide
+        // 358, 352: 128 activation rows to a tile, 256 and 128 wide; 452: 128 by 128 on four stages
         if ((force == 358 || force == 352) && k % slices == 0 && dma_tile_takes(m, n, k / slices) && dma_tile_takes(m, n, k))
             return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, 128, force == 358 ? 4 : 2, slices, s);
+        if (force == 452 && k % slices == 0 && (k / slices) % (4 * DM_BK) == 0 && dma_tile_takes(m, n, k))
+            return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, 128, 2, slices, s, 4);
         const int tiles_m = (m + BG_BM - 1) / BG_BM, tiles_n = (n + BG_BN - 1) / BG_BN;
         const long long total = (long long)tiles_m * tiles_n;
         if (total > 0x7fffff00LL) return IMPARO_BAD_ARGUMENT;
@@ -1417,7 +1484,7 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
 // that each kernel can be met at any shape: 1 the K-split kernel, 2, 4 or 8 the shared-activation
 // kernel with that many waves, 256 the 256x256 tile with register staging, 258 / 263 / 262 the tile
 // with loads straight into LDS at 256 rows by 256 / 192 / 128, 358 / 352 the same at 128 rows by
-// 256 / 128; with a variant, any number of K slices is taken.
+// 256 / 128, 452 the 128 by 128 tile on four stages; with a variant, any number of K slices is taken.
 static int gemm_variant(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
                         int m, int n, int k, int epilogue, int slices, int variant, imparo_stream stream) {
     if (!x || !w || !y || m < 0 || n <= 0 || k <= 0) return IMPARO_BAD_ARGUMENT;

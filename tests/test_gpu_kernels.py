@@ -156,7 +156,8 @@ def test_gemm_with_many_weight_rows(m, k):
 @pytest.mark.parametrize("m,n,k,tile", [(2600, 3900, 256, 0), (2600, 3904, 1152, 0), (3900, 4002, 384, 0),
                                         (1500, 3900, 640, 0), (2600, 3904, 200, 0), (70, 100, 128, 0),
                                         (700, 1000, 384, 258), (700, 1000, 384, 262), (700, 1000, 384, 263),
-                                        (700, 1000, 384, 358), (700, 1000, 384, 352)])
+                                        (700, 1000, 384, 358), (700, 1000, 384, 352),
+                                        (700, 1000, 256, 452), (700, 1000, 1280, 452), (130, 250, 2048, 452)])
 def test_gemm_with_large_tiles(m, n, k, tile):
     """Many rows: K a multiple of 128 goes to the kernel that loads straight into LDS, with a tile
     of 256 or 128 rows by 256, 192 or 128 weight rows, whichever its plan finds fastest (`tile`
@@ -185,9 +186,11 @@ def _large_tile_case(m, n, k, variant=0):
     assert torch.equal(outb.cpu(), out.cpu().to(torch.bfloat16))
 
 
-@pytest.mark.parametrize("m,n,k,slices", [(1900, 2000, 8192, 2), (1000, 2000, 8192, 4), (1900, 2100, 4096, 2)])
+@pytest.mark.parametrize("m,n,k,slices", [(1000, 2000, 8192, 2), (500, 2000, 8192, 4), (4000, 2000, 8192, 2),
+                                          (300, 2000, 4096, 4)])
 def test_gemm_with_large_tiles_in_slices_of_k(m, n, k, slices):
-    """Few tiles and a long K: slices of K on the large tiles, as many as give one block per CU."""
+    """Few tiles and a long K: slices of K on the large tiles, as many as the plan's model of the time finds
+    fastest (on two stages or on four)."""
     assert ops().gemm_slices(m, n, k, torch.bfloat16) == slices
     x, w, b = rnd(m, k, seed=1, scale=0.5).to(torch.bfloat16), rnd(n, k, seed=2, scale=0.3).to(torch.bfloat16), rnd(n, seed=3)
     y = x.float() @ w.float().t() + b
