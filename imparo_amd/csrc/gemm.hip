@@ -1430,6 +1430,9 @@ template <typename TOut>
 static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
                        int force, int slices, hipStream_t s) {
     // `force` (for measurements): 1 = K-split kernel, 2/4/8 = shared activations with that many waves
+    // 452: the 128 by 128 tile on four stages, at any number of rows
+    if (force == 452 && k % slices == 0 && (k / slices) % (4 * DM_BK) == 0 && dma_tile_takes(m, n, k))
+        return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, 128, 2, slices, s, 4);
     int nw = stream_waves(m, n, k);
     if (force == 1) nw = 0;
     if (force == 2 || force == 4 || force == 8) nw = force;
@@ -1463,11 +1466,9 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
         if ((force == 258 || force == 262 || force == 263) && k % slices == 0 && dma_tile_takes(m, n, k / slices) &&
             dma_tile_takes(m, n, k))
             return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, 256, force == 258 ? 4 : force - 260, slices, s);
-        // 358, 352: 128 activation rows to a tile, 256 and 128 wide; 452: 128 by 128 on four stages
+        // 358, 352: 128 activation rows to a tile, 256 and 128 wide
         if ((force == 358 || force == 352) && k % slices == 0 && dma_tile_takes(m, n, k / slices) && dma_tile_takes(m, n, k))
             return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, 128, force == 358 ? 4 : 2, slices, s);
-        if (force == 452 && k % slices == 0 && (k / slices) % (4 * DM_BK) == 0 && dma_tile_takes(m, n, k))
-            return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, 128, 2, slices, s, 4);
         const int tiles_m = (m + BG_BM - 1) / BG_BM, tiles_n = (n + BG_BN - 1) / BG_BN;
         const long long total = (long long)tiles_m * tiles_n;
         if (total > 0x7fffff00LL) return IMPARO_BAD_ARGUMENT;
