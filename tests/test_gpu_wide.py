@@ -57,12 +57,13 @@ def _logits_at(plain, tokens, rows):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("live", [24, 64])
+@pytest.mark.parametrize("live", [24, 64, 100])
 def test_many_decoding_requests_at_benchmark_width(wide, dtype, live):
-    """24 and 64 live requests of different contexts decode six tokens each, every row held
+    """24, 64 and 100 live requests of different contexts decode six tokens each, every row held
     to the plain implementation: the step run launch by launch, the captured one and its
     replays. Beyond 16 rows the few-row products take more weight rows a block, the conv
-    mixer takes two launches instead of the fused one, and the captured graph is another."""
+    mixer takes two launches instead of the fused one, and the captured graph is another;
+    beyond 64 rows the products go to the tile kernels, in slices of K."""
     from imparo_amd.engine import StepEntry
     d, _, _, plain = wide
     rng = random.Random(live)
