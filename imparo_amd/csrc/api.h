@@ -42,6 +42,9 @@ int imparo_rms_norm(float* x, const float* delta, int n_delta, int n_x_rows, con
 int imparo_gemm(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
                 int m, int n, int k, int epilogue, int slices, imparo_stream stream);
 int imparo_gemm_slices(int m, int n, int k, int dtype);
+// epilogue 2 (float32 out, `slices` 1): Y[m, n] += the product (+ bias), each element of Y read where it
+// is stored. Only for shapes for which imparo_gemm_adds gives 1 (many rows, a K the tile kernel takes).
+int imparo_gemm_adds(int m, int n, int k, int dtype);
 // imparo_gemm with the kernel named by the caller instead of chosen by the library: for tests and
 // measurements, so that every kernel can be met at any shape (the numbers are listed in gemm.hip).
 // Nothing in the library keeps the choice: it is this call's argument.

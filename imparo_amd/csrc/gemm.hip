@@ -22,6 +22,7 @@ union Frag8 {
 
 #define EPI_NONE 0
 #define EPI_SWIGLU 1   // weight rows interleaved gate, up, gate, up...: out[m, j] = silu(y[m, 2j]) * y[m, 2j+1]
+#define EPI_ADD 2      // float32 out only: Y += y, what Y holds being read where the result is stored
 
 __device__ __forceinline__ float silu_mul_f(float g, float u) { return g / (1.0f + expf(-g)) * u; }
 // The same with the hardware's exp2 and reciprocal (an ulp each) for the bfloat16 kernels: the exact
@@ -544,6 +545,14 @@ static int launch_big(const bf16_t* x, const bf16_t* w, const float* bias, TOut*
 // work queued while the waves meet. Needs K a multiple of 128 (two K-steps).
 #define DM_BK 64
 
+// What the output holds where four results of a row will go (the epilogue that adds; float32 out only)
+template <typename T> __device__ __forceinline__ float4 held_vector(const T*) { return make_float4(0.f, 0.f, 0.f, 0.f); }
+template <> __device__ __forceinline__ float4 held_vector<float>(const float* dst) {
+    return *reinterpret_cast<const float4*>(dst);
+}
+template <typename T> __device__ __forceinline__ float held_f32(const T*, int) { return 0.f; }
+template <> __device__ __forceinline__ float held_f32<float>(const float* dst, int c) { return dst[c]; }
+
 // Two (`pair`) or four outputs of one row in one store; the address is aligned to the store
 template <typename T> __device__ __forceinline__ void store_vector(T* dst, const float (&o)[4], bool pair);
 template <> __device__ __forceinline__ void store_vector<float>(float* dst, const float (&o)[4], bool pair) {
@@ -761,6 +770,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void k_gemm_bf16_dma(const bf16_t* 
             if (n + c < N) bn[c] = bias[n + c];
     }
     const bool swiglu = epilogue == EPI_SWIGLU;
+    const bool adds = epilogue == EPI_ADD;             // (float32 out; the launcher sees to it)
     const int out_n = swiglu ? N / 2 : N;              // columns of Y
     const int per_lane = swiglu ? 2 : 4;               // outputs a lane holds of a row
     // whole vectors: every row of this tile inside, the lane's columns inside, rows of Y aligned
@@ -786,6 +796,10 @@ __global__ __launch_bounds__(64 * NWM * NWN) void k_gemm_bf16_dma(const bf16_t* 
             }
             TOut* dst = Y + (size_t)m * out_n + (swiglu ? n / 2 : n);
             if (vectors) {
+                if (adds) {
+                    const float4 held = held_vector<TOut>(dst);
+                    o[0] = held.x + o[0], o[1] = held.y + o[1], o[2] = held.z + o[2], o[3] = held.w + o[3];
+                }
                 store_vector<TOut>(dst, o, swiglu);
             } else if (m < M) {
                 if (swiglu) {
@@ -794,7 +808,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void k_gemm_bf16_dma(const bf16_t* 
                 } else {
 #pragma unroll
                     for (int c = 0; c < 4; ++c)
-                        if (n + c < N) store_f32<TOut>(dst, c, o[c]);
+                        if (n + c < N) store_f32<TOut>(dst, c, adds ? held_f32<TOut>(dst, c) + o[c] : o[c]);
                 }
             }
         }
@@ -1249,6 +1263,12 @@ extern "C" int imparo_gemm_slices(int m, int n, int k, int dtype) {
     return whole_slices(slices, k, 128);
 }
 
+// Whether imparo_gemm takes the epilogue that adds the product to what Y holds (float32 out, K in one
+// piece) for this shape: where the tile kernel with loads straight into LDS runs it.
+extern "C" int imparo_gemm_adds(int m, int n, int k, int dtype) {
+    return dtype == IMPARO_BF16 && m > 64 && dma_plan(m, n, k, 1).tn != 0;
+}
+
 // ------------------------------------------------------------------ bfloat16, some rows (17..64)
 // A block of ST_WAVES waves takes 16 weight rows per wave and up to 16*MT
 // activation rows, and walks its part of K in chunks of 128. The activation
@@ -1494,8 +1514,11 @@ static int gemm_variant(const void* x, const void* w, const float* bias, void* y
     const int slices_ok = imparo_gemm_slices(m, n, k, dtype);
     if (slices > 1 && ((slices != slices_ok && variant == 0) || out_dtype != IMPARO_F32 || epilogue != EPI_NONE))
         return IMPARO_BAD_ARGUMENT;
-    if (epilogue != EPI_NONE && epilogue != EPI_SWIGLU) return IMPARO_BAD_ARGUMENT;
+    if (epilogue != EPI_NONE && epilogue != EPI_SWIGLU && epilogue != EPI_ADD) return IMPARO_BAD_ARGUMENT;
     if (epilogue == EPI_SWIGLU && (n % 2 != 0)) return IMPARO_BAD_ARGUMENT;
+    // adding into Y: the tile kernel that loads straight into LDS only, chosen by the library, K in one piece
+    if (epilogue == EPI_ADD && (variant != 0 || slices != 1 || out_dtype != IMPARO_F32 || !imparo_gemm_adds(m, n, k, dtype)))
+        return IMPARO_BAD_ARGUMENT;
     if (m == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;
     if (dtype == IMPARO_F32) {

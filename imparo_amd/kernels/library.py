@@ -26,6 +26,7 @@ _SIGNATURES = {
     "imparo_rms_norm": [P, P, I, I, P, P, P, I, I, I, F, I, P],
     "imparo_gemm": [P, P, P, P, I, I, I, I, I, I, I, P],
     "imparo_gemm_slices": [I, I, I, I],
+    "imparo_gemm_adds": [I, I, I, I],
     "imparo_gemm_variant": [P, P, P, P, I, I, I, I, I, I, I, I, P],
     "imparo_short_conv_decode": [P, P, P, P, P, P, I, I, I, I, I, P],
     "imparo_in_proj_conv_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],

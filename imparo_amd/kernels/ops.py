@@ -132,12 +132,18 @@ def gemm_slices(m: int, n: int, k: int, dtype: torch.dtype) -> int:
     return int(library().imparo_gemm_slices(m, n, k, _CODES.get(dtype, -1)))
 
 
+def gemm_adds(m: int, n: int, k: int, dtype: torch.dtype) -> bool:
+    """Whether `gemm(..., add=True)` is taken for this shape (many rows on the tile kernel, K in one piece)."""
+    return bool(library().imparo_gemm_adds(m, n, k, _CODES.get(dtype, -1)))
+
+
 def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
-         swiglu: bool = False, variant: int = 0) -> torch.Tensor:
+         swiglu: bool = False, variant: int = 0, add: bool = False) -> torch.Tensor:
     """out[m, n] = x[m, k] . w[n, k]^T (+ bias[n]); x and w share a dtype; float32
     accumulate. With `swiglu` the rows of w alternate gate and up and out is
     [m, n/2] = silu(gate) * up. An `out` of shape [slices, m, n] (slices =
     gemm_slices(...)) receives the sums over slices of K, to be added by the consumer.
+    With `add` (float32 out, where gemm_adds(...) says so) the product is added to what `out` holds.
     `variant` other than 0 names the kernel (tests and measurements only; see imparo_gemm_variant)."""
     m, k = x.shape
     n, kw = w.shape
@@ -157,8 +163,10 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[tor
         _dev(out, "gemm out", torch.float32, (slices, m, n))
     else:
         _dev(out, "gemm out", None, (m, n // 2 if swiglu else n))
+    if add and (swiglu or slices != 1 or variant or out.dtype != torch.float32 or not gemm_adds(m, n, k, x.dtype)):
+        raise KernelArgumentError("gemm: this product cannot be added to what its output holds")
     args = (_dev(x, "gemm x"), _dev(w, "gemm weight"), _dev(bias, "gemm bias", torch.float32, (n,)),
-            out.data_ptr(), _code(x, "gemm x"), _code(out, "gemm out"), m, n, k, int(swiglu), slices)
+            out.data_ptr(), _code(x, "gemm x"), _code(out, "gemm out"), m, n, k, 2 if add else int(swiglu), slices)
     if variant:
         _check(library().imparo_gemm_variant(*args, int(variant), _stream()), "gemm")
     else:

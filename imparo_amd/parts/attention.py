@@ -125,7 +125,7 @@ class Attention:
                                      part_o, part_ml, ctx.single_rows, ctx.n_single_rows, ctx.seg_start,
                                      ctx.positions, table, self.heads, self.scale, self.window, ctx.max_context,
                                      interleaved=interleaved)
-            return self.out(ctx, o, torch.float32, "mixer_out", sliced_ok=True)
+            return self.out(ctx, o, torch.float32, "mixer_out", sliced_ok=True, into=ctx.stream)
         q = ctx.workspace.get("q", (T, self.heads, self.head_dim), ctx.dtype)
         ops.qk_norm_rope_store(qkv, self.q_norm, self.k_norm, self.norm_eps, inv_freq,
                                ctx.positions, ctx.row_of_token, table if owns_cache else None, ctx.page_size,
@@ -157,7 +157,7 @@ class Attention:
         if o.dtype != self.out.in_dtype:
             raise ValueError("the output projection's weight dtype differs from the attention output's")
         # a delta for the residual stream: the next norm adds slices, so it may come sliced
-        return self.out(ctx, o, torch.float32, "mixer_out", sliced_ok=True)
+        return self.out(ctx, o, torch.float32, "mixer_out", sliced_ok=True, into=ctx.stream)
 
 
 register_part("mixer", "attention", Attention)

@@ -96,6 +96,9 @@ class StepContext:
     n_portion_rows: int = 0
     host_seg_len: Optional[Sequence[int]] = None
     memo: Dict[object, object] = field(default_factory=dict)   # what parts derive from the batch, once a step
+    # The float32 residual stream while a block runs the part whose result goes into it, with nothing pending
+    # on it: the part may add its result there itself and return the stream instead of a delta. None: return a delta.
+    stream: Optional[torch.Tensor] = None
 
     def paged(self, site: int):
         """The site's paged arrays by name, and the block table of its group."""

@@ -28,9 +28,20 @@ class PreNormBlock:
 
     def forward(self, ctx: StepContext, res: Residual, site: int, owns_cache: bool) -> None:
         h = self.mixer_norm.forward(ctx, res, self.mixer.in_dtype)
-        res.pending = self.mixer.forward(ctx, site, owns_cache, h)
+        res.pending = self._delta(ctx, res, lambda: self.mixer.forward(ctx, site, owns_cache, h))
         n = self.ffn_norm.forward(ctx, res, self.ffn.in_dtype)
-        res.pending = self.ffn.forward(ctx, n)
+        res.pending = self._delta(ctx, res, lambda: self.ffn.forward(ctx, n))
+
+    @staticmethod
+    def _delta(ctx: StepContext, res: Residual, run):
+        """Runs a part whose result goes into the stream. With nothing pending the part may add its
+        result to the stream itself (it then returns the stream); otherwise it returns a delta."""
+        ctx.stream = res.x if res.pending is None else None
+        try:
+            delta = run()
+        finally:
+            ctx.stream = None
+        return None if delta is res.x else delta
 
 
 register_part("block", "pre_norm", PreNormBlock)

@@ -65,7 +65,7 @@ class SwiGlu:
         # the gated hidden may lie where the mixer's input projection lay: that is dead by now
         g = self.gate_up(ctx, n, self.down.in_dtype, "gated", swiglu=True, alias="mixer_in")
         # the result is a delta for the residual stream, whose next norm adds slices: it may come sliced
-        return self.down(ctx, g, torch.float32, "ffn_out", sliced_ok=True)
+        return self.down(ctx, g, torch.float32, "ffn_out", sliced_ok=True, into=ctx.stream)
 
 
 register_part("feed_forward", "swiglu", SwiGlu)

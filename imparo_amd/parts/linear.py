@@ -28,12 +28,15 @@ class Linear:
         return self.weight.dtype
 
     def __call__(self, ctx: StepContext, x: torch.Tensor, out_dtype: torch.dtype, name: str,
-                 swiglu: bool = False, sliced_ok: bool = False, alias: Optional[str] = None) -> torch.Tensor:
+                 swiglu: bool = False, sliced_ok: bool = False, alias: Optional[str] = None,
+                 into: Optional[torch.Tensor] = None) -> torch.Tensor:
         """`swiglu`: the weight's rows alternate gate and up; the output is
         silu(gate) * up, half as wide. `sliced_ok`: the caller's consumer adds
         slices, so the result may come as [slices, rows, out] sums over parts
         of K (few rows and a long K keep more of the chip busy that way).
-        `alias`: the workspace group the output may share memory with."""
+        `alias`: the workspace group the output may share memory with.
+        `into`: a float32 [rows, out] tensor the result may be added to instead
+        (the residual stream); where the kernels do that, `into` itself is returned."""
         width = self.out_features // 2 if swiglu else self.out_features
         m = x.shape[0]
         if sliced_ok and not swiglu and out_dtype == torch.float32:
@@ -41,6 +44,11 @@ class Linear:
             if slices > 1:
                 out = ctx.workspace.get(name + "_sliced", (slices, m, width), out_dtype)
                 return ops.gemm(x, self.weight, out, bias=self.bias)
+        if (into is not None and not swiglu and out_dtype == torch.float32 and into.dtype == torch.float32
+                and tuple(into.shape) == (m, width) and into.is_contiguous()
+                and ops.gemm_adds(m, self.out_features, self.in_features, self.weight.dtype)):
+            # one pass less over the rows for the norm that follows: the product's epilogue reads and writes the stream
+            return ops.gemm(x, self.weight, into, bias=self.bias, add=True)
         out = ctx.workspace.get(name, (m, width), out_dtype, alias=alias)
         return ops.gemm(x, self.weight, out, bias=self.bias, swiglu=swiglu)
 

@@ -71,12 +71,12 @@ class ShortConv:
             # a decode step's few rows: projection and conv in one launch
             ops.in_proj_conv_decode(h, self.in_proj.weight, self.in_proj.bias, self.conv_weight, self.conv_bias,
                                     ctx.fixed_state(site), ctx.slot, y)
-            return self.out_proj(ctx, y, torch.float32, "mixer_out", sliced_ok=True)
+            return self.out_proj(ctx, y, torch.float32, "mixer_out", sliced_ok=True, into=ctx.stream)
         bcx = self.in_proj(ctx, h, torch.float32, "bcx", alias="mixer_in")
         ops.short_conv(bcx, self.conv_weight, self.conv_bias, ctx.fixed_state(site), ctx.row_of_token,
                        ctx.seg_start, ctx.seg_len, ctx.slot, y, single_tokens=ctx.max_seg_len == 1)
         # a delta for the residual stream: the next norm adds slices, so it may come sliced
-        return self.out_proj(ctx, y, torch.float32, "mixer_out", sliced_ok=True)
+        return self.out_proj(ctx, y, torch.float32, "mixer_out", sliced_ok=True, into=ctx.stream)
 
 
 register_part("mixer", "short_conv", ShortConv)

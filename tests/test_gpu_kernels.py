@@ -186,6 +186,28 @@ def _large_tile_case(m, n, k, variant=0):
     assert torch.equal(outb.cpu(), out.cpu().to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("m,n,k", [(700, 1000, 384), (2048, 2048, 2048), (130, 250, 1024), (1500, 3902, 640)])
+def test_gemm_added_to_what_the_output_holds(m, n, k):
+    """The epilogue that adds: bit for bit what adding the plain product afterwards gives, at the
+    tiles' edges too; refused where the tile kernel does not run the product."""
+    from imparo_amd.kernels import KernelArgumentError
+    x, w, b = rnd(m, k, seed=1, scale=0.5).to(torch.bfloat16), rnd(n, k, seed=2, scale=0.3).to(torch.bfloat16), rnd(n, seed=3)
+    assert ops().gemm_adds(m, n, k, torch.bfloat16)
+    held = rnd(m, n, seed=4).to(DEV)
+    plain = torch.full((m, n), float("nan"), device=DEV)
+    ops().gemm(x.to(DEV), w.to(DEV), plain, bias=b.to(DEV)) if ops().gemm_slices(m, n, k, torch.bfloat16) == 1 else None
+    out = held.clone()
+    ops().gemm(x.to(DEV), w.to(DEV), out, bias=b.to(DEV), add=True)
+    y = x.float() @ w.float().t() + b
+    assert (out.cpu() - (held.cpu() + y)).abs().max() <= 4e-6 * math.sqrt(k) * float(y.abs().max())
+    if ops().gemm_slices(m, n, k, torch.bfloat16) == 1:
+        assert torch.equal(out, held + plain)
+    with pytest.raises(KernelArgumentError, match="cannot be added"):
+        ops().gemm(x[:8].to(DEV), w.to(DEV), held[:8].clone(), add=True)
+    with pytest.raises(KernelArgumentError, match="cannot be added"):
+        ops().gemm(x.to(DEV), w.to(DEV), torch.empty(m, n, dtype=torch.bfloat16, device=DEV), add=True)
+
+
 @pytest.mark.parametrize("m,n,k,slices", [(1000, 2000, 8192, 2), (500, 2000, 8192, 4), (4000, 2000, 8192, 2),
                                           (300, 2000, 4096, 4)])
 def test_gemm_with_large_tiles_in_slices_of_k(m, n, k, slices):
