@@ -776,15 +776,27 @@ __global__ __launch_bounds__(64 * NWM * NWN) void k_gemm_bf16_dma(const bf16_t* 
     // whole vectors: every row of this tile inside, the lane's columns inside, rows of Y aligned
     const bool vectors = m0 + BM <= M && n0 + BN <= N && out_n % per_lane == 0 &&
                          ((uintptr_t)Y % (per_lane * sizeof(TOut))) == 0;
+    constexpr int ITS = 32 * LPR / 64;                 // rows of a pass that a lane stores
+    constexpr bool CAN_ADD = std::is_same<TOut, float>::value;
 #pragma unroll
     for (int i = 0; i < TMI; ++i) {
+        // what the output holds (the epilogue that adds): a pass's rows asked for together, before the
+        // accumulators go through LDS, so that the trips to memory overlap each other and the staging
+        float4 held[CAN_ADD ? ITS : 1];
+        if (CAN_ADD && adds && vectors && lane_on) {
+#pragma unroll
+            for (int it = 0; it < ITS; ++it) {
+                const int m = m0 + wm * WM + i * 32 + it * (64 / LPR) + lane / LPR;
+                held[CAN_ADD ? it : 0] = held_vector<TOut>(Y + (size_t)m * out_n + n);
+            }
+        }
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 staged[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * EP_LD + j * 32 + (lane & 31)] = acc[i][j][r];
-#pragma unroll 2
-        for (int it = 0; it < 32 * LPR / 64; ++it) {
+#pragma unroll
+        for (int it = 0; it < ITS; ++it) {
             if (!lane_on) continue;
             const int row = it * (64 / LPR) + lane / LPR;
             const float4 v = *reinterpret_cast<const float4*>(&staged[row * EP_LD + out_col]);
@@ -796,9 +808,9 @@ __global__ __launch_bounds__(64 * NWM * NWN) void k_gemm_bf16_dma(const bf16_t* 
             }
             TOut* dst = Y + (size_t)m * out_n + (swiglu ? n / 2 : n);
             if (vectors) {
-                if (adds) {
-                    const float4 held = held_vector<TOut>(dst);
-                    o[0] = held.x + o[0], o[1] = held.y + o[1], o[2] = held.z + o[2], o[3] = held.w + o[3];
+                if (CAN_ADD && adds) {
+                    const float4 h = held[CAN_ADD ? it : 0];
+                    o[0] = h.x + o[0], o[1] = h.y + o[1], o[2] = h.z + o[2], o[3] = h.w + o[3];
                 }
                 store_vector<TOut>(dst, o, swiglu);
             } else if (m < M) {
