@@ -459,9 +459,16 @@ __global__ void k_attn_decode_merge(const float* __restrict__ part_o, const floa
                                     bf16_t* __restrict__ out, const int32_t* __restrict__ rows,
                                     const int32_t* __restrict__ seg_start, const int32_t* __restrict__ positions,
                                     int heads, int head_dim, int n_splits, int window) {
-    constexpr int GROUP = 8, NJ = 2;          // head_dim <= NJ * WAVE
+    // A lane holds four neighbouring elements of the head, head_dim / 4 lanes a split's output, so the wave
+    // takes several splits side by side (4 at head size 64), each lane GROUP of its splits' loads in flight at
+    // once: a wave that fetches split after split makes one trip to memory after the other, and at 128 splits
+    // (32,768 keys) the kernel was nothing but those trips (15 us; 4.7 at 16 splits, which is what a launch costs).
+    constexpr int GROUP = 8;
     const int ri = blockIdx.x / heads, head = blockIdx.x % heads;
     const int lane = threadIdx.x;
+    const int lanes_a_split = head_dim / 4, side = WAVE / lanes_a_split;   // splits side by side
+    const int sub = lane / lanes_a_split, d = (lane % lanes_a_split) * 4;
+    const bool works = sub < side;
     const int t = seg_start[rows[ri]];
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
@@ -473,11 +480,9 @@ __global__ void k_attn_decode_merge(const float* __restrict__ part_o, const floa
         ms = fmaxf(ms, s <= s_hi ? part_ml[(base + s) * 2] : -INFINITY);
     }
     ms = wave_max(ms);
-    float acc[NJ];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) acc[j] = 0.f;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
     float ls = 0.f;
-    for (int s0 = s_lo; s0 <= s_hi; s0 += WAVE) {
+    for (int s0 = s_lo; s0 <= s_hi; s0 += WAVE) {        // lane i holds the weight of split s0 + i
         const int s = s0 + lane;
         float wgt = 0.f, l = 0.f;
         if (s <= s_hi) {
@@ -485,35 +490,40 @@ __global__ void k_attn_decode_merge(const float* __restrict__ part_o, const floa
             wgt = (m == -INFINITY) ? 0.f : __expf(m - ms);
             l = part_ml[(base + s) * 2 + 1] * wgt;
         }
+        ls += l;
         const int n_here = min(WAVE, s_hi - s0 + 1);
-        for (int k0 = 0; k0 < n_here; k0 += GROUP) {
-            float v[GROUP][NJ];
+        for (int k0 = 0; k0 < n_here; k0 += GROUP * side) {
+            float4 v[GROUP];
 #pragma unroll
-            for (int i = 0; i < GROUP; ++i) {
-                const float* po = part_o + (base + s0 + min(k0 + i, n_here - 1)) * head_dim;
-#pragma unroll
-                for (int j = 0; j < NJ; ++j) {
-                    const int d = lane + j * WAVE;
-                    v[i][j] = d < head_dim ? po[d] : 0.f;
-                }
+            for (int i = 0; i < GROUP; ++i) {            // past the last split: the last again, weighing nothing
+                const int k = min(k0 + i * side + min(sub, side - 1), n_here - 1);
+                v[i] = *reinterpret_cast<const float4*>(part_o + (base + s0 + k) * head_dim + d);
             }
 #pragma unroll
             for (int i = 0; i < GROUP; ++i) {
-                const bool on = k0 + i < n_here;
-                const int src = min(k0 + i, WAVE - 1);
-                const float wk = on ? __shfl(wgt, src, WAVE) : 0.f;
-                ls += on ? __shfl(l, src, WAVE) : 0.f;
-#pragma unroll
-                for (int j = 0; j < NJ; ++j) acc[j] += v[i][j] * wk;
+                const int k = k0 + i * side + sub;
+                const float wk = __shfl(wgt, min(k, WAVE - 1), WAVE);
+                const bool on = works && k < n_here;
+                acc[0] += on ? v[i].x * wk : 0.f;
+                acc[1] += on ? v[i].y * wk : 0.f;
+                acc[2] += on ? v[i].z * wk : 0.f;
+                acc[3] += on ? v[i].w * wk : 0.f;
             }
         }
     }
-    const float inv = ls > 0.f ? 1.0f / ls : 0.f;
+    ls = wave_sum(ls);
+    // the sums of the splits side by side, added in the order of the sides
+    float total[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < side; ++k) {
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-        const int d = lane + j * WAVE;
-        if (d < head_dim) out[((size_t)t * heads + head) * head_dim + d] = f32_to_bf16(acc[j] * inv);
+        for (int c = 0; c < 4; ++c) total[c] += __shfl(acc[c], (lane % lanes_a_split) + k * lanes_a_split, WAVE);
     }
+    if (sub != 0) return;
+    const float inv = ls > 0.f ? 1.0f / ls : 0.f;
+    uint2 packed;
+    packed.x = f32x2_to_bf16x2(total[0] * inv, total[1] * inv);
+    packed.y = f32x2_to_bf16x2(total[2] * inv, total[3] * inv);
+    *reinterpret_cast<uint2*>(out + ((size_t)t * heads + head) * head_dim + d) = packed;
 }
 
 // ---------------------------------------------------------------- prompt portions
@@ -1213,6 +1223,8 @@ static int attention_decode_launch(const void* q, const void* k_cache, const voi
                                    int heads, int kv_heads, int head_dim, int n_pages, float scale, int window,
                                    int n_splits, hipStream_t s, const FromQkv* from_qkv = nullptr) {
     const int G = heads / kv_heads;
+    // the merge moves four elements of a head in one access
+    if (n_splits > 1 && (((uintptr_t)part_o & 15) || ((uintptr_t)out & 7))) return IMPARO_BAD_ARGUMENT;
     dim3 grid(n_splits, kv_heads * ((G + 15) / 16), n_rows);
     if (from_qkv) {
 #define DECODE_FROM_QKV(ND)                                                                                          \

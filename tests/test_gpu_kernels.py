@@ -537,6 +537,49 @@ def test_matrix_core_attention(H, Hk, D, page_size, window):
     torch.testing.assert_close(got, ref, rtol=2 ** -6, atol=2 ** -6)
 
 
+@pytest.mark.parametrize("H,Hk,D,window", [(8, 2, 64, None), (4, 1, 128, None), (6, 2, 48, None), (8, 2, 64, 9000)])
+def test_decode_attention_over_many_splits(H, Hk, D, window):
+    """Single tokens deep in long contexts: 79, 65, 33 and 2 splits of 256 keys meet in the merge, which takes
+    several splits side by side and in groups (more than one group, more than one round of 64 splits, an
+    odd remainder). One far key stands out for every query, so a split lost or weighed wrongly shows."""
+    page_size, ctx_lens = 64, (20001, 16385, 8200, 300)
+    tables, nxt = [], 0
+    for c in ctx_lens:
+        n = (c + page_size - 1) // page_size
+        tables.append(list(range(nxt, nxt + n)))
+        nxt += n
+    ctx = hand_context([(c - 1, 1) for c in ctx_lens], page_size, nxt, torch.bfloat16, DEV, kv_sites={0: (Hk, D)},
+                       tables=tables, v_transposed=True)
+    k_cache, v_cache, table = ctx.kv(0)
+    qs, refs = [], []
+    scale = 1.0 / math.sqrt(D)
+    for r, c in enumerate(ctx_lens):
+        q, k, v = rnd(1, H, D, seed=50 + r), rnd(c, Hk, D, seed=60 + r), rnd(c, Hk, D, seed=70 + r)
+        far = 700 * (r + 1) % c if window is None else max(0, c - window) + 3 * r        # (near the window's far end)
+        k[far] = 0
+        k[far, :, 0] = 6.0
+        q[0, :, 0] = 6.0 / scale / 6.0 * 1.5            # the far key's score stands 9 above the others' spread
+        q, k, v = (t.to(torch.bfloat16).float() for t in (q, k, v))
+        pages = len(tables[r])
+        kp = torch.zeros(pages * page_size, Hk, D); kp[:c] = k
+        vp = torch.zeros(pages * page_size, Hk, D); vp[:c] = v
+        k_cache[tables[r]] = kp.reshape(pages, page_size, Hk, D).permute(0, 2, 1, 3).to(torch.bfloat16).to(DEV)
+        v_cache[tables[r]] = vp.reshape(pages, page_size, Hk, D).permute(0, 2, 3, 1).to(torch.bfloat16).to(DEV)
+        lo = 0 if window is None else max(0, c - window)
+        kk, vv = k[lo:].repeat_interleave(H // Hk, dim=1), v[lo:].repeat_interleave(H // Hk, dim=1)
+        w = torch.softmax(torch.einsum("hd,chd->hc", q[0].double(), kk.double()) * scale, dim=-1)
+        refs.append(torch.einsum("hc,chd->hd", w, vv.double()).float())
+        qs.append(q)
+    q_all = torch.cat(qs).to(torch.bfloat16).to(DEV)
+    out = torch.full((ctx.n_tokens, H * D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    n_splits = (ctx.max_context + 255) // 256
+    part_o = torch.full((ctx.n_single_rows * H * n_splits * D,), float("nan"), device=DEV)
+    part_ml = torch.full((ctx.n_single_rows * H * n_splits * 2,), float("nan"), device=DEV)
+    ops().attention_decode(q_all, k_cache, v_cache, out, part_o, part_ml, ctx.single_rows, ctx.n_single_rows,
+                           ctx.seg_start, ctx.positions, table, scale, window, ctx.max_context)
+    torch.testing.assert_close(out.cpu().float().reshape(-1, H, D), torch.stack(refs), rtol=2 ** -6, atol=2 ** -6)
+
+
 @pytest.mark.parametrize("H,Hk,D", [(6, 3, 64), (40, 2, 32), (12, 3, 96), (8, 1, 128)])
 @pytest.mark.parametrize("page_size,window", [(16, None), (32, 19), (128, 300)])
 @pytest.mark.parametrize("parts", [2, 3, 8])
