@@ -154,6 +154,7 @@ class Engine:
         self._graphs: Dict[Tuple[int, int], _DecodeGraph] = {}
         self._decode_code_loaded = False
         self._graph_pool = None
+        self._capture_stream = None
         self.vocab_size = self.plan.vocab_size
         self.max_position = self.plan.max_position
         self.steps_run = 0
@@ -300,8 +301,19 @@ class Engine:
             if self._graph_pool is None:
                 self._graph_pool = torch.cuda.graph_pool_handle()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self._graph_pool), ops.on_current_stream():
-                g.logits = self.model.forward(ctx, token_ids, want_rows)
+            # Captured by hand, on a stream of its own: the library's context manager waits for the device, collects
+            # garbage and empties the allocator's cache before every capture, which is most of what a new shape costs.
+            if self._capture_stream is None:
+                self._capture_stream = torch.cuda.Stream(device=self.device)
+            here = torch.cuda.current_stream(self.device)
+            self._capture_stream.wait_stream(here)
+            with torch.cuda.stream(self._capture_stream), ops.on_current_stream():
+                graph.capture_begin(pool=self._graph_pool)
+                try:
+                    g.logits = self.model.forward(ctx, token_ids, want_rows)
+                finally:
+                    graph.capture_end()
+            here.wait_stream(self._capture_stream)
             g.pinned = self.workspace.pin()          # the buffers whose addresses the graph holds
             g.graph = graph
         else:
