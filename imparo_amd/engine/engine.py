@@ -97,8 +97,20 @@ class _DecodeGraph:
         self.last_used = 0
 
 
-TABLE_BUCKET = 8     # captured steps round their block-table width up to this many pages
-MAX_GRAPHS = 96      # captured batch shapes kept; beyond that the one unused for longest goes
+TABLE_BUCKET = 8     # captured steps round their block-table width up to a multiple of this many pages, or more
+MAX_GRAPHS = 256     # captured batch shapes kept; beyond that the one unused for longest goes
+
+
+def table_bucket(pages: int) -> int:
+    """The block-table width a captured step is sized for: `pages` rounded up to a multiple of 8 up to 127
+    pages, of 16 up to 255, of 32 up to 511, and so on: at most an eighth wider than the longest context
+    needs (the attention grid is sized by it, and a split nobody needs still costs its blocks' launch:
+    0.7 us a layer for each 256 keys too many at 13 rows), and a long run meets few widths (a shape is a
+    number of rows and a width, and a new one costs several steps' time to capture)."""
+    step = TABLE_BUCKET
+    while step * 16 <= pages:
+        step *= 2
+    return -(-pages // step) * step
 
 
 class Engine:
@@ -282,7 +294,7 @@ class Engine:
         launch (a capture cannot load code onto the device, and every module of
         kernels a decode step uses is loaded once one has run); after that a
         batch shape is captured when it first comes and replayed from then on."""
-        width = -(-batch.widest // TABLE_BUCKET) * TABLE_BUCKET
+        width = table_bucket(batch.widest)
         key = (len(entries), width)
         if not self._decode_code_loaded:
             self._decode_code_loaded = True
