@@ -785,7 +785,11 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     const int32_t* __restrict__ block_table, int table_stride, int page_size, int heads, int kv_heads, int n_pages,
     float scale, int window, int heads_per_block, float* __restrict__ part_o, float* __restrict__ part_ml) {
     constexpr int D = ND * 16, NK = ND / 2;
-    constexpr int LDK = D + 8, LDV = PX_KEYS + 8;
+    // Rows of K lie their length + 32 bytes apart: the fragment reads (row lane % 16, 16-byte piece lane / 16) then
+    // meet no bank conflict at any head size (with 16 bytes of padding each read takes 8 cycles instead of 4; counted
+    // with SQ_LDS_BANK_CONFLICT on reads alone). V^T rows keep 16 bytes: 32 would free its reads too but make the
+    // staging stores of its reordered keys collide instead, and the kernel gains nothing more from it (measured).
+    constexpr int LDK = D + 16, LDV = PX_KEYS + 8;
     static_assert(ND % 2 == 0, "head sizes in steps of 32");
     const int page_shift = __ffs(page_size) - 1;
     __shared__ __attribute__((aligned(16))) bf16_t ks[2][PX_KEYS * LDK];
