@@ -29,6 +29,19 @@ class RefCache:
         return self._memo[key]
 
 
+def assert_picks_near_best(plain, prompt, generated, rel, what=""):
+    """For runs whose rounding may turn a near-tie the other way (bfloat16): every generated
+    token must be, in the plain implementation's logits of the same prefix, within `rel` of the
+    largest logit magnitude below the best token. A token recomputed from a wrong prefix or a
+    stale state misses by far more."""
+    ref = plain.logits(list(prompt) + list(generated))
+    scale = float(ref.abs().max())
+    for i, tok in enumerate(generated):
+        row = ref[len(prompt) - 1 + i]
+        gap = float(row.max() - row[tok])
+        assert gap <= rel * scale, f"{what}: token {i} ({tok}) lies {gap:.3g} below the best, allowed {rel * scale:.3g}"
+
+
 def step_all(engine, rid, tokens, cuts: Sequence[int]) -> torch.Tensor:
     """Feeds `tokens` as request `rid` in portions of the sizes in `cuts`
     (repeated as needed), wanting every position; returns [T, V] on the CPU."""

@@ -8,8 +8,8 @@ import pytest
 import torch
 
 from conftest import assert_varied, prompt_tokens
-from gpu_helpers import make_engine
-from tolerances import check_logits
+from gpu_helpers import assert_picks_near_best, make_engine
+from tolerances import BF16_REL, check_logits
 
 pytestmark = pytest.mark.gpu
 
@@ -116,16 +116,21 @@ def loud_long_model(tmp_path_factory):
     return d
 
 
-def test_serving_workload_under_page_pressure(loud_long_model):
-    long_model = loud_long_model
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_serving_workload_under_page_pressure(loud_long_model, dtype):
     """32 requests in waves, prompts of 20..600 tokens, 5..40 new tokens each, a pool that holds
-    about a third of them at once: every output equals the request's output when it runs alone."""
+    about a third of them at once: every output equals the request's output when it runs alone.
+    In bfloat16 a request that runs alone takes other kernels than it took in a batch (the fused
+    launches of steps with few rows), so a near-tie may fall the other way; there every token a
+    request was given must be among the plain implementation's best for the tokens before it,
+    to twice the bound on a logit (two logits, each off by the bound, can swap places)."""
+    long_model = loud_long_model
     from imparo_amd.engine import Engine
     from imparo_amd.engine.scheduler import Scheduler, generate
     from imparo_amd.sampling import Sampler, SamplingParams
     rng = random.Random(3)
     reqs = [(prompt_tokens(512, rng.randint(20, 600), 500 + i), rng.randint(5, 40)) for i in range(32)]
-    eng = Engine(long_model, dtype="float32", page_size=16, max_tokens=3200, max_requests=12)
+    eng = Engine(long_model, dtype=dtype, page_size=16, max_tokens=3200, max_requests=12)
     sched = Scheduler(eng, Sampler(eng.device).pick, max_batch_tokens=512, max_running=12, portion=128)
     pending = list(enumerate(reqs))
     while pending or sched.has_work():
@@ -138,10 +143,18 @@ def test_serving_workload_under_page_pressure(loud_long_model):
             eng.cache.check()
     assert any(e[0] == "preempt" for e in sched.log) and any(e[0] == "wait" for e in sched.log)
     assert eng.free_pages() == [200, 200] and eng.cache.slots.n_free == 12
-    alone = Engine(long_model, dtype="float32", page_size=16, max_tokens=1024, max_requests=2)
     checked = rng.sample(range(32), 10)
     assert_varied([sched.finished[i].generated for i in checked if reqs[i][1] >= 8])
+    if dtype == "float32":
+        alone = Engine(long_model, dtype="float32", page_size=16, max_tokens=1024, max_requests=2)
+        for i in checked:
+            prompt, n = reqs[i]
+            assert sched.finished[i].finish_reason == "length"
+            assert sched.finished[i].generated == generate(alone, [prompt], max_tokens=n)[0], f"request {i}"
+        return
+    from plain_lfm2 import PlainLfm2
+    plain = PlainLfm2(long_model)
     for i in checked:
         prompt, n = reqs[i]
-        assert sched.finished[i].finish_reason == "length"
-        assert sched.finished[i].generated == generate(alone, [prompt], max_tokens=n)[0], f"request {i}"
+        assert sched.finished[i].finish_reason == "length" and len(sched.finished[i].generated) == n
+        assert_picks_near_best(plain, prompt, sched.finished[i].generated, 2 * BF16_REL, f"request {i}")

@@ -293,3 +293,116 @@ def test_a_conv_block_is_the_library_conv_between_two_gates(plain_models):
                     groups=m.E)[0].t()
     want = F.linear(C * conv, m.w[p + "out_proj.weight"], m.w[p + "out_proj.bias"])
     torch.testing.assert_close(m.mixer_conv(0, h), want, rtol=1e-5, atol=1e-6)
+
+
+def _attention_layer_input(m, layer, tokens, seed):
+    """A normed input for one attention layer of a plain model, and its positions."""
+    g = torch.Generator().manual_seed(seed)
+    T = len(tokens)
+    return torch.randn(T, m.E, generator=g), np.arange(T)
+
+
+def test_values_are_not_normed_so_twice_the_values_give_twice_the_delta(plain_models):
+    """/root/reference/crates/imparo-model/src/lfm2/workflow_cpu.rs:218-229 norms q and k per head and
+    leaves v as projected. Doubling v_proj must then double the attention mixer's output, exactly (a
+    power of two commutes with every rounding); a norm on v would swallow the factor."""
+    import copy
+    for name, layer in (("A", 1), ("B", 2)):
+        m = copy.copy(plain_models[name])
+        m.w = dict(m.w)
+        h, pos = _attention_layer_input(m, layer, range(13), 4)
+        once, (_, v1) = m.mixer_attention(layer, h, pos, None)
+        key = f"model.layers.{layer}.self_attn.v_proj.weight"
+        m.w[key] = 2 * m.w[key]
+        twice, (_, v2) = m.mixer_attention(layer, h, pos, None)
+        assert torch.equal(v2, 2 * v1)
+        assert torch.equal(twice, 2 * once)
+        assert once.abs().max() > 1e-4
+
+
+def test_keys_and_queries_are_normed_so_their_projections_scale_away(plain_models):
+    """workflow_cpu.rs:218-229: the RMS norm over each head of q and of k. With eps far below the heads'
+    mean squares, three times k_proj (or q_proj) changes nothing; without the norm on k the scores
+    would be three times as sharp and the logits would move."""
+    import copy
+    for name, vocab in (("A", 256), ("B", 384)):
+        base = copy.copy(plain_models[name])
+        base.w = dict(base.w)
+        base.eps = 1e-12
+        toks = [(13 * i + 5) % vocab for i in range(20)]
+        want = base.logits(toks)
+        for which in ("k_proj", "q_proj"):
+            m = copy.copy(base)
+            m.w = dict(base.w)
+            for k in list(m.w):
+                if k.endswith(f"self_attn.{which}.weight"):
+                    m.w[k] = 3 * m.w[k]
+            torch.testing.assert_close(m.logits(toks), want, rtol=1e-4, atol=1e-6)
+        # the same factor on a weight that no norm follows does show: the test can fail
+        m = copy.copy(base)
+        m.w = dict(base.w)
+        for k in list(m.w):
+            if k.endswith("self_attn.v_proj.weight"):
+                m.w[k] = 3 * m.w[k]
+        assert (m.logits(toks) - want).abs().max() > 1e-3
+
+
+def test_the_attention_mixer_is_library_attention_at_its_default_scale(plain_models):
+    """workflow_cpu.rs:243 scales scores by 1/sqrt(head size), which is what
+    F.scaled_dot_product_attention does when no scale is given. The mixer, from its projections to its
+    output projection, against the library routine on the same normed and rotated q and k, the plain v,
+    causal, each group of H/Hk neighbouring heads on one kv head (cpu_support.rs:402-445)."""
+    F = torch.nn.functional
+    for name, layer in (("A", 3), ("B", 4)):
+        m = plain_models[name]
+        T = 17
+        h, pos = _attention_layer_input(m, layer, range(T), 9)
+        p = f"model.layers.{layer}.self_attn."
+        q = F.linear(h, m.w[p + "q_proj.weight"]).reshape(T, m.H, m.D)
+        k = F.linear(h, m.w[p + "k_proj.weight"]).reshape(T, m.Hk, m.D)
+        v = F.linear(h, m.w[p + "v_proj.weight"]).reshape(T, m.Hk, m.D)
+        q = m.norm_and_rotate(q, m.w[p + "q_layernorm.weight"], pos)
+        k = m.norm_and_rotate(k, m.w[p + "k_layernorm.weight"], pos)
+        per_kv = m.H // m.Hk
+        kk = k.repeat_interleave(per_kv, dim=1)
+        vv = v.repeat_interleave(per_kv, dim=1)
+        o = F.scaled_dot_product_attention(q.transpose(0, 1), kk.transpose(0, 1), vv.transpose(0, 1), is_causal=True)
+        want = F.linear(o.transpose(0, 1).reshape(T, m.H * m.D), m.w[p + "out_proj.weight"])
+        got, _ = m.mixer_attention(layer, h, pos, None)
+        torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+        # another scale would show: scores of this size move the output far above the tolerance
+        wrong = F.scaled_dot_product_attention(q.transpose(0, 1), kk.transpose(0, 1), vv.transpose(0, 1),
+                                               is_causal=True, scale=1.0)
+        assert (F.linear(wrong.transpose(0, 1).reshape(T, m.H * m.D), m.w[p + "out_proj.weight"]) - want
+                ).abs().max() > 100 * (got - want).abs().max() + 1e-5
+
+
+def test_a_block_adds_its_mixer_first_and_feeds_the_sum_to_the_feed_forward(plain_models):
+    """workflow_cpu.rs:293-316: x1 = x + mixer(norm_a(x)); x2 = x1 + ffn(norm_b(x1)). One block of each
+    kind, put together here from the part functions, equals what the model computes for that block; the
+    other order (feed-forward first, the mixer on the sum) and the parallel form (both on x) do not."""
+    for name, vocab in (("A", 256), ("B", 384)):
+        m = plain_models[name]
+        toks = [(3 * i + 7) % vocab for i in range(15)]
+        e = m.w["model.embed_tokens.weight"][toks]
+        kinds = m.cfg["layer_types"]
+        for layer in (kinds.index("conv"), kinds.index("full_attention")):
+            p = f"model.layers.{layer}."
+            norm_a = lambda x: P.rms_norm(x, m.w[p + "operator_norm.weight"], m.eps)
+            norm_b = lambda x: P.rms_norm(x, m.w[p + "ffn_norm.weight"], m.eps)
+            ffn = lambda n: P.swiglu(n, m.w[p + "feed_forward.w1.weight"], m.w[p + "feed_forward.w3.weight"],
+                                     m.w[p + "feed_forward.w2.weight"])
+            if kinds[layer] == "conv":
+                mixer = lambda h: m.mixer_conv(layer, h)
+            else:
+                mixer = lambda h: m.mixer_attention(layer, h, np.arange(len(toks)), None)[0]
+            x1 = e + mixer(norm_a(e))
+            want = x1 + ffn(norm_b(x1))
+            got = m.hidden(toks, order=[(layer, None)])
+            torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-7)
+            f1 = e + ffn(norm_b(e))
+            ffn_first = f1 + mixer(norm_a(f1))
+            parallel = e + mixer(norm_a(e)) + ffn(norm_b(e))
+            gap = (got - want).abs().max()
+            assert (got - ffn_first).abs().max() > 1e-5 + 100 * gap
+            assert (got - parallel).abs().max() > 1e-5 + 100 * gap
