@@ -14,6 +14,11 @@ typedef void* imparo_stream;
 // The hash of the sources this library was built from, as the build computed it.
 const char* imparo_hip_source_hash();
 
+// Loads the code of every kernel file onto the current device. The runtime would load each file's
+// code when one of its kernels is first launched, which a stream under graph capture cannot do: call
+// this once per device before the first capture.
+int imparo_load_code(void);
+
 // x[t, :] = table[ids[t], :] as float32.
 int imparo_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* x,
                         int n_tokens, int width, int vocab, imparo_stream stream);
@@ -186,6 +191,100 @@ int imparo_fill_f32(float* p, float value, int64_t n, imparo_stream stream);
 // and value are device arrays of n_sites entries that the caller built from tensors it owns.
 int imparo_fill_sites(const uint64_t* base, const int64_t* per_slot, const float* value, int n_sites, int slot,
                       imparo_stream stream);
+
+// ---------------------------------------------------------------------------------------------
+// A model's step as one call. A program is the model's run order as a list of operations over a
+// float32 residual stream: the embedding, then per layer a norm, a mixer, a norm and a
+// feed-forward, then the norm and head of the wanted rows. Each operation launches the kernels
+// above, chosen by the batch's shape exactly as a caller of the single entry points would choose
+// them; what the program saves is the caller's time between launches. The reference issues a
+// step's kernels from one native routine as well
+// (/root/reference/crates/imparo-model/src/lfm2/workflow_gpu.rs:317-1633).
+//
+// Scratch lives in regions that the caller binds: the program names them (imparo_program_region_*),
+// says how many bytes of each a step needs (imparo_program_needs) and refuses to run with
+// IMPARO_SCRATCH_TOO_SMALL, before any launch, when a bound region is too small for the step.
+// Nothing here allocates device memory.
+typedef struct ImparoProgram ImparoProgram;
+
+// A projection Y = X . W^T (+ bias): W is [n, k] in `dtype`, bias float32 [n] or null.
+typedef struct {
+    const void* weight;
+    const float* bias;
+    int32_t dtype, n, k;
+} ImparoLinearDesc;
+
+typedef struct {
+    ImparoLinearDesc qkv, out;           // fused q | k | v projection, output projection
+    const float* q_norm;                 // per-head RMS norm weights [head_dim], both null: no norm
+    const float* k_norm;
+    float norm_eps;
+    const float* inv_freq;               // [n_freq] or null
+    int32_t n_freq, interleaved;
+    int32_t heads, kv_heads, head_dim;
+    float scale;
+    int32_t window;                      // 0: every key
+    void* k_cache;                       // this call's cache site
+    void* v_cache;
+    int32_t n_pages, v_transposed, group; // group: which of the step's block tables
+    int32_t owns_cache;                  // 0: reads a cache that an earlier call of the step has written
+} ImparoAttentionDesc;
+
+typedef struct {
+    ImparoLinearDesc in_proj, out_proj;
+    const float* conv_weight;            // [width, taps]
+    const float* conv_bias;              // [width] or null
+    int32_t width, taps;
+    float* state;                        // [n_slots, taps - 1, width]
+    int32_t n_slots;
+} ImparoShortConvDesc;
+
+typedef struct {
+    ImparoLinearDesc gate_up, down;      // gate and up rows alternate in gate_up
+} ImparoSwigluDesc;
+
+// One batch: device arrays as imparo_cache_pack lays them out (any placement), and the sizes the
+// host knows. tables[g] is [n_rows, table_width] for cache group g.
+#define IMPARO_MAX_GROUPS 8
+typedef struct {
+    const int32_t* tokens;               // [n_tokens]
+    const int32_t* positions;            // [n_tokens]
+    const int32_t* row_of_token;         // [n_tokens]
+    const int32_t* seg_start;            // [n_rows]
+    const int32_t* seg_len;              // [n_rows]
+    const int32_t* slot;                 // [n_rows]
+    const int32_t* single_rows;          // [n_single]: rows that bring one token
+    const int32_t* portion_rows;         // [n_portion]: rows that bring more
+    const int32_t* want_rows;            // [n_want]: places in the packed batch whose logits are wanted
+    const int32_t* tables[IMPARO_MAX_GROUPS];
+    int32_t n_groups, table_width;
+    int32_t n_tokens, n_rows, n_want, n_single, n_portion;
+    int32_t max_seg_len, max_context;    // longest segment; longest context after the step (a bound will do)
+    int32_t portion_tiles;               // sum over the portion rows of ceil(tokens / imparo_attention_prefill_tile())
+} ImparoStepArgs;
+
+ImparoProgram* imparo_program_new(int engine_dtype, int page_size);
+void imparo_program_delete(ImparoProgram* p);
+// Operations, in run order. Each returns IMPARO_OK or IMPARO_BAD_ARGUMENT (sizes that do not fit).
+int imparo_program_embedding(ImparoProgram* p, const void* table, int table_dtype, int vocab, int width);
+// h = norm(stream + what the last mixer or feed-forward left pending), in out_dtype; the sum goes back to the stream
+int imparo_program_norm(ImparoProgram* p, const float* weight, float eps, int width, int out_dtype);
+int imparo_program_attention(ImparoProgram* p, const ImparoAttentionDesc* d);
+int imparo_program_short_conv(ImparoProgram* p, const ImparoShortConvDesc* d);
+int imparo_program_swiglu(ImparoProgram* p, const ImparoSwigluDesc* d);
+// logits = head(norm(stream + pending) at the wanted rows); the stream is left as it is
+int imparo_program_head(ImparoProgram* p, const float* norm_weight, float eps, int width, const ImparoLinearDesc* head);
+
+int imparo_program_n_regions(const ImparoProgram* p);
+const char* imparo_program_region_name(const ImparoProgram* p, int region);
+int imparo_program_bind(ImparoProgram* p, int region, void* ptr, int64_t bytes);
+// needs[region] = bytes of each region that a step of this shape uses (0: not used)
+int imparo_program_needs(ImparoProgram* p, const ImparoStepArgs* args, int64_t* needs);
+// Runs the step on `stream`. *logits = where the float32 [n_want, vocab] logits are (inside the
+// "logits" region), or null if nothing is wanted. IMPARO_SCRATCH_TOO_SMALL: nothing was launched,
+// imparo_program_needs says what to bind. Any other failure: imparo_program_error names the operation.
+int imparo_program_run(ImparoProgram* p, const ImparoStepArgs* args, float** logits, imparo_stream stream);
+const char* imparo_program_error(const ImparoProgram* p);
 
 #ifdef __cplusplus
 }

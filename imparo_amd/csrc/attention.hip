@@ -160,3 +160,12 @@ extern "C" int imparo_attention(const void* q, const void* k_cache, const void* 
         return IMPARO_BAD_ARGUMENT;
     return launch_status();
 }
+
+// Asks the runtime about one kernel of this file, which makes it load the file's code onto the
+// current device (it loads a file's kernels when one of them is first used; a stream under capture
+// cannot do that).
+int imparo_load_code_attention() {
+    hipFuncAttributes attributes;
+    return hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&k_attention_wave<float>)) == hipSuccess ? IMPARO_OK
+                                                                                              : IMPARO_LAUNCH_FAILED;
+}

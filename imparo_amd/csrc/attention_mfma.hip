@@ -1475,3 +1475,12 @@ extern "C" int imparo_attention_prefill(const void* q, const void* k_cache, cons
         seg_len, positions, block_table, table_stride, page_size, heads, kv_heads, n_pages, scale, window)));
     return launch_status();
 }
+
+// Asks the runtime about one kernel of this file, which makes it load the file's code onto the
+// current device (it loads a file's kernels when one of them is first used; a stream under capture
+// cannot do that).
+int imparo_load_code_attention_mfma() {
+    hipFuncAttributes attributes;
+    return hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&k_attn_decode_merge)) == hipSuccess ? IMPARO_OK
+                                                                                              : IMPARO_LAUNCH_FAILED;
+}

@@ -113,6 +113,14 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// One per file of kernels: loads that file's code onto the current device (imparo_load_code calls them all).
+int imparo_load_code_attention();
+int imparo_load_code_attention_mfma();
+int imparo_load_code_elementwise();
+int imparo_load_code_gemm();
+int imparo_load_code_rope_cache();
+int imparo_load_code_sampling();
+
 static inline int launch_status() {
     return hipGetLastError() == hipSuccess ? IMPARO_OK : IMPARO_LAUNCH_FAILED;
 }

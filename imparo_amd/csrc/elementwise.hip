@@ -540,3 +540,12 @@ extern "C" int imparo_short_conv_state(const float* bcx, float* state, const int
     k_short_conv_state<<<grid, threads, 0, (hipStream_t)stream>>>(bcx, state, seg_start, seg_len, slot, width, taps);
     return launch_status();
 }
+
+// Asks the runtime about one kernel of this file, which makes it load the file's code onto the
+// current device (it loads a file's kernels when one of them is first used; a stream under capture
+// cannot do that).
+int imparo_load_code_elementwise() {
+    hipFuncAttributes attributes;
+    return hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&k_fill_f32)) == hipSuccess ? IMPARO_OK
+                                                                                              : IMPARO_LAUNCH_FAILED;
+}

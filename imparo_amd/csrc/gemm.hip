@@ -1575,3 +1575,12 @@ extern "C" int imparo_gemm_variant(const void* x, const void* w, const float* bi
                                    int m, int n, int k, int epilogue, int slices, int variant, imparo_stream stream) {
     return gemm_variant(x, w, bias, y, dtype, out_dtype, m, n, k, epilogue, slices, variant, stream);
 }
+
+// Asks the runtime about one kernel of this file, which makes it load the file's code onto the
+// current device (it loads a file's kernels when one of them is first used; a stream under capture
+// cannot do that).
+int imparo_load_code_gemm() {
+    hipFuncAttributes attributes;
+    return hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&k_gemm_f32_rows<float>)) == hipSuccess ? IMPARO_OK
+                                                                                              : IMPARO_LAUNCH_FAILED;
+}

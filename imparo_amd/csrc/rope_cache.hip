@@ -413,3 +413,12 @@ extern "C" int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight
         return IMPARO_BAD_ARGUMENT;
     return launch_status();
 }
+
+// Asks the runtime about one kernel of this file, which makes it load the file's code onto the
+// current device (it loads a file's kernels when one of them is first used; a stream under capture
+// cannot do that).
+int imparo_load_code_rope_cache() {
+    hipFuncAttributes attributes;
+    return hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&k_qk_norm_rope_store<float>)) == hipSuccess ? IMPARO_OK
+                                                                                              : IMPARO_LAUNCH_FAILED;
+}

@@ -174,3 +174,12 @@ extern "C" int imparo_sample_rows(const float* logits, const float* temperature,
 #define IMPARO_SOURCE_HASH "unknown"
 #endif
 extern "C" const char* imparo_hip_source_hash() { return IMPARO_SOURCE_HASH; }
+
+// Asks the runtime about one kernel of this file, which makes it load the file's code onto the
+// current device (it loads a file's kernels when one of them is first used; a stream under capture
+// cannot do that).
+int imparo_load_code_sampling() {
+    hipFuncAttributes attributes;
+    return hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&k_argmax_rows)) == hipSuccess ? IMPARO_OK
+                                                                                              : IMPARO_LAUNCH_FAILED;
+}

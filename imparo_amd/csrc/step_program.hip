@@ -1,0 +1,492 @@
+// A model's step issued by one native call: the run order as a list of operations, each of which
+// launches the kernels of this library chosen by the batch's shape. Host code only; the kernels are
+// reached through the library's own C entry points, so a step issued from here and a step issued
+// launch by launch by a caller of those entry points run the same kernels with the same arguments.
+//
+// The list mirrors the pre-norm arrangement of parts: a float32 residual stream x, a delta that the
+// last mixer or feed-forward left pending on it (possibly in slices of K, added in order by the next
+// norm), and the normed rows h that the next part reads
+// (/root/reference/crates/imparo-model/src/lfm2/workflow_cpu.rs:8-15 for the arrangement,
+// /root/reference/crates/imparo-model/src/lfm2/workflow_gpu.rs:317-1633 for a step issued natively).
+#include <stdio.h>
+#include <string.h>
+
+#include <string>
+#include <vector>
+
+#include "api.h"
+#include "common.h"
+
+namespace {
+
+struct Region {
+    std::string name;
+    char* ptr = nullptr;
+    int64_t bytes = 0;
+};
+
+enum OpKind { OP_EMBEDDING, OP_NORM, OP_ATTENTION, OP_SHORT_CONV, OP_SWIGLU, OP_HEAD };
+
+struct Op {
+    OpKind kind;
+    // embedding
+    const void* table = nullptr;
+    int table_dtype = 0, vocab = 0, width = 0;
+    // norm (and the head's norm)
+    const float* weight = nullptr;
+    float eps = 0.f;
+    int out_dtype = 0;
+    ImparoAttentionDesc attention{};
+    ImparoShortConvDesc conv{};
+    ImparoSwigluDesc swiglu{};
+    ImparoLinearDesc head{};
+};
+
+inline int64_t element_size(int dtype) { return dtype == IMPARO_F32 ? 4 : 2; }
+
+}  // namespace
+
+struct ImparoProgram {
+    int engine_dtype = IMPARO_BF16, page_size = 0;
+    std::vector<Region> regions;
+    std::vector<Op> ops;
+    std::string error;
+    // regions by role
+    int r_residual, r_normed, r_mixer_in, r_mixer_mid, r_q, r_mixer_out, r_mixer_out_sliced, r_ffn_out, r_ffn_out_sliced,
+        r_part_o, r_part_ml, r_prefill_part_o, r_prefill_part_ml, r_normed_rows, r_logits;
+
+    int region(const char* name) {
+        regions.push_back(Region{name});
+        return (int)regions.size() - 1;
+    }
+};
+
+namespace {
+
+// One walk over the operations. A dry walk launches nothing and notes what each region must hold;
+// the real walk hands out the bound memory. Both take every decision from the same code.
+struct Walk {
+    ImparoProgram* p;
+    const ImparoStepArgs* a;
+    imparo_stream stream;
+    bool dry;
+    std::vector<int64_t> need;
+    int status = IMPARO_OK;
+    int op_index = 0;
+    // the residual stream, what is pending on it, the rows the next part reads
+    float* x = nullptr;
+    const float* pending = nullptr;
+    int n_pending = 0;
+    void* h = nullptr;
+    int h_dtype = IMPARO_F32;
+    float* logits = nullptr;
+
+    Walk(ImparoProgram* p, const ImparoStepArgs* a, imparo_stream s, bool dry)
+        : p(p), a(a), stream(s), dry(dry), need(p->regions.size(), 0) {}
+
+    void* get(int region, int64_t bytes) {
+        if (bytes < 1) bytes = 1;
+        if (bytes > need[region]) need[region] = bytes;
+        if (dry) return (void*)(uintptr_t)256;          // never read: a dry walk launches nothing
+        return p->regions[region].ptr;
+    }
+
+    void fail(int code, const char* what) {
+        if (status != IMPARO_OK) return;
+        status = code;
+        char buf[256];
+        snprintf(buf, sizeof buf, "operation %d: %s %s", op_index, what,
+                 code == IMPARO_BAD_ARGUMENT ? "refused its arguments" : "failed to launch");
+        p->error = buf;
+    }
+
+    // runs a launch unless the walk is dry or has failed
+    template <typename F>
+    void launch(const char* what, F&& f) {
+        if (dry || status != IMPARO_OK) return;
+        const int rc = f();
+        if (rc != IMPARO_OK) fail(rc, what);
+    }
+
+    struct Out {
+        void* ptr;
+        int slices;      // > 0: [slices, m, width] (1: plain); 0: added into the stream
+    };
+
+    // A projection of m rows, as a part's Linear runs it: in slices of K where the consumer adds
+    // slices and the library says that pays, added into `into` where the library's epilogue can,
+    // else plain into `region`.
+    Out linear(const ImparoLinearDesc& lin, const void* in, int in_dtype, int m, int out_dtype, int region,
+               int sliced_region, bool swiglu, bool sliced_ok, float* into) {
+        if (in_dtype != lin.dtype) {
+            fail(IMPARO_BAD_ARGUMENT, "a projection whose input is not in its weight's dtype");
+            return Out{nullptr, 1};
+        }
+        const int width = swiglu ? lin.n / 2 : lin.n;
+        if (sliced_ok && !swiglu && out_dtype == IMPARO_F32) {
+            const int slices = imparo_gemm_slices(m, lin.n, lin.k, lin.dtype);
+            if (slices > 1) {
+                void* out = get(sliced_region, (int64_t)slices * m * width * 4);
+                launch("imparo_gemm (slices of K)", [&] {
+                    return imparo_gemm(in, lin.weight, lin.bias, out, lin.dtype, IMPARO_F32, m, lin.n, lin.k, 0, slices, stream);
+                });
+                return Out{out, slices};
+            }
+        }
+        if (into && !swiglu && out_dtype == IMPARO_F32 && imparo_gemm_adds(m, lin.n, lin.k, lin.dtype)) {
+            launch("imparo_gemm (added to the stream)", [&] {
+                return imparo_gemm(in, lin.weight, lin.bias, into, lin.dtype, IMPARO_F32, m, lin.n, lin.k, 2, 1, stream);
+            });
+            return Out{into, 0};
+        }
+        void* out = get(region, (int64_t)m * width * element_size(out_dtype));
+        launch("imparo_gemm", [&] {
+            return imparo_gemm(in, lin.weight, lin.bias, out, lin.dtype, out_dtype, m, lin.n, lin.k, swiglu ? 1 : 0, 1, stream);
+        });
+        return Out{out, 1};
+    }
+
+    // what a mixer or feed-forward returned becomes the pending delta (or went into the stream already)
+    void leave(const Out& out) {
+        if (out.slices == 0) {
+            pending = nullptr;
+            n_pending = 0;
+        } else {
+            pending = (const float*)out.ptr;
+            n_pending = out.slices;
+        }
+    }
+
+    float* stream_if_nothing_pending() const { return pending ? nullptr : x; }
+
+    void embedding(const Op& op) {
+        const int T = a->n_tokens;
+        x = (float*)get(p->r_residual, (int64_t)T * op.width * 4);
+        pending = nullptr;
+        n_pending = 0;
+        launch("imparo_embed_gather", [&] {
+            return imparo_embed_gather(op.table, op.table_dtype, a->tokens, x, T, op.width, op.vocab, stream);
+        });
+    }
+
+    void norm(const Op& op) {
+        const int T = a->n_tokens;
+        void* out = get(p->r_normed, (int64_t)T * op.width * element_size(op.out_dtype));
+        const float* delta = pending;
+        const int n_delta = pending ? n_pending : 0;
+        launch("imparo_rms_norm", [&] {
+            return imparo_rms_norm(x, delta, n_delta, T, nullptr, op.weight, out, op.out_dtype, T, op.width, op.eps,
+                                   delta ? 1 : 0, stream);
+        });
+        pending = nullptr;
+        n_pending = 0;
+        h = out;
+        h_dtype = op.out_dtype;
+    }
+
+    void decode_parts(const ImparoAttentionDesc& d, float** part_o, float** part_ml, int* n_splits) {
+        const int split = imparo_attention_decode_split();
+        *n_splits = (a->max_context + split - 1) / split;
+        if (*n_splits < 1) *n_splits = 1;
+        *part_o = (float*)get(p->r_part_o, (int64_t)a->n_single * d.heads * *n_splits * d.head_dim * 4);
+        *part_ml = (float*)get(p->r_part_ml, (int64_t)a->n_single * d.heads * *n_splits * 2 * 4);
+    }
+
+    void attention(const Op& op) {
+        const ImparoAttentionDesc& d = op.attention;
+        const int T = a->n_tokens;
+        const int dt = p->engine_dtype;
+        if (d.group < 0 || d.group >= a->n_groups) return fail(IMPARO_BAD_ARGUMENT, "an attention whose cache group the step has no table for");
+        const int32_t* table = a->tables[d.group];
+        const int stride = a->table_width;
+        const Out qkv = linear(d.qkv, h, h_dtype, T, IMPARO_F32, p->r_mixer_in, -1, false, false, nullptr);
+        const int64_t o_bytes = (int64_t)T * d.heads * d.head_dim * element_size(dt);
+        if (dt != d.out.dtype) return fail(IMPARO_BAD_ARGUMENT, "an output projection whose weight dtype differs from the attention output's");
+        float* into = stream_if_nothing_pending();
+        if (d.v_transposed && d.owns_cache && a->n_single == T && a->n_portion == 0 && imparo_attention_decode_qkv_pays(T) &&
+            imparo_attention_decode_qkv_takes(d.head_dim, d.n_freq)) {
+            // every row brings one token: head norm, rotation and the write of the new key and value ride in the attention launch
+            void* o = get(p->r_mixer_mid, o_bytes);
+            float *part_o, *part_ml;
+            int n_splits;
+            decode_parts(d, &part_o, &part_ml, &n_splits);
+            launch("imparo_attention_decode_qkv", [&] {
+                return imparo_attention_decode_qkv((const float*)qkv.ptr, d.q_norm, d.k_norm, d.norm_eps, d.inv_freq, d.n_freq,
+                                                   d.interleaved, d.k_cache, d.v_cache, 1, o, part_o, part_ml, a->single_rows,
+                                                   a->n_single, a->seg_start, a->positions, table, stride, p->page_size,
+                                                   d.heads, d.kv_heads, d.head_dim, d.n_pages, d.scale, d.window, n_splits,
+                                                   stream);
+            });
+            return leave(linear(d.out, o, dt, T, IMPARO_F32, p->r_mixer_out, p->r_mixer_out_sliced, false, true, into));
+        }
+        void* q = get(p->r_q, o_bytes);
+        launch("imparo_qk_norm_rope_store", [&] {
+            return imparo_qk_norm_rope_store((const float*)qkv.ptr, d.q_norm, d.k_norm, d.norm_eps, d.inv_freq, d.n_freq,
+                                             d.interleaved, a->positions, a->row_of_token, d.owns_cache ? table : nullptr,
+                                             d.owns_cache ? stride : 0, p->page_size, q, d.owns_cache ? d.k_cache : nullptr,
+                                             d.owns_cache ? d.v_cache : nullptr, dt, d.owns_cache ? 1 : 0, T, d.heads,
+                                             d.kv_heads, d.head_dim, d.owns_cache ? d.n_pages : 0, d.v_transposed, stream);
+        });
+        void* o = get(p->r_mixer_mid, o_bytes);
+        if (d.v_transposed) {
+            // matrix-core kernels: single tokens split over their keys, portions tiled over their queries
+            if (a->n_single) {
+                float *part_o, *part_ml;
+                int n_splits;
+                decode_parts(d, &part_o, &part_ml, &n_splits);
+                launch("imparo_attention_decode", [&] {
+                    return imparo_attention_decode(q, d.k_cache, d.v_cache, o, part_o, part_ml, a->single_rows, a->n_single,
+                                                   a->seg_start, a->positions, table, stride, p->page_size, d.heads,
+                                                   d.kv_heads, d.head_dim, d.n_pages, d.scale, d.window, n_splits, stream);
+                });
+            }
+            if (a->n_portion) {
+                const int parts = imparo_attention_prefill_splits(a->portion_tiles, d.heads, d.kv_heads, d.head_dim, a->max_context);
+                float *part_o = nullptr, *part_ml = nullptr;
+                if (parts > 1) {
+                    part_o = (float*)get(p->r_prefill_part_o, (int64_t)T * d.heads * parts * d.head_dim * 4);
+                    part_ml = (float*)get(p->r_prefill_part_ml, (int64_t)T * d.heads * parts * 2 * 4);
+                }
+                launch("imparo_attention_prefill", [&] {
+                    return imparo_attention_prefill(q, d.k_cache, d.v_cache, o, part_o, part_ml, parts, a->portion_rows,
+                                                    a->n_portion, a->portion_tiles, a->seg_start, a->seg_len, a->positions,
+                                                    table, stride, p->page_size, d.heads, d.kv_heads, d.head_dim, d.n_pages,
+                                                    d.scale, d.window, stream);
+                });
+            }
+        } else {
+            launch("imparo_attention", [&] {
+                return imparo_attention(q, d.k_cache, d.v_cache, o, dt, a->positions, a->row_of_token, table, stride,
+                                        p->page_size, T, d.heads, d.kv_heads, d.head_dim, d.n_pages, d.scale, d.window, 0,
+                                        stream);
+            });
+        }
+        leave(linear(d.out, o, dt, T, IMPARO_F32, p->r_mixer_out, p->r_mixer_out_sliced, false, true, into));
+    }
+
+    void short_conv(const Op& op) {
+        const ImparoShortConvDesc& d = op.conv;
+        const int T = a->n_tokens, R = a->n_rows;
+        const int y_dtype = d.out_proj.dtype;
+        void* y = get(p->r_mixer_mid, (int64_t)T * d.width * element_size(y_dtype));
+        float* into = stream_if_nothing_pending();
+        const bool single = a->max_seg_len == 1;
+        if (single && d.in_proj.dtype == IMPARO_BF16 && T > 0 && T <= 16 && d.in_proj.n % 24 == 0 && d.in_proj.k % 8 == 0) {
+            // a decode step's few rows: projection and conv in one launch
+            if (h_dtype != IMPARO_BF16) return fail(IMPARO_BAD_ARGUMENT, "a conv input projection whose input is not in its weight's dtype");
+            launch("imparo_in_proj_conv_decode", [&] {
+                return imparo_in_proj_conv_decode(h, d.in_proj.weight, d.in_proj.bias, d.conv_weight, d.conv_bias, d.state,
+                                                  a->slot, y, y_dtype, T, d.width, d.in_proj.k, d.taps, d.n_slots, stream);
+            });
+            return leave(linear(d.out_proj, y, y_dtype, T, IMPARO_F32, p->r_mixer_out, p->r_mixer_out_sliced, false, true, into));
+        }
+        const Out bcx = linear(d.in_proj, h, h_dtype, T, IMPARO_F32, p->r_mixer_in, -1, false, false, nullptr);
+        if (single) {
+            if (T != R) return fail(IMPARO_BAD_ARGUMENT, "a step of single tokens whose rows and tokens differ in number");
+            launch("imparo_short_conv_decode", [&] {
+                return imparo_short_conv_decode((const float*)bcx.ptr, d.conv_weight, d.conv_bias, d.state, a->slot, y, y_dtype, R,
+                                                d.width, d.taps, d.n_slots, stream);
+            });
+        } else {
+            launch("imparo_short_conv", [&] {
+                return imparo_short_conv((const float*)bcx.ptr, d.conv_weight, d.conv_bias, d.state, a->row_of_token, a->seg_start,
+                                         a->slot, y, y_dtype, T, d.width, d.taps, d.n_slots, R, stream);
+            });
+            launch("imparo_short_conv_state", [&] {
+                return imparo_short_conv_state((const float*)bcx.ptr, d.state, a->seg_start, a->seg_len, a->slot, R, T, d.width,
+                                               d.taps, d.n_slots, stream);
+            });
+        }
+        leave(linear(d.out_proj, y, y_dtype, T, IMPARO_F32, p->r_mixer_out, p->r_mixer_out_sliced, false, true, into));
+    }
+
+    void swiglu(const Op& op) {
+        const ImparoSwigluDesc& d = op.swiglu;
+        const int T = a->n_tokens;
+        float* into = stream_if_nothing_pending();
+        // the gated hidden may lie where the mixer's input projection lay: that is dead by now
+        const Out g = linear(d.gate_up, h, h_dtype, T, d.down.dtype, p->r_mixer_in, -1, true, false, nullptr);
+        leave(linear(d.down, g.ptr, d.down.dtype, T, IMPARO_F32, p->r_ffn_out, p->r_ffn_out_sliced, false, true, into));
+    }
+
+    void head(const Op& op) {
+        const int W = a->n_want;
+        if (W == 0) return;
+        void* rows = get(p->r_normed_rows, (int64_t)W * op.width * element_size(op.head.dtype));
+        const float* delta = pending;
+        const int n_delta = pending ? n_pending : 0;
+        launch("imparo_rms_norm (wanted rows)", [&] {
+            return imparo_rms_norm(x, delta, n_delta, a->n_tokens, a->want_rows, op.weight, rows, op.head.dtype, W, op.width,
+                                   op.eps, 0, stream);
+        });
+        const Out out = linear(op.head, rows, op.head.dtype, W, IMPARO_F32, p->r_logits, -1, false, false, nullptr);
+        logits = (float*)out.ptr;
+    }
+
+    void run() {
+        if (a->n_tokens < 1 || a->n_rows < 1 || a->n_groups < 0 || a->n_groups > IMPARO_MAX_GROUPS)
+            return fail(IMPARO_BAD_ARGUMENT, "a step without tokens, or with more cache groups than the library takes;");
+        for (op_index = 0; op_index < (int)p->ops.size() && status == IMPARO_OK; ++op_index) {
+            const Op& op = p->ops[op_index];
+            switch (op.kind) {
+                case OP_EMBEDDING: embedding(op); break;
+                case OP_NORM: norm(op); break;
+                case OP_ATTENTION: attention(op); break;
+                case OP_SHORT_CONV: short_conv(op); break;
+                case OP_SWIGLU: swiglu(op); break;
+                case OP_HEAD: head(op); break;
+            }
+        }
+    }
+};
+
+bool good_linear(const ImparoLinearDesc& l) {
+    return l.weight && l.n > 0 && l.k > 0 && (l.dtype == IMPARO_F32 || l.dtype == IMPARO_BF16);
+}
+
+}  // namespace
+
+extern "C" int imparo_load_code() {
+    const int status[] = {imparo_load_code_attention(), imparo_load_code_attention_mfma(), imparo_load_code_elementwise(),
+                          imparo_load_code_gemm(),      imparo_load_code_rope_cache(),     imparo_load_code_sampling()};
+    for (int s : status)
+        if (s != IMPARO_OK) return s;
+    return IMPARO_OK;
+}
+
+extern "C" ImparoProgram* imparo_program_new(int engine_dtype, int page_size) {
+    if ((engine_dtype != IMPARO_F32 && engine_dtype != IMPARO_BF16) || page_size < 1) return nullptr;
+    ImparoProgram* p = new ImparoProgram();
+    p->engine_dtype = engine_dtype;
+    p->page_size = page_size;
+    // the names are those under which a caller that runs the parts one by one keeps the same buffers
+    p->r_residual = p->region("residual");
+    p->r_normed = p->region("normed");
+    p->r_mixer_in = p->region("mixer_in");
+    p->r_mixer_mid = p->region("mixer_mid");
+    p->r_q = p->region("q");
+    p->r_mixer_out = p->region("mixer_out");
+    p->r_mixer_out_sliced = p->region("mixer_out_sliced");
+    p->r_ffn_out = p->region("ffn_out");
+    p->r_ffn_out_sliced = p->region("ffn_out_sliced");
+    p->r_part_o = p->region("attn_part_o");
+    p->r_part_ml = p->region("attn_part_ml");
+    p->r_prefill_part_o = p->region("attn_prefill_part_o");
+    p->r_prefill_part_ml = p->region("attn_prefill_part_ml");
+    p->r_normed_rows = p->region("normed_rows");
+    p->r_logits = p->region("logits");
+    return p;
+}
+
+extern "C" void imparo_program_delete(ImparoProgram* p) { delete p; }
+
+extern "C" int imparo_program_embedding(ImparoProgram* p, const void* table, int table_dtype, int vocab, int width) {
+    if (!p || !table || vocab < 1 || width < 1 || !p->ops.empty()) return IMPARO_BAD_ARGUMENT;
+    Op op{OP_EMBEDDING};
+    op.table = table;
+    op.table_dtype = table_dtype;
+    op.vocab = vocab;
+    op.width = width;
+    p->ops.push_back(op);
+    return IMPARO_OK;
+}
+
+extern "C" int imparo_program_norm(ImparoProgram* p, const float* weight, float eps, int width, int out_dtype) {
+    if (!p || !weight || width < 1 || p->ops.empty()) return IMPARO_BAD_ARGUMENT;
+    Op op{OP_NORM};
+    op.weight = weight;
+    op.eps = eps;
+    op.width = width;
+    op.out_dtype = out_dtype;
+    p->ops.push_back(op);
+    return IMPARO_OK;
+}
+
+extern "C" int imparo_program_attention(ImparoProgram* p, const ImparoAttentionDesc* d) {
+    if (!p || !d || p->ops.empty() || !good_linear(d->qkv) || !good_linear(d->out)) return IMPARO_BAD_ARGUMENT;
+    if (d->heads < 1 || d->kv_heads < 1 || d->heads % d->kv_heads || d->head_dim < 16 || d->head_dim % 16) return IMPARO_BAD_ARGUMENT;
+    if (d->qkv.n != (d->heads + 2 * d->kv_heads) * d->head_dim || d->out.k != d->heads * d->head_dim) return IMPARO_BAD_ARGUMENT;
+    if (!d->k_cache || !d->v_cache || d->n_pages < 1 || d->group < 0 || d->group >= IMPARO_MAX_GROUPS) return IMPARO_BAD_ARGUMENT;
+    if ((d->q_norm == nullptr) != (d->k_norm == nullptr) || (d->n_freq > 0 && !d->inv_freq)) return IMPARO_BAD_ARGUMENT;
+    Op op{OP_ATTENTION};
+    op.attention = *d;
+    p->ops.push_back(op);
+    return IMPARO_OK;
+}
+
+extern "C" int imparo_program_short_conv(ImparoProgram* p, const ImparoShortConvDesc* d) {
+    if (!p || !d || p->ops.empty() || !good_linear(d->in_proj) || !good_linear(d->out_proj)) return IMPARO_BAD_ARGUMENT;
+    if (d->width < 1 || d->taps < 2 || d->in_proj.n != 3 * d->width || d->out_proj.k != d->width || !d->conv_weight ||
+        !d->state || d->n_slots < 1)
+        return IMPARO_BAD_ARGUMENT;
+    Op op{OP_SHORT_CONV};
+    op.conv = *d;
+    p->ops.push_back(op);
+    return IMPARO_OK;
+}
+
+extern "C" int imparo_program_swiglu(ImparoProgram* p, const ImparoSwigluDesc* d) {
+    if (!p || !d || p->ops.empty() || !good_linear(d->gate_up) || !good_linear(d->down)) return IMPARO_BAD_ARGUMENT;
+    if (d->gate_up.n % 2 || d->down.k != d->gate_up.n / 2) return IMPARO_BAD_ARGUMENT;
+    Op op{OP_SWIGLU};
+    op.swiglu = *d;
+    p->ops.push_back(op);
+    return IMPARO_OK;
+}
+
+extern "C" int imparo_program_head(ImparoProgram* p, const float* norm_weight, float eps, int width,
+                                   const ImparoLinearDesc* head) {
+    if (!p || !norm_weight || !head || p->ops.empty() || !good_linear(*head) || head->k != width) return IMPARO_BAD_ARGUMENT;
+    Op op{OP_HEAD};
+    op.weight = norm_weight;
+    op.eps = eps;
+    op.width = width;
+    op.head = *head;
+    p->ops.push_back(op);
+    return IMPARO_OK;
+}
+
+extern "C" int imparo_program_n_regions(const ImparoProgram* p) { return p ? (int)p->regions.size() : 0; }
+
+extern "C" const char* imparo_program_region_name(const ImparoProgram* p, int region) {
+    if (!p || region < 0 || region >= (int)p->regions.size()) return "";
+    return p->regions[region].name.c_str();
+}
+
+extern "C" int imparo_program_bind(ImparoProgram* p, int region, void* ptr, int64_t bytes) {
+    if (!p || region < 0 || region >= (int)p->regions.size() || bytes < 0 || (bytes > 0 && !ptr)) return IMPARO_BAD_ARGUMENT;
+    if ((uintptr_t)ptr & 15) return IMPARO_BAD_ARGUMENT;       // the kernels load 16 bytes at a time
+    p->regions[region].ptr = (char*)ptr;
+    p->regions[region].bytes = bytes;
+    return IMPARO_OK;
+}
+
+extern "C" int imparo_program_needs(ImparoProgram* p, const ImparoStepArgs* args, int64_t* needs) {
+    if (!p || !args || !needs) return IMPARO_BAD_ARGUMENT;
+    Walk w(p, args, nullptr, true);
+    w.run();
+    for (size_t i = 0; i < w.need.size(); ++i) needs[i] = w.need[i];
+    return w.status;
+}
+
+extern "C" int imparo_program_run(ImparoProgram* p, const ImparoStepArgs* args, float** logits, imparo_stream stream) {
+    if (!p || !args || !logits) return IMPARO_BAD_ARGUMENT;
+    *logits = nullptr;
+    Walk dry(p, args, nullptr, true);
+    dry.run();
+    if (dry.status != IMPARO_OK) return dry.status;
+    for (size_t i = 0; i < dry.need.size(); ++i)
+        if (dry.need[i] > p->regions[i].bytes) {
+            char buf[200];
+            snprintf(buf, sizeof buf, "region %s holds %lld bytes and the step needs %lld", p->regions[i].name.c_str(),
+                     (long long)p->regions[i].bytes, (long long)dry.need[i]);
+            p->error = buf;
+            return IMPARO_SCRATCH_TOO_SMALL;
+        }
+    Walk w(p, args, stream, false);
+    w.run();
+    *logits = w.logits;
+    return w.status;
+}
+
+extern "C" const char* imparo_program_error(const ImparoProgram* p) { return p ? p->error.c_str() : ""; }

@@ -22,6 +22,7 @@ from ..cache.pages import CacheError, CacheManager
 from ..cache.storage import CacheStorage
 from ..config import plan_from_config, read_config_json
 from ..kernels import library, ops
+from ..kernels.program import StepArgs
 from ..parts.base import StepContext, Workspace
 from ..weights import load_weights
 from .model import Model, declared_tensors
@@ -97,6 +98,7 @@ class _DecodeGraph:
         self.last_used = 0
 
 
+REGION_CAP = 256 << 20   # bytes of one scratch region that are reserved up front; beyond that it grows when needed
 TABLE_BUCKET = 8     # captured steps round their block-table width up to a multiple of this many pages, or more
 MAX_GRAPHS = 256     # captured batch shapes kept; beyond that the one unused for longest goes
 
@@ -121,11 +123,16 @@ class Engine:
     from a memory budget the same way and carries a cap in pages for tests,
     /root/reference/crates/imparo-model/src/kv.rs:574-621), or `num_pages`
     gives the pool size outright (one number, or one per cache group).
-    `max_step_tokens` bounds the tokens of one step; a larger batch is refused."""
+    `max_step_tokens` bounds the tokens of one step; a larger batch is refused.
+    `native_step`: a step's kernels are issued by one call into the kernel
+    library (a step program) where every part of the model can describe itself
+    to it; False, or a model with a part that cannot, runs the parts one by one
+    from here. Both issue the same kernels with the same arguments."""
 
     def __init__(self, model_dir: str, dtype: str = "bfloat16", max_tokens: Optional[int] = None, page_size: int = 64,
                  max_requests: int = 64, device: str = "cuda:0", use_graphs: bool = True,
-                 kv_budget_bytes: Optional[int] = None, num_pages=None, max_step_tokens: int = 8192):
+                 kv_budget_bytes: Optional[int] = None, num_pages=None, max_step_tokens: int = 8192,
+                 native_step: bool = True):
         if dtype not in DTYPES:
             raise ValueError(f"dtype must be one of {sorted(DTYPES)}, got {dtype!r}")
         if sum(x is not None for x in (max_tokens, kv_budget_bytes, num_pages)) > 1:
@@ -164,12 +171,18 @@ class Engine:
         # HIP graph: the launches of a step cost more host time than the step's kernels take
         self.use_graphs = use_graphs
         self._graphs: Dict[Tuple[int, int], _DecodeGraph] = {}
-        self._decode_code_loaded = False
         self._graph_pool = None
         self._capture_stream = None
         self.vocab_size = self.plan.vocab_size
         self.max_position = self.plan.max_position
         self.steps_run = 0
+        ops.load_code()                 # every kernel file's code is on the device before any capture
+        self.program = (self.model.build_program(self.storage, self.cache.group_of_site, page_size)
+                        if native_step else None)
+        self._args = StepArgs()
+        self._prefill_tile = ops.prefill_tile()
+        if self.program is not None:
+            self._size_workspace(max_requests)
 
     @staticmethod
     def pool_sizes(site_specs, page_size: int, dtype: torch.dtype, max_tokens: Optional[int],
@@ -257,9 +270,7 @@ class Engine:
                     and bool((batch.n_want == 1).all())):
                 logits = self._decode_step(entries, batch)       # one token each, wanted
             else:
-                ctx, token_ids, want_rows = self._pack(batch)
-                with ops.on_current_stream():
-                    logits = self.model.forward(ctx, token_ids, want_rows)
+                logits = self._run(self._pack(batch))
         except BaseException:
             # Pages and new admissions are rolled back. Fixed-size state is not a thing that can be
             # rolled back (a conv history has been shifted by the layers that ran), so the requests
@@ -290,65 +301,84 @@ class Engine:
         return f"request {e.request!r}: the cache manager refused the step with code {code}"
 
     def _decode_step(self, entries: Sequence[StepEntry], batch) -> torch.Tensor:
-        """A step of single tokens. The engine's first such step runs launch by
-        launch (a capture cannot load code onto the device, and every module of
-        kernels a decode step uses is loaded once one has run); after that a
-        batch shape is captured when it first comes and replayed from then on."""
+        """A step of single tokens: a batch shape is captured when it first
+        comes and replayed from then on."""
         width = table_bucket(batch.widest)
-        key = (len(entries), width)
-        if not self._decode_code_loaded:
-            self._decode_code_loaded = True
-            ctx, token_ids, want_rows = self._pack(batch)
-            with ops.on_current_stream():
-                return self.model.forward(ctx, token_ids, want_rows)
+        g = self._graph_for(len(entries), width)
+        if g.graph is None:
+            self._capture(g, self._pack(batch, table_width=width, graph=g))
+        else:
+            self._pack(batch, table_width=width, graph=g)
+        g.graph.replay()
+        return g.logits
+
+    def _graph_for(self, rows: int, width: int) -> _DecodeGraph:
+        key = (rows, width)
         g = self._graphs.get(key)
         if g is None:
             if len(self._graphs) >= MAX_GRAPHS:      # each holds an executable graph and its index arrays
                 del self._graphs[min(self._graphs, key=lambda k: self._graphs[k].last_used)]
             g = self._graphs[key] = _DecodeGraph()
         g.last_used = self.steps_run
-        if g.graph is None:
-            # the capture fixes grid sizes: they are sized for the widest context the tables can hold
-            ctx, token_ids, want_rows = self._pack(batch, table_width=width, graph=g)
-            if self._graph_pool is None:
-                self._graph_pool = torch.cuda.graph_pool_handle()
-            graph = torch.cuda.CUDAGraph()
-            # Captured by hand, on a stream of its own: the library's context manager waits for the device, collects
-            # garbage and empties the allocator's cache before every capture, which is most of what a new shape costs.
-            if self._capture_stream is None:
-                self._capture_stream = torch.cuda.Stream(device=self.device)
-            here = torch.cuda.current_stream(self.device)
-            self._capture_stream.wait_stream(here)
-            with torch.cuda.stream(self._capture_stream), ops.on_current_stream():
-                graph.capture_begin(pool=self._graph_pool)
-                try:
-                    g.logits = self.model.forward(ctx, token_ids, want_rows)
-                finally:
-                    graph.capture_end()
-            here.wait_stream(self._capture_stream)
-            g.pinned = self.workspace.pin()          # the buffers whose addresses the graph holds
-            g.graph = graph
-        else:
-            self._pack(batch, table_width=width, graph=g)
-        g.graph.replay()
-        return g.logits
+        return g
 
-    def _pack(self, batch, table_width: Optional[int] = None, graph: Optional[_DecodeGraph] = None):
-        """Builds the step's index arrays, sends them to the device in one
-        copy and wraps them in a StepContext. For a captured step the arrays go
-        to the capture's own fixed buffer and sizes are the capture's bounds."""
+    def _capture(self, g: _DecodeGraph, packed: "_Packed") -> None:
+        """Records the step that `packed` describes into `g`. The capture fixes grid sizes: they are
+        sized for the widest context the tables can hold."""
+        if self.program is not None:
+            self._grow_for(packed)                   # a capture must not meet a region that is too small
+        if self._graph_pool is None:
+            self._graph_pool = torch.cuda.graph_pool_handle()
+        graph = torch.cuda.CUDAGraph()
+        # Captured by hand, on a stream of its own: the library's context manager waits for the device, collects
+        # garbage and empties the allocator's cache before every capture, which is most of what a new shape costs.
+        if self._capture_stream is None:
+            self._capture_stream = torch.cuda.Stream(device=self.device)
+        here = torch.cuda.current_stream(self.device)
+        self._capture_stream.wait_stream(here)
+        with torch.cuda.stream(self._capture_stream):
+            graph.capture_begin(pool=self._graph_pool)
+            try:
+                g.logits = self._run(packed)
+            finally:
+                graph.capture_end()
+        here.wait_stream(self._capture_stream)
+        g.pinned = self.workspace.pin()          # the buffers whose addresses the graph holds
+        g.graph = graph
+
+    def warm(self, rows: Sequence[int], contexts: Sequence[int] = (1,)) -> int:
+        """Captures the decode steps of `rows` single-token requests whose longest context is
+        `contexts` tokens, for every pair of the two, before any request needs them: a shape that is
+        met for the first time while serving costs several steps' time. Returns how many shapes it
+        captured. Nothing runs and no request is touched: a capture records launches only."""
+        made = 0
+        if not (self.use_graphs and self.model.graph_safe):
+            return made
+        G = len(self.cache.groups)
+        for n in sorted(set(int(r) for r in rows)):
+            for context in sorted(set(int(c) for c in contexts)):
+                if n < 1 or context < 1:
+                    raise ValueError("warm: rows and contexts are positive numbers")
+                width = table_bucket(-(-context // self.page_size))
+                g = self._graph_for(n, width)
+                if g.graph is not None:
+                    continue
+                lay = dict(T=n, R=n, W=n, G=G, P=width, n_single=n, n_multi=0, max_seg_len=1,
+                           max_context=width * self.page_size, total=3 * n + 4 * n + n + G * n * width)
+                g.meta = torch.zeros(lay["total"] + 2 * n, dtype=torch.int32, device=self.device)
+                self._capture(g, _Packed(g.meta, lay, width * self.page_size, np.ones(n, dtype=np.int32)))
+                made += 1
+        return made
+
+    def _pack(self, batch, table_width: Optional[int] = None, graph: Optional[_DecodeGraph] = None) -> "_Packed":
+        """Builds the step's index arrays and sends them to the device in one
+        copy. For a captured step the arrays go to the capture's own fixed
+        buffer and sizes are the capture's bounds."""
         a, lay = self.cache.pack_batch(batch, table_width or 0)
-        T, R, W, G, P, total = lay["T"], lay["R"], lay["W"], lay["G"], lay["P"], lay["total"]
+        T, R, total = lay["T"], lay["R"], lay["total"]
         placed = batch.device_tokens
         if placed is not None:               # where the ids go, and where they come from, ride along
             a = np.concatenate([a, placed[1], placed[2]])
-        o_pos, o_row = T, 2 * T
-        o_start, o_len, o_slot = 3 * T, 3 * T + R, 3 * T + 2 * R
-        o_lists = 3 * T + 3 * R
-        o_want = 3 * T + 4 * R
-        o_tab = o_want + W
-        o_tok = 0
-        n_dec = lay["n_single"]
         if graph is not None:
             if graph.meta is None:
                 graph.meta = torch.empty(total + 2 * R, dtype=torch.int32, device=self.device)
@@ -357,8 +387,97 @@ class Engine:
             dev = self._upload.send(a)
         if placed is not None:
             n = placed[1].shape[0]
-            ops.place_tokens(dev[o_tok:o_tok + T], dev[total:total + n], placed[0], dev[total + n:total + 2 * n],
-                             self.vocab_size)
+            with ops.on_current_stream():
+                ops.place_tokens(dev[:T], dev[total:total + n], placed[0], dev[total + n:total + 2 * n], self.vocab_size)
+        return _Packed(dev, lay, lay["max_context"] if table_width is None else table_width * self.page_size,
+                       batch.n_tok)
+
+    def _run(self, packed: "_Packed") -> Optional[torch.Tensor]:
+        """Issues the kernels of a packed step on the current stream and returns its logits."""
+        if self.program is None:
+            ctx, token_ids, want_rows = self._context(packed)
+            with ops.on_current_stream():
+                return self.model.forward(ctx, token_ids, want_rows)
+        W = packed.lay["W"]
+        at = self.program.run(self._step_args(packed), self.workspace, torch.cuda.current_stream().cuda_stream)
+        if at is None:
+            return None
+        logits = self.workspace.get("logits", (W, self.vocab_size), torch.float32)
+        assert logits.data_ptr() == at
+        return logits
+
+    def _step_args(self, packed: "_Packed") -> StepArgs:
+        """The packed step as the native program takes it: addresses inside the one device array."""
+        lay = packed.lay
+        T, R, W, G, P = lay["T"], lay["R"], lay["W"], lay["G"], lay["P"]
+        base = packed.dev.data_ptr()
+        n_single = lay["n_single"]
+        at = lambda offset: base + 4 * offset
+        a = self._args
+        a.tokens, a.positions, a.row_of_token = at(0), at(T), at(2 * T)
+        a.seg_start, a.seg_len, a.slot = at(3 * T), at(3 * T + R), at(3 * T + 2 * R)
+        a.single_rows, a.portion_rows = at(3 * T + 3 * R), at(3 * T + 3 * R + n_single)
+        a.want_rows = at(3 * T + 4 * R)
+        tables = 3 * T + 4 * R + W
+        if G > len(a.tables):
+            raise StepError(f"the step program takes {len(a.tables)} cache groups, this model has {G}")
+        for g in range(G):
+            a.tables[g] = at(tables + g * R * P)
+        a.n_groups, a.table_width = G, P
+        a.n_tokens, a.n_rows, a.n_want, a.n_single, a.n_portion = T, R, W, n_single, lay["n_multi"]
+        a.max_seg_len, a.max_context = lay["max_seg_len"], packed.max_context
+        n = packed.host_seg_len
+        tile = self._prefill_tile
+        a.portion_tiles = int(((n[n > 1] + (tile - 1)) // tile).sum()) if lay["n_multi"] else 0
+        return a
+
+    def _grow_for(self, packed: "_Packed") -> None:
+        for name, need in self.program.needs(self._step_args(packed)).items():
+            self.workspace.reserve(name, need)
+
+    def _size_workspace(self, max_requests: int) -> None:
+        """Reserves the program's scratch for the largest steps this engine takes, so that no step
+        meets a buffer that must grow: steps of 1 to `max_requests` single tokens, and steps of one
+        portion of up to `max_step_tokens` tokens, each at the longest context the pools can hold.
+        A region that would pass REGION_CAP is left to grow when a step needs it (the partial
+        results of very long contexts)."""
+        G = len(self.cache.groups)
+        longest = max([self.page_size] + [g.pool.n_pages * self.page_size for g in self.cache.groups])
+        longest = min(longest, self.max_position)
+        a = self._args
+        need: Dict[str, int] = {}
+
+        def shape(T, R, single, context):
+            a.n_groups, a.table_width = G, -(-context // self.page_size)
+            a.n_tokens, a.n_rows, a.n_want = T, R, R
+            a.n_single, a.n_portion = (R, 0) if single else (0, R)
+            a.max_seg_len, a.max_context = (1 if single else T), context
+            a.portion_tiles = 0 if single else -(-T // self._prefill_tile)
+            for name, n in self.program.needs(a).items():
+                need[name] = max(need.get(name, 0), n)
+
+        for rows in range(1, max_requests + 1):
+            shape(rows, rows, True, longest)
+        # (the products' slices of K depend on the rows: every count to 64, then every 16th to 512, then doublings)
+        sizes = {n for n in list(range(2, 65)) + list(range(80, 513, 16)) if n <= self.max_step_tokens}
+        sizes |= {n for n in (1024, 2048, 4096, 8192, 16384) if n < self.max_step_tokens} | {self.max_step_tokens}
+        for tokens in sorted(sizes):
+            shape(tokens, 1, False, min(longest, max(tokens, self.page_size)))
+            shape(tokens, 1, False, longest)
+        for name, n in need.items():
+            self.workspace.reserve(name, min(n, REGION_CAP))
+        self.program.bind(self.workspace)
+
+    def _context(self, packed: "_Packed"):
+        """The packed step as the parts see it when they run one by one."""
+        dev, lay = packed.dev, packed.lay
+        T, R, W, G, P = lay["T"], lay["R"], lay["W"], lay["G"], lay["P"]
+        o_pos, o_row = T, 2 * T
+        o_start, o_len, o_slot = 3 * T, 3 * T + R, 3 * T + 2 * R
+        o_lists = 3 * T + 3 * R
+        o_want = 3 * T + 4 * R
+        o_tab = o_want + W
+        n_dec = lay["n_single"]
         block_tables = {g: dev[o_tab + g * R * P:o_tab + (g + 1) * R * P].view(R, P) for g in range(G)}
         ctx = StepContext(
             n_tokens=T, n_rows=R,
@@ -366,11 +485,19 @@ class Engine:
             seg_start=dev[o_start:o_start + R], seg_len=dev[o_len:o_len + R], slot=dev[o_slot:o_slot + R],
             block_tables=block_tables, page_size=self.page_size, dtype=self.dtype,
             workspace=self.workspace, storage=self.storage, group_of_site=self.cache.group_of_site,
-            max_seg_len=lay["max_seg_len"],
-            max_context=lay["max_context"] if table_width is None else table_width * self.page_size,
+            max_seg_len=lay["max_seg_len"], max_context=packed.max_context,
             single_rows=dev[o_lists:o_lists + n_dec], n_single_rows=n_dec,
             portion_rows=dev[o_lists + n_dec:o_lists + R], n_portion_rows=lay["n_multi"],
-            host_seg_len=batch.n_tok,
+            host_seg_len=packed.host_seg_len,
         )
         want_rows = dev[o_want:o_want + W] if W else None
-        return ctx, dev[o_tok:o_tok + T], want_rows
+        return ctx, dev[:T], want_rows
+
+
+class _Packed:
+    """A step's index arrays on the device (one int32 array, laid out as the cache manager packs
+    them), the sizes of its parts, the bound on every row's context, tokens per row on the host."""
+    __slots__ = ("dev", "lay", "max_context", "host_seg_len")
+
+    def __init__(self, dev: torch.Tensor, lay: Dict[str, int], max_context: int, host_seg_len):
+        self.dev, self.lay, self.max_context, self.host_seg_len = dev, lay, max_context, host_seg_len

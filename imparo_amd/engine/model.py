@@ -15,7 +15,7 @@ import torch
 from ..cache.pages import StateSpec
 from ..config.plan import ModelPlan, PartSpec
 from ..parts import part_class
-from ..parts.base import Declared, Residual, StepContext
+from ..parts.base import Declared, Residual, StepContext, emits
 
 
 def _declare(role: str, spec: PartSpec) -> Declared:
@@ -91,6 +91,24 @@ class Model:
             return None
         h = self.final_norm.forward_rows(ctx, res, want_rows, self.head.in_dtype)
         return self.head.forward(ctx, h)
+
+    def build_program(self, storage, group_of_site: Dict[int, int], page_size: int):
+        """The run order as a native step program (one call issues a step's
+        kernels), or None if some part cannot append itself to one: a part
+        registered from outside, say; the parts then run one by one."""
+        from ..kernels.program import MAX_GROUPS, Program
+        if len(set(group_of_site.values())) > MAX_GROUPS:
+            return None
+        blocks_emit = all(emits(b) and getattr(b, "can_emit", lambda: True)() for b in self.blocks)
+        if not (blocks_emit and emits(self.embedding) and emits(self.final_norm, "emit_head", "forward_rows")
+                and emits(self.head, "emit_projection")):
+            return None
+        program = Program(self.dtype, page_size, storage, group_of_site)
+        self.embedding.emit(program)
+        for i, call in enumerate(self.plan.order):
+            self.blocks[call.layer].emit(program, self.site_of_call[i], call.cache_of is None)
+        self.final_norm.emit_head(program, self.head.emit_projection())
+        return program
 
     def weight_bytes(self) -> int:
         seen, total = set(), 0

@@ -49,6 +49,22 @@ _SIGNATURES = {
     "imparo_fill_f32": [P, F, c_int64, P],
     "imparo_fill_sites": [P, P, P, I, I, P],
     "imparo_attention_decode_static": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
+    "imparo_load_code": [],
+    # a model's step as one call (kernels/program.py holds the structures)
+    "imparo_program_new": ([I, I], P),
+    "imparo_program_delete": ([P], None),
+    "imparo_program_embedding": [P, P, I, I, I],
+    "imparo_program_norm": [P, P, F, I, I],
+    "imparo_program_attention": [P, P],
+    "imparo_program_short_conv": [P, P],
+    "imparo_program_swiglu": [P, P],
+    "imparo_program_head": [P, P, F, I, P],
+    "imparo_program_n_regions": [P],
+    "imparo_program_region_name": ([P, I], ctypes.c_char_p),
+    "imparo_program_bind": [P, I, P, c_int64],
+    "imparo_program_needs": [P, P, P],
+    "imparo_program_run": [P, P, P, P],
+    "imparo_program_error": ([P], ctypes.c_char_p),
 }
 
 
@@ -85,8 +101,10 @@ def library() -> ctypes.CDLL:
             except AttributeError:
                 raise KernelLibraryError(f"{path} lacks the entry point {name}; rebuild it "
                                          f"(python -m imparo_amd.csrc.build)") from None
-            fn.argtypes = argtypes
-            fn.restype = c_int
+            if isinstance(argtypes, tuple):          # (arguments, what it returns) where that is no status
+                fn.argtypes, fn.restype = argtypes
+            else:
+                fn.argtypes, fn.restype = argtypes, c_int
         _lib = lib
         return _lib
 

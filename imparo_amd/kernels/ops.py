@@ -78,6 +78,12 @@ def _check(status: int, name: str) -> None:
     raise KernelArgumentError(f"{name}: {why}")
 
 
+def load_code() -> None:
+    """Loads every kernel file's code onto the current device (the runtime would do so at each
+    file's first launch, which a stream under graph capture cannot)."""
+    _check(library().imparo_load_code(), "load_code")
+
+
 def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     vocab, width = table.shape
     n = ids.shape[0]

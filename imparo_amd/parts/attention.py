@@ -160,4 +160,20 @@ class Attention:
         return self.out(ctx, o, torch.float32, "mixer_out", sliced_ok=True, into=ctx.stream)
 
 
+    def emit(self, program, site: int, owns_cache: bool) -> None:
+        """Appends `forward` to a native step program."""
+        from ..kernels.program import AttentionDesc
+        arrays = program.storage.paged[site]
+        k_cache, v_cache = arrays["k"], arrays["v"]
+        inv_freq = self.position.inv_freq
+        program.attention(AttentionDesc(
+            program.linear(self.qkv), program.linear(self.out),
+            program._hold(self.q_norm, "q norm weight", torch.float32),
+            program._hold(self.k_norm, "k norm weight", torch.float32), self.norm_eps,
+            program._hold(inv_freq, "inverse frequencies", torch.float32), 0 if inv_freq is None else inv_freq.shape[0],
+            int(bool(getattr(self.position, "interleaved", False))), self.heads, self.kv_heads, self.head_dim,
+            self.scale, int(self.window or 0), program._hold(k_cache, "k cache"), program._hold(v_cache, "v cache"),
+            k_cache.shape[0], int(self.v_transposed), program.group_of_site[site], int(owns_cache)))
+
+
 register_part("mixer", "attention", Attention)

@@ -36,6 +36,21 @@ class Workspace:
     def __init__(self, device: torch.device):
         self.device = device
         self._buffers: Dict[str, torch.Tensor] = {}      # by name or alias group: raw bytes
+        self.version = 0                                 # counts new buffers: who keeps addresses looks here
+
+    def reserve(self, key: str, nbytes: int) -> torch.Tensor:
+        """Makes the buffer of a name (or alias group) at least `nbytes` large and returns it."""
+        buf = self._buffers.get(key)
+        if buf is None or buf.numel() < nbytes:
+            grown = nbytes if buf is None else max(nbytes, 2 * buf.numel())
+            buf = torch.empty((max(grown, 1) + 255) // 256 * 256, dtype=torch.uint8, device=self.device)
+            self._buffers[key] = buf
+            self.version += 1
+        return buf
+
+    def buffer(self, key: str) -> Optional[torch.Tensor]:
+        """The buffer of a name or alias group as it is now, or None."""
+        return self._buffers.get(key)
 
     def get(self, name: str, shape: Tuple[int, ...], dtype: torch.dtype, alias: Optional[str] = None) -> torch.Tensor:
         n = 1
@@ -45,9 +60,7 @@ class Workspace:
         key = alias or name
         buf = self._buffers.get(key)
         if buf is None or buf.numel() < need:
-            grown = need if buf is None else max(need, 2 * buf.numel())
-            buf = torch.empty((grown + 255) // 256 * 256, dtype=torch.uint8, device=self.device)
-            self._buffers[key] = buf
+            buf = self.reserve(key, need)
         return buf[:n * _ELEMENT_SIZE[dtype]].view(dtype).view(shape)
 
     def pin(self) -> list:
@@ -110,6 +123,16 @@ class StepContext:
 
     def fixed_state(self, site: int) -> torch.Tensor:
         return self.storage.fixed[site]
+
+
+def emits(part, emit: str = "emit", forward: str = "forward") -> bool:
+    """Whether a part can append itself to a native step program: it has the
+    method `emit`, and no class below the one that defines it has replaced
+    `forward`, the method it describes (a subclass that computes something
+    else must not inherit the description of what its parent computes)."""
+    owner_of = lambda name: next((i for i, c in enumerate(type(part).__mro__) if name in c.__dict__), None)
+    e, f = owner_of(emit), owner_of(forward)
+    return e is not None and (f is None or e <= f)
 
 
 @dataclass

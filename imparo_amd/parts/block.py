@@ -8,7 +8,7 @@ from __future__ import annotations
 
 from typing import Dict
 
-from .base import Residual, StepContext
+from .base import Residual, StepContext, emits
 from .registry import register_part
 
 
@@ -31,6 +31,16 @@ class PreNormBlock:
         res.pending = self._delta(ctx, res, lambda: self.mixer.forward(ctx, site, owns_cache, h))
         n = self.ffn_norm.forward(ctx, res, self.ffn.in_dtype)
         res.pending = self._delta(ctx, res, lambda: self.ffn.forward(ctx, n))
+
+    def can_emit(self) -> bool:
+        return all(emits(p) for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn))
+
+    def emit(self, program, site: int, owns_cache: bool) -> None:
+        """Appends `forward` to a native step program: the four parts in the order they run."""
+        self.mixer_norm.emit(program, self.mixer.in_dtype)
+        self.mixer.emit(program, site, owns_cache)
+        self.ffn_norm.emit(program, self.ffn.in_dtype)
+        self.ffn.emit(program)
 
     @staticmethod
     def _delta(ctx: StepContext, res: Residual, run):

@@ -36,6 +36,10 @@ class Embedding:
         x = ctx.workspace.get("residual", (token_ids.shape[0], self.width), torch.float32)
         return ops.embed_gather(self.table, token_ids, x)
 
+    def emit(self, program) -> None:
+        """Appends `forward` to a native step program."""
+        program.embedding(self.table, self.vocab, self.width)
+
 
 class LinearHead:
     role = "head"
@@ -59,6 +63,10 @@ class LinearHead:
 
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         return self.proj(ctx, h, torch.float32, "logits")
+
+    def emit_projection(self) -> Linear:
+        """What `forward` computes, for a native step program: this projection, float32 out."""
+        return self.proj
 
 
 register_part("embedding", "embedding", Embedding)

@@ -68,4 +68,10 @@ class SwiGlu:
         return self.down(ctx, g, torch.float32, "ffn_out", sliced_ok=True, into=ctx.stream)
 
 
+    def emit(self, program) -> None:
+        """Appends `forward` to a native step program."""
+        from ..kernels.program import SwigluDesc
+        program.swiglu(SwigluDesc(program.linear(self.gate_up), program.linear(self.down)))
+
+
 register_part("feed_forward", "swiglu", SwiGlu)

@@ -41,6 +41,14 @@ class RmsNorm:
             ops.rms_norm(res.x, self.weight, self.eps, out)
         return out
 
+    def emit(self, program, out_dtype: torch.dtype) -> None:
+        """Appends `forward` to a native step program."""
+        program.norm(self.weight, self.eps, self.width, out_dtype)
+
+    def emit_head(self, program, head_linear) -> None:
+        """Appends `forward_rows` followed by the head's projection."""
+        program.head(self.weight, self.eps, self.width, head_linear)
+
     def forward_rows(self, ctx: StepContext, res: Residual, rows: torch.Tensor, out_dtype: torch.dtype,
                      name: str = "normed_rows") -> torch.Tensor:
         """Norm of selected rows only (the rows whose logits are wanted); the

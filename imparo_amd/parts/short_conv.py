@@ -79,4 +79,17 @@ class ShortConv:
         return self.out_proj(ctx, y, torch.float32, "mixer_out", sliced_ok=True, into=ctx.stream)
 
 
+    def emit(self, program, site: int, owns_cache: bool) -> None:
+        """Appends `forward` to a native step program."""
+        from ..kernels.program import ShortConvDesc
+        if not owns_cache:
+            raise ValueError("a short conv's state cannot be read from another layer")
+        state = program.storage.fixed[site]
+        program.short_conv(ShortConvDesc(
+            program.linear(self.in_proj), program.linear(self.out_proj),
+            program._hold(self.conv_weight, "conv weight", torch.float32),
+            program._hold(self.conv_bias, "conv bias", torch.float32),
+            self.width, self.taps, program._hold(state, "conv state", torch.float32), state.shape[0]))
+
+
 register_part("mixer", "short_conv", ShortConv)
