@@ -110,6 +110,77 @@ def prefill_run(engine, tokens, vocab, reps, seed):
     return times
 
 
+def small_steps(engine, vocab, seed):
+    """Steps whose kernels take about as long as a caller needs to issue them: eight decoding
+    requests beside a 32-token portion of a prompt, and a 128-token prompt alone; neither is a
+    captured graph. For each: `ms`, a step as the engine runs it, one after the other; `gpu_ms`, its
+    kernels back to back (the step is queued while the GPU is still busy with something else, then
+    timed between two events); `host_ms`, what the host needs to check, pack and issue it when the
+    GPU is idle. A step is bound by the host where ms is well above gpu_ms."""
+    import torch
+    from imparo_amd.engine import StepEntry
+    g = torch.Generator().manual_seed(seed)
+    draw = lambda n: torch.randint(0, vocab, (n,), generator=g).tolist()
+    busy_a = torch.randn(4096, 4096, device=engine.device, dtype=torch.bfloat16)
+
+    def keep_gpu_busy():                       # a few milliseconds of work that has nothing to do with the step
+        for _ in range(24):
+            torch.mm(busy_a, busy_a)
+
+    def measure(make_step, after_step, reps=12):
+        for _ in range(3):
+            make_step()
+            after_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            make_step()
+            after_step()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) / reps
+        gpu, host = [], []
+        for _ in range(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            make_step()
+            host.append(time.perf_counter() - t0)
+            after_step()
+            keep_gpu_busy()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            make_step()
+            e1.record()
+            after_step()
+            torch.cuda.synchronize()
+            gpu.append(e0.elapsed_time(e1) * 1e-3)
+        return {"ms": round(wall * 1e3, 4), "gpu_ms": round(median(gpu) * 1e3, 4), "host_ms": round(median(host) * 1e3, 4)}
+
+    out = {}
+    ids = [f"s{i}" for i in range(8)]
+    for rid in ids:
+        engine.step([StepEntry(rid, draw(600), [])])
+    portion = draw(32)
+
+    def mixed():
+        engine.step([StepEntry(rid, [7], [0]) for rid in ids] + [StepEntry("sp", portion, [31])])
+
+    def mixed_after():
+        if engine.length("sp") >= 1024:
+            engine.release("sp")
+        if engine.length(ids[0]) >= 1500:
+            for rid in ids:
+                engine.release(rid)
+                engine.step([StepEntry(rid, draw(600), [])])
+
+    out["mixed_small"] = dict(measure(mixed, mixed_after), decode_rows=8, portion_tokens=32)
+    for rid in ids + ["sp"]:
+        engine.release(rid)
+    prompt = draw(128)
+    out["prefill_128"] = dict(measure(lambda: engine.step([StepEntry("s128", prompt, [127])]),
+                                      lambda: engine.release("s128")), tokens=128)
+    return out
+
+
 def median(xs):
     xs = sorted(xs)
     n = len(xs)
@@ -406,6 +477,7 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b * k / d, 1)
             points[f"decode_b{b}_ms_per_step"] = round(d / k * 1e3, 4)
             points[f"decode_b{b}_frac"] = round(step_bytes(b, k) / (d / k) / 1e9 / HBM_PEAK_GBS, 4)
+        points.update(small_steps(engine, c.vocab_size, 5))
         line["points"] = points
     print(json.dumps(line), flush=True)
     return 0

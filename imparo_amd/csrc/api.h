@@ -137,6 +137,8 @@ int imparo_attention_decode_static(const void* q, const void* k_cache, const voi
 // imparo_attention_prefill_splits, or 1) parts of each block's keys, merged by a
 // second launch; then part_o holds [tokens, heads, n_splits, head_dim] floats
 // and part_ml [tokens, heads, n_splits, 2], tokens counted over the whole batch.
+// `max_context` is the bound on the contexts that imparo_attention_prefill itself goes by: what its
+// block table can hold, table_stride x page_size (both lay a launch out from that one number).
 int imparo_attention_prefill_splits(int n_tiles, int heads, int kv_heads, int head_dim, int max_context);
 int imparo_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
                              float* part_o, float* part_ml, int n_splits,

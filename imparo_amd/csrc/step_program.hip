@@ -241,7 +241,7 @@ struct Walk {
                 });
             }
             if (a->n_portion) {
-                const int parts = imparo_attention_prefill_splits(a->portion_tiles, d.heads, d.kv_heads, d.head_dim, a->max_context);
+                const int parts = imparo_attention_prefill_splits(a->portion_tiles, d.heads, d.kv_heads, d.head_dim, stride * p->page_size);
                 float *part_o = nullptr, *part_ml = nullptr;
                 if (parts > 1) {
                     part_o = (float*)get(p->r_prefill_part_o, (int64_t)T * d.heads * parts * d.head_dim * 4);

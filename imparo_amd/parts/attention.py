@@ -141,8 +141,9 @@ class Attention:
             if ctx.n_portion_rows:
                 # few queries over long contexts: each block's keys in parts, merged by a second launch
                 n_tiles = self._portion_tiles(ctx)
+                # (the bound on the contexts that the launch itself sees: what its block table can hold)
                 parts = ops.attention_prefill_splits(n_tiles, self.heads, self.kv_heads, self.head_dim,
-                                                     ctx.max_context)
+                                                     table.shape[1] * ctx.page_size)
                 part_o = part_ml = None
                 if parts > 1:
                     part_o = ctx.workspace.get("attn_prefill_part_o", (T * self.heads * parts * self.head_dim,),

@@ -46,7 +46,10 @@ class SamplingParams:
 class PendingPick:
     """Token ids that the sampling kernel has been asked for. `on_device` is
     the int32 vector they land in (to feed the next step from, without
-    waiting); `tokens()` waits for the copy to the host and returns them."""
+    waiting); `tokens()` waits for the copy to the host and returns them.
+    The vectors are the sampler's own and are used again after `Sampler.RING`
+    further picks: feed `on_device` to the next step or two, not later (the
+    ids themselves are read out in time by the sampler if the caller has not)."""
 
     def __init__(self, on_device, host, event):
         self.on_device = on_device
@@ -61,31 +64,63 @@ class PendingPick:
         return self._tokens
 
 
+class _PickBuffers:
+    """What one pick needs, allocated once: the ids on the device and in pinned host memory,
+    temperatures and uniform numbers in pinned host memory and on the device."""
+
+    def __init__(self, torch, device, capacity: int):
+        self.capacity = capacity
+        self.ids = torch.empty(capacity, dtype=torch.int32, device=device)
+        self.ids_host = torch.empty(capacity, dtype=torch.int32, pin_memory=True)
+        self.params_host = torch.empty(2, capacity, dtype=torch.float32, pin_memory=True)
+        self.params = torch.empty(2, capacity, dtype=torch.float32, device=device)
+        self.last: Optional[PendingPick] = None
+
+
 class Sampler:
-    """Runs the sampling kernels over the logits rows a step returned."""
+    """Runs the sampling kernels over the logits rows a step returned. Its
+    buffers go round in a ring, so a pick allocates nothing once the ring has
+    seen the batch size."""
+    RING = 8
 
     def __init__(self, device):
         import torch
         self.device = device
         self._torch = torch
+        self._ring: List[Optional[_PickBuffers]] = [None] * self.RING
+        self._turn = 0
+
+    def _buffers(self, n: int) -> _PickBuffers:
+        i = self._turn
+        self._turn = (i + 1) % self.RING
+        b = self._ring[i]
+        if b is not None and b.last is not None:
+            b.last.tokens()          # whoever still holds that pick finds its ids read out; the buffers are free
+            b.last = None
+        if b is None or b.capacity < n:
+            b = self._ring[i] = _PickBuffers(self._torch, self.device, max(64, 1 << (n - 1).bit_length()))
+        return b
 
     def pick_async(self, logits, temperatures: Sequence[float], uniforms: Sequence[float]) -> PendingPick:
         """Queues the kernel and the copy of its result to the host; returns at once."""
         torch = self._torch
         from ..kernels import ops
         n = logits.shape[0]
-        out = torch.empty(n, dtype=torch.int32, device=logits.device)
+        b = self._buffers(n)
+        out = b.ids[:n]
         if all(t <= 0 for t in temperatures):
             ops.argmax_rows(logits, out)
         else:
-            host = torch.tensor([list(temperatures), list(uniforms)], dtype=torch.float32, pin_memory=True)
-            dev = host.to(logits.device, non_blocking=True)
-            ops.sample_rows(logits, dev[0], dev[1], out)
-        back = torch.empty(n, dtype=torch.int32, pin_memory=True)
+            b.params_host[0, :n] = torch.tensor(list(temperatures), dtype=torch.float32)
+            b.params_host[1, :n] = torch.tensor(list(uniforms), dtype=torch.float32)
+            b.params.copy_(b.params_host, non_blocking=True)
+            ops.sample_rows(logits, b.params[0, :n], b.params[1, :n], out)
+        back = b.ids_host[:n]
         back.copy_(out, non_blocking=True)
         event = torch.cuda.Event()
         event.record()
-        return PendingPick(out, back, event)
+        b.last = PendingPick(out, back, event)
+        return b.last
 
     def pick(self, logits, temperatures: Sequence[float], uniforms: Sequence[float]) -> List[int]:
         return self.pick_async(logits, temperatures, uniforms).tokens()
