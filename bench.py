@@ -66,7 +66,7 @@ def decode_run(engine, sampler, batch, context, steps, warmup, vocab, seed):
         for lo in range(0, start, 2048):
             hi = min(start, lo + 2048)
             out = engine.step([StepEntry(rid, prompt[lo:hi], [hi - lo - 1] if hi == start else [])])
-        last = out if last is None else torch.cat([last, out])
+        last = out.clone() if last is None else torch.cat([last, out])
     temps, unis = [0.0] * batch, [0.0] * batch
     picked = sampler.pick_async(last, temps, unis)
 
@@ -199,6 +199,24 @@ def shape(hidden, heads, block_ff_dim):
     return cfg
 
 
+LFM2_700M = shape(1536, 24, 10240)
+LFM2_350M = shape(1024, 16, 6656)
+
+
+def build_engine(cfg, seed, dtype, **kw):
+    """Random weights of `cfg` drawn from `seed`, written to a temporary folder, loaded, and the folder removed."""
+    from imparo_amd import write_random_model
+    from imparo_amd.engine import Engine
+    tmp = tempfile.mkdtemp(prefix="imparo_bench_")
+    try:
+        write_random_model(cfg, seed, tmp)
+        return Engine(tmp, dtype=dtype, page_size=64, **kw)
+    finally:
+        for f in os.listdir(tmp):
+            os.remove(os.path.join(tmp, f))
+        os.rmdir(tmp)
+
+
 class StepClock:
     """Stands between the scheduler and the engine and notes, for every step, what it fed and a GPU
     event at its start: the time from one step's event to the next is that step's time on the GPU
@@ -259,30 +277,32 @@ class StepClock:
         return out
 
 
-def serving_workload(dtype):
+def serving_workload(dtype, engine=None):
     """Continuous batching: 32 requests, prompts of 64..3072 tokens, replies of 32..512 tokens, in 4
-    waves of 8 (a wave every 48 steps), 512-token portions beside decoded tokens. LFM2-700M shape."""
+    waves of 8 (a wave every 48 steps), 512-token portions beside decoded tokens. LFM2-700M shape.
+    The decode steps' graphs are captured before the clock starts (Scheduler.warm), as a server
+    would do at start-up. Returns the record."""
     import numpy as np
     import torch
-    from imparo_amd import write_random_model
-    from imparo_amd.engine import Engine
     from imparo_amd.engine.scheduler import Scheduler
     from imparo_amd.sampling import Sampler, SamplingParams
-    cfg = shape(1536, 24, 10240)
+    cfg = LFM2_700M
     nums = model_numbers(cfg)
-    tmp = tempfile.mkdtemp(prefix="imparo_bench_")
-    write_random_model(cfg, 3, tmp)
     elem = 2 if dtype == "bfloat16" else 4
-    engine = StepClock(Engine(tmp, dtype=dtype, max_tokens=32 * (3072 + 512 + 64), page_size=64, max_requests=32),
-                       nums["layer_params"] * elem, nums["head_params"] * elem, nums["kv_bytes_per_token"] * elem // 2,
-                       2.0 * nums["layer_params"])
+    if engine is None:
+        engine = build_engine(cfg, 3, dtype, max_tokens=32 * (3072 + 512 + 64), max_requests=32)
+    engine = StepClock(engine, nums["layer_params"] * elem, nums["head_params"] * elem,
+                       nums["kv_bytes_per_token"] * elem // 2, 2.0 * nums["layer_params"])
     sampler = Sampler(engine.device)
     rng = np.random.default_rng(3)
     jobs = [(i, rng.integers(0, cfg["vocab_size"], size=int(rng.integers(64, 3073))).tolist(), int(rng.integers(32, 513)))
             for i in range(32)]
     sched = Scheduler(engine, sampler.pick, max_batch_tokens=2048, max_running=32, portion=512,
                       pick_async=sampler.pick_async)
+    t_warm = time.perf_counter()
+    warmed = sched.warm(3072 + 512)
     torch.cuda.synchronize()
+    t_warm = time.perf_counter() - t_warm
     t0 = time.perf_counter()
     steps = 0
     while jobs or sched.has_work():
@@ -299,30 +319,28 @@ def serving_workload(dtype):
     n_out = sum(len(r.generated) for r in done.values())
     assert len(done) == 32 and all(r.finish_reason == "length" for r in done.values())
     c = nums["cfg"]
-    print(json.dumps({
+    return {
         "metric": "continuous batching, LFM2-700M shape: generated tok/s over the whole run", "value": round(n_out / dt, 1),
         "unit": "tok/s", "n_gpus": 1, "seconds": round(dt, 3), "steps": steps, "prompt_tokens": n_prompt,
         "generated_tokens": n_out, "all_tokens_per_s": round((n_prompt + n_out) / dt, 1),
         "preemptions": sum(r.preemptions for r in done.values()), "dtype": "bf16" if dtype == "bfloat16" else "fp32",
         "data": "synthetic token ids, random weights (seed 3)",
+        "graphs_captured_before_the_clock": warmed, "seconds_to_capture_them": round(t_warm, 3),
         "step_times": engine.by_kind(HBM_PEAK_GBS, MFMA_PEAK["bf16" if dtype == "bfloat16" else "fp32"]),
         "config": {"model": "LFM2-700M shape", "requests": 32, "waves": 4, "portion": 512, "max_batch_tokens": 2048,
                    "hidden_size": c.hidden_size, "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads,
-                   "ff_dim": c.ff_dim, "layers": c.num_hidden_layers}}), flush=True)
-    return 0
+                   "ff_dim": c.ff_dim, "layers": c.num_hidden_layers}}
 
 
-def long_workload(dtype, requests, prompt_len, portion=2048):
+def long_workload(dtype, requests, prompt_len, portion=2048, quiet=False, engine=None):
     """Long contexts: `requests` concurrent requests, each a prompt of `prompt_len` tokens fed in
-    portions of `portion` tokens (2,048), then 128 decoded tokens each. LFM2-350M shape."""
+    portions of `portion` tokens (2,048), then 128 decoded tokens each. LFM2-350M shape. Returns the record."""
     import torch
-    from imparo_amd import write_random_model
-    from imparo_amd.engine import DeviceToken, Engine, StepEntry
+    from imparo_amd.engine import DeviceToken, StepEntry
     from imparo_amd.sampling import Sampler
-    cfg = shape(1024, 16, 6656)
-    tmp = tempfile.mkdtemp(prefix="imparo_bench_")
-    write_random_model(cfg, 4, tmp)
-    engine = Engine(tmp, dtype=dtype, max_tokens=requests * (prompt_len + 128 + 64), page_size=64, max_requests=requests)
+    cfg = LFM2_350M
+    if engine is None:
+        engine = build_engine(cfg, 4, dtype, max_tokens=requests * (prompt_len + 128 + 64), max_requests=requests)
     sampler = Sampler(engine.device)
     g = torch.Generator().manual_seed(4)
     ids = list(range(requests))
@@ -331,11 +349,12 @@ def long_workload(dtype, requests, prompt_len, portion=2048):
     last = []
     for rid in ids:
         prompt = torch.randint(0, cfg["vocab_size"], (prompt_len,), generator=g).tolist()
+        out = None
         for lo in range(0, prompt_len, portion):
             hi = min(prompt_len, lo + portion)
             out = engine.step([StepEntry(rid, prompt[lo:hi], [hi - lo - 1] if hi == prompt_len else [])])
-        last.append(out)
-        if rid % 8 == 7:
+        last.append(out.clone())                   # (the engine's next step writes its logits where these lie)
+        if rid % 8 == 7 and not quiet:
             print(f"[bench] {rid + 1} of {requests} prompts are in the cache", file=sys.stderr, flush=True)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
@@ -349,16 +368,23 @@ def long_workload(dtype, requests, prompt_len, portion=2048):
     picked.tokens()
     torch.cuda.synchronize()
     t2 = time.perf_counter()
-    print(json.dumps({
+    pages_used = engine.cache.groups[0].pool.n_pages - engine.free_pages()[0]
+    for rid in ids:
+        engine.release(rid)
+    nums = model_numbers(cfg)
+    step_bytes = ((nums["layer_params"] + nums["head_params"]) * 2
+                  + requests * ((prompt_len + 64) * nums["kv_bytes_per_token"] + nums["conv_state_bytes"]))
+    return {
         "metric": "long contexts, LFM2-350M shape: decode tok/s with every request at its full context",
         "value": round(requests * 127 / (t2 - t1), 1), "unit": "tok/s", "n_gpus": 1,
         "prefill_tok_s": round(requests * prompt_len / (t1 - t0), 1), "prefill_seconds": round(t1 - t0, 3),
-        "decode_ms_per_step": round((t2 - t1) / 127 * 1e3, 3), "dtype": "bf16" if dtype == "bfloat16" else "fp32",
+        "decode_ms_per_step": round((t2 - t1) / 127 * 1e3, 3),
+        "decode_hbm_frac": round(step_bytes / ((t2 - t1) / 127) / 1e9 / HBM_PEAK_GBS, 4),
+        "dtype": "bf16" if dtype == "bfloat16" else "fp32",
         "data": "synthetic token ids, random weights (seed 4)",
         "config": {"model": "LFM2-350M shape", "requests": requests, "prompt_len": prompt_len, "portion": portion,
                    "decode_tokens": 128, "hidden_size": 1024, "heads": 16, "kv_heads": 8, "ff_dim": 4608, "layers": 16,
-                   "cache_pages_used": engine.cache.groups[0].pool.n_pages - engine.free_pages()[0]}}), flush=True)
-    return 0
+                   "cache_pages_used": pages_used}}
 
 
 def main() -> int:
@@ -384,13 +410,13 @@ def main() -> int:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
     if args.workload == "serving":
-        return serving_workload(args.dtype)
+        print(json.dumps(serving_workload(args.dtype)), flush=True)
+        return 0
     if args.workload == "long":
-        return long_workload(args.dtype, args.requests, args.prompt_len, args.portion)
+        print(json.dumps(long_workload(args.dtype, args.requests, args.prompt_len, args.portion)), flush=True)
+        return 0
 
     import torch
-    from imparo_amd import write_random_model
-    from imparo_amd.engine import Engine
     from imparo_amd.sampling import Sampler
 
     cfg = dict(LFM2_1_2B)
@@ -400,33 +426,35 @@ def main() -> int:
         cfg["layer_types"] = cfg["layer_types"][:args.layers]
     nums = model_numbers(cfg)
     c = nums["cfg"]
-    tmp = tempfile.mkdtemp(prefix="imparo_bench_")
     print(f"[bench] writing random weights ({(nums['layer_params'] + nums['head_params']) / 1e9:.2f} B parameters) ...",
           file=sys.stderr, flush=True)
-    write_random_model(cfg, 2, tmp)
-    biggest = max(args.batch, 1 if (args.no_points or args.prefill_only) else 64)
-    engine = Engine(tmp, dtype=args.dtype, max_tokens=biggest * (args.context + 64), page_size=64,
-                    max_requests=biggest)
-    for f in os.listdir(tmp):
-        os.remove(os.path.join(tmp, f))
-    os.rmdir(tmp)
+    further = not (args.no_points or args.prefill_only)
+    # the pools hold the largest point: 256 requests at the context (which also holds 8 at 32,768)
+    biggest = max(args.batch, 256 if further else 1)
+    engine = build_engine(cfg, 2, args.dtype, max_tokens=biggest * (args.context + 64), max_requests=biggest,
+                          max_step_tokens=32768 if further else 8192)
     sampler = Sampler(engine.device)
     elem = 2 if args.dtype == "bfloat16" else 4
+    peak = MFMA_PEAK["bf16" if args.dtype == "bfloat16" else "fp32"]
     if args.prefill_only:
         pts = prefill_run(engine, 2048, c.vocab_size, 5, 3)
         print(json.dumps({"prefill_ms": round(median(pts) * 1e3, 3), "tokens": 2048,
                           "all_ms": [round(t * 1e3, 3) for t in pts]}), flush=True)
         return 0
 
-    def step_bytes(batch, steps):
+    def step_bytes(batch, steps, context=None):
         """Bytes one decode step has to read: every weight once, the cache of the live requests."""
-        mean_ctx = args.context - steps / 2
+        mean_ctx = (context or args.context) - steps / 2
         return ((nums["layer_params"] + nums["head_params"]) * elem
                 + batch * (mean_ctx * nums["kv_bytes_per_token"] * elem / 2 + nums["conv_state_bytes"]))
 
-    # Every figure is the median of PASSES measurements taken in turn (batch 8, batch 1, batch 64,
-    # prefill, and again), so that a slow moment of the machine does not fall on one of them alone.
-    # A decode measurement is W warmup steps and exactly K timed steps, each time on freshly filled contexts.
+    def prefill_flops(T):
+        return 2.0 * T * nums["layer_params"] + 2.0 * nums["head_params"] + nums["attn_flops_per_pair"] * T * (T + 1) / 2
+
+    # Every figure of the headline and of the points at batch 1 and 64 is the median of PASSES measurements
+    # taken in turn (batch 8, batch 1, batch 64, prefill, and again), so that a slow moment of the machine
+    # does not fall on one of them alone. A decode measurement is W warmup steps and exactly K timed steps,
+    # each time on freshly filled contexts.
     PASSES = 3
     points_steps = max(8, args.steps // 2)
     widths = [args.batch] + ([] if args.no_points else [b for b in (1, 64) if b != args.batch])
@@ -465,22 +493,74 @@ def main() -> int:
     }
     if not args.no_points:
         pt = median(prefills)
-        flops = 2.0 * T * nums["layer_params"] + 2.0 * nums["head_params"] + nums["attn_flops_per_pair"] * T * (T + 1) / 2
-        peak = MFMA_PEAK["bf16" if args.dtype == "bfloat16" else "fp32"]
         line["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
-                           "frac": round(flops / pt / peak, 4), "runs": len(prefills),
+                           "frac": round(prefill_flops(T) / pt / peak, 4), "runs": len(prefills),
                            "min_ms": round(min(prefills) * 1e3, 3), "max_ms": round(max(prefills) * 1e3, 3)}
         points = {}
+
+        def decode_point(name, b, k, d, context=None):
+            points[name] = round(b * k / d, 1)
+            points[name + "_ms_per_step"] = round(d / k * 1e3, 4)
+            points[name + "_frac"] = round(step_bytes(b, k, context) / (d / k) / 1e9 / HBM_PEAK_GBS, 4)
+
         for b in (1, 64):
-            k = args.steps if b == args.batch else points_steps
-            d = median(seconds[b])
-            points[f"decode_b{b}"] = round(b * k / d, 1)
-            points[f"decode_b{b}_ms_per_step"] = round(d / k * 1e3, 4)
-            points[f"decode_b{b}_frac"] = round(step_bytes(b, k) / (d / k) / 1e9 / HBM_PEAK_GBS, 4)
+            decode_point(f"decode_b{b}", b, args.steps if b == args.batch else points_steps, median(seconds[b]))
+        # further sizes, one measurement each: larger batches, a long context, longer prompts
+        for b in (128, 256):
+            print(f"[bench] decode at batch {b} ...", file=sys.stderr, flush=True)
+            decode_point(f"decode_b{b}", b, points_steps, decode_run(engine, sampler, b, args.context, points_steps, 4,
+                                                                      c.vocab_size, 900 + b))
+        print("[bench] decode at batch 8, context 32768 ...", file=sys.stderr, flush=True)
+        decode_point("decode_b8_ctx32768", 8, points_steps,
+                     decode_run(engine, sampler, 8, 32768, points_steps, 4, c.vocab_size, 33), context=32768)
+        for tokens in (8192, 32768):
+            print(f"[bench] prefill of {tokens} tokens ...", file=sys.stderr, flush=True)
+            t = median(prefill_run(engine, tokens, c.vocab_size, 2, 40 + tokens))
+            points[f"prefill_{tokens}"] = {"value": round(tokens / t, 1), "ms": round(t * 1e3, 3),
+                                           "frac": round(prefill_flops(tokens) / t / peak, 4)}
+        print("[bench] steps of a few dozen tokens ...", file=sys.stderr, flush=True)
         points.update(small_steps(engine, c.vocab_size, 5))
+        del engine
+        torch.cuda.empty_cache()
+        points.update(smaller_shapes(args.dtype, points_steps))
         line["points"] = points
     print(json.dumps(line), flush=True)
     return 0
+
+
+def smaller_shapes(dtype, steps):
+    """The two smaller checkpoints' shapes, compact: a decode step at batch 8 and context 4096 with its
+    share of the HBM peak, the continuous-batching workload (700M) and four 32,768-token requests (350M)."""
+    import torch
+    from imparo_amd.sampling import Sampler
+    out = {}
+    elem = 2 if dtype == "bfloat16" else 4
+    for name, cfg, seed in (("lfm2_700m", LFM2_700M, 3), ("lfm2_350m", LFM2_350M, 4)):
+        print(f"[bench] the {name} shape ...", file=sys.stderr, flush=True)
+        nums = model_numbers(cfg)
+        tokens = 32 * (3072 + 512 + 64) if name == "lfm2_700m" else 4 * (32768 + 128 + 64)
+        engine = build_engine(cfg, seed, dtype, max_tokens=tokens, max_requests=32)
+        d = decode_run(engine, Sampler(engine.device), 8, 4096, steps, 4, cfg["vocab_size"], 71)
+        to_read = ((nums["layer_params"] + nums["head_params"]) * elem
+                   + 8 * ((4096 - steps / 2) * nums["kv_bytes_per_token"] * elem / 2 + nums["conv_state_bytes"]))
+        out[f"decode_b8_{name}_ms_per_step"] = round(d / steps * 1e3, 4)
+        out[f"decode_b8_{name}_frac"] = round(to_read / (d / steps) / 1e9 / HBM_PEAK_GBS, 4)
+        if name == "lfm2_700m":
+            r = serving_workload(dtype, engine)
+            times = r["step_times"]
+            out["serving_lfm2_700m"] = {
+                "generated_tok_s": r["value"], "all_tok_s": r["all_tokens_per_s"], "seconds": r["seconds"],
+                "steps": r["steps"], "requests": 32,
+                "decode_only": {k: times["decode_only"][k] for k in ("p50_ms", "max_ms", "mean_rows", "hbm_frac_p50")},
+                "mixed": {k: times["mixed"][k] for k in ("p50_ms", "max_ms", "mean_prompt_tokens", "mfma_frac_p50")}}
+        else:
+            r = long_workload(dtype, 4, 32768, quiet=True, engine=engine)
+            out["long_lfm2_350m"] = {"requests": 4, "prompt_len": 32768, "prefill_tok_s": r["prefill_tok_s"],
+                                     "decode_tok_s": r["value"], "decode_ms_per_step": r["decode_ms_per_step"],
+                                     "decode_hbm_frac": r["decode_hbm_frac"]}
+        del engine
+        torch.cuda.empty_cache()
+    return out
 
 
 if __name__ == "__main__":

@@ -171,6 +171,28 @@ int imparo_in_proj_conv_decode(const void* x, const void* w, const float* in_bia
                                const float* conv_b, float* state, const int32_t* slot, void* out, int out_dtype,
                                int m, int e, int k, int taps, int n_slots, imparo_stream stream);
 
+// The same on activations that are the residual stream times a norm's weight, each row still to be
+// scaled: ssq_in [n_parts, 16] holds the partial sums of squares of the stream's rows and the launch
+// multiplies B, C and x of row r by rsqrt(sum_p ssq_in[p][r] / k + eps). ssq_in null: as above.
+int imparo_in_proj_conv_decode_normed(const void* x, const float* ssq_in, int n_parts, float eps, const void* w,
+                                      const float* in_bias, const float* conv_w, const float* conv_b, float* state,
+                                      const int32_t* slot, void* out, int out_dtype, int m, int e, int k, int taps,
+                                      int n_slots, imparo_stream stream);
+
+// Products for a step of at most 16 rows with a norm of the residual stream folded into them
+// (decode_rows.hip). x [m, k] and w [n, k] bfloat16, k a multiple of 8, bias float32 [n] or null.
+// With ssq_in [n_parts, 16] and eps, x is the stream times a norm's weight, each row still to be
+// scaled, and row r's result is multiplied by rsqrt(sum_p ssq_in[p][r] / k + eps) at the end, in float32.
+// epilogue 0: y [m, n] in out_dtype; 1: SwiGLU, y [m, n/2] (rows of w alternate gate, up);
+// 2: x_io [m, n] float32 += the result, in place, and ssq_out [imparo_rows_parts(n), 16] receives the
+// partial sums of squares of the new rows (entries of rows >= m are zero); with weighted_by [n] (the
+// weight of the norm that reads the stream next), weighted_out [m, n] bfloat16 receives the new rows
+// times it. A block sums the whole of K, in an order that depends on k alone.
+int imparo_rows_parts(int n);
+int imparo_rows_gemm(const void* x, const float* ssq_in, int n_parts, float eps, const void* w, const float* bias,
+                     void* y, int out_dtype, float* x_io, float* ssq_out, void* weighted_out, const float* weighted_by,
+                     int m, int n, int k, int epilogue, imparo_stream stream);
+
 // state' = the last taps-1 rows of (state ++ B*x) for every request; runs after
 // imparo_short_conv on the same stream.
 int imparo_short_conv_state(const float* bcx, float* state, const int32_t* seg_start, const int32_t* seg_len,
@@ -267,6 +289,11 @@ typedef struct {
 
 ImparoProgram* imparo_program_new(int engine_dtype, int page_size);
 void imparo_program_delete(ImparoProgram* p);
+// In a step of at most 16 single tokens a norm of the stream can be folded into the products around
+// it (decode_rows.hip): mode 0 never, 1 where imparo_rows_fold_pays says so (the default), 2 wherever
+// the operations allow. Folding changes results by rounding only.
+int imparo_program_set_fold(ImparoProgram* p, int mode);
+int imparo_rows_fold_pays(int m, int n, int k);
 // Operations, in run order. Each returns IMPARO_OK or IMPARO_BAD_ARGUMENT (sizes that do not fit).
 int imparo_program_embedding(ImparoProgram* p, const void* table, int table_dtype, int vocab, int width);
 // h = norm(stream + what the last mixer or feed-forward left pending), in out_dtype; the sum goes back to the stream

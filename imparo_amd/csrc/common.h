@@ -116,6 +116,7 @@ __device__ __forceinline__ void wave_lds_sync() {
 // One per file of kernels: loads that file's code onto the current device (imparo_load_code calls them all).
 int imparo_load_code_attention();
 int imparo_load_code_attention_mfma();
+int imparo_load_code_decode_rows();
 int imparo_load_code_elementwise();
 int imparo_load_code_gemm();
 int imparo_load_code_rope_cache();

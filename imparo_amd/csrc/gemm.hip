@@ -10,6 +10,7 @@
 
 #include <algorithm>
 #include "api.h"
+#include "rows.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -1061,12 +1062,16 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, const float* bias, T
 // oldest first exactly as the conv kernels sum them, the C gate, and the shift of the state
 // (a lane owns its channels' history, so nothing races). With HIST > 0 the history, the taps
 // and the biases are asked for before the walk along K, so they are there when it ends.
+// With ssq_in, X is the residual stream times a norm's weight, not yet scaled: the partial sums of
+// squares of its rows [n_parts, 16] give each row's scale, which multiplies B, C and x at the end (rows.h).
 template <typename TOut, int NW, int HIST>
 __global__ __launch_bounds__(NW * 64) void k_in_proj_conv_decode(
-    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, const float* __restrict__ in_bias,
+    const bf16_t* __restrict__ X, const float* __restrict__ ssq_in, int n_parts, float eps,
+    const bf16_t* __restrict__ W, const float* __restrict__ in_bias,
     const float* __restrict__ conv_w, const float* __restrict__ conv_b, float* __restrict__ state,
     const int32_t* __restrict__ slot, TOut* __restrict__ out, int M, int E, int K, int taps) {
     __shared__ float red[NW][2][64][4];
+    __shared__ float norm_part[NW * 4 * 16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, g = lane >> 4;
     const int c0 = blockIdx.x * 8;
@@ -1117,6 +1122,9 @@ __global__ __launch_bounds__(NW * 64) void k_in_proj_conv_decode(
     Frags cur, nxt;
     int k0 = wave * 128;
     if (k0 < K) load(k0, cur);
+    // the row's scale multiplies the sums at the end: its sums of squares are asked for now
+    RowsSsq early;
+    if (ssq_in) rows_ssq_ask(early, ssq_in, n_parts, 0);
     while (k0 < K) {
         const int k1 = k0 + NW * 128;
         if (k1 < K) load(k1, nxt);
@@ -1129,8 +1137,10 @@ __global__ __launch_bounds__(NW * 64) void k_in_proj_conv_decode(
         red[wave][0][lane][i] = acc0[i];
         red[wave][1][lane][i] = acc1[i];
     }
+    if (ssq_in) norm_part[(threadIdx.x >> 4) * 16 + (threadIdx.x & 15)] = rows_ssq_sum(early, ssq_in, n_parts);
     __syncthreads();
     if (!finisher) return;
+    const float scale = ssq_in ? rows_scale(norm_part, r16, K, eps) : 1.f;
     // D layout: lane holds column lane%16 (a token), tile rows 4*(lane/16) + i: B and C of channel
     // cb + i sit in this lane's entries, x of the same channel 8 tile rows further: lane + 32
     float b[4], c[4], x[4];
@@ -1144,6 +1154,11 @@ __global__ __launch_bounds__(NW * 64) void k_in_proj_conv_decode(
             b[i] += red[w][0][lane][i];
             x[i] += red[w][0][lane + 32][i];
             c[i] += red[w][1][lane][i];
+        }
+        if (ssq_in) {
+            b[i] = __fmul_rn(b[i], scale);
+            x[i] = __fmul_rn(x[i], scale);
+            c[i] = __fmul_rn(c[i], scale);
         }
     }
     float y[4];
@@ -1186,25 +1201,33 @@ __global__ __launch_bounds__(NW * 64) void k_in_proj_conv_decode(
 }
 
 template <typename TOut, int NW>
-static void launch_in_proj_conv(const bf16_t* x, const bf16_t* w, const float* in_bias, const float* conv_w,
-                                const float* conv_b, float* state, const int32_t* slot, TOut* out, int m, int e, int k,
-                                int taps, hipStream_t s) {
+static void launch_in_proj_conv(const bf16_t* x, const float* ssq_in, int n_parts, float eps, const bf16_t* w,
+                                const float* in_bias, const float* conv_w, const float* conv_b, float* state,
+                                const int32_t* slot, TOut* out, int m, int e, int k, int taps, hipStream_t s) {
     const unsigned blocks = (unsigned)(e / 8);
+#define CONV_GO(HIST)                                                                                              \
+    k_in_proj_conv_decode<TOut, NW, HIST><<<blocks, NW * 64, 0, s>>>(x, ssq_in, n_parts, eps, w, in_bias, conv_w, conv_b, \
+                                                                   state, slot, out, m, e, k, taps)
     switch (taps - 1) {
-        case 1: k_in_proj_conv_decode<TOut, NW, 1><<<blocks, NW * 64, 0, s>>>(x, w, in_bias, conv_w, conv_b, state, slot, out, m, e, k, taps); break;
-        case 2: k_in_proj_conv_decode<TOut, NW, 2><<<blocks, NW * 64, 0, s>>>(x, w, in_bias, conv_w, conv_b, state, slot, out, m, e, k, taps); break;
-        case 3: k_in_proj_conv_decode<TOut, NW, 3><<<blocks, NW * 64, 0, s>>>(x, w, in_bias, conv_w, conv_b, state, slot, out, m, e, k, taps); break;
-        default: k_in_proj_conv_decode<TOut, NW, 0><<<blocks, NW * 64, 0, s>>>(x, w, in_bias, conv_w, conv_b, state, slot, out, m, e, k, taps);
+        case 1: CONV_GO(1); break;
+        case 2: CONV_GO(2); break;
+        case 3: CONV_GO(3); break;
+        default: CONV_GO(0);
     }
+#undef CONV_GO
 }
 
 // x [m, k] bfloat16 (m <= 16 single tokens), w [3 e, k] bfloat16, conv_w [e, taps], state
 // [n_slots, taps-1, e], slot [m] (distinct): out [m, e] = the gated conv's output, state shifted.
-extern "C" int imparo_in_proj_conv_decode(const void* x, const void* w, const float* in_bias, const float* conv_w,
-                                          const float* conv_b, float* state, const int32_t* slot, void* out,
-                                          int out_dtype, int m, int e, int k, int taps, int n_slots,
-                                          imparo_stream stream) {
+// ssq_in [n_parts, 16] (or null) and eps: x is the residual stream times a norm's weight, each row
+// still to be scaled by rsqrt(sum of its partial sums of squares / k + eps), which the launch does.
+extern "C" int imparo_in_proj_conv_decode_normed(const void* x, const float* ssq_in, int n_parts, float eps,
+                                                 const void* w, const float* in_bias, const float* conv_w,
+                                                 const float* conv_b, float* state, const int32_t* slot, void* out,
+                                                 int out_dtype, int m, int e, int k, int taps, int n_slots,
+                                                 imparo_stream stream) {
     if (!x || !w || !conv_w || !state || !slot || !out) return IMPARO_BAD_ARGUMENT;
+    if (ssq_in && (n_parts <= 0 || !(eps > 0.f))) return IMPARO_BAD_ARGUMENT;
     if (m < 0 || m > 16 || e <= 0 || e % 8 != 0 || k <= 0 || k % 8 != 0 || taps < 2 || taps > 64 || n_slots <= 0)
         return IMPARO_BAD_ARGUMENT;
     if (((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return IMPARO_BAD_ARGUMENT;
@@ -1214,19 +1237,28 @@ extern "C" int imparo_in_proj_conv_decode(const void* x, const void* w, const fl
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w;
     // waves over K as the K-split kernel has them: chunks of 128, few per wave
+#define CONV_CALL(TOut, NW)                                                                                          \
+    launch_in_proj_conv<TOut, NW>(xb, ssq_in, n_parts, eps, wb, in_bias, conv_w, conv_b, state, slot, (TOut*)out, m, e, \
+                                  k, taps, s)
     if (out_dtype == IMPARO_F32) {
-        if (k <= 512)
-            launch_in_proj_conv<float, 4>(xb, wb, in_bias, conv_w, conv_b, state, slot, (float*)out, m, e, k, taps, s);
-        else
-            launch_in_proj_conv<float, 8>(xb, wb, in_bias, conv_w, conv_b, state, slot, (float*)out, m, e, k, taps, s);
+        if (k <= 512) CONV_CALL(float, 4);
+        else CONV_CALL(float, 8);
     } else {
-        if (k <= 512)
-            launch_in_proj_conv<bf16_t, 4>(xb, wb, in_bias, conv_w, conv_b, state, slot, (bf16_t*)out, m, e, k, taps, s);
-        else
-            launch_in_proj_conv<bf16_t, 8>(xb, wb, in_bias, conv_w, conv_b, state, slot, (bf16_t*)out, m, e, k, taps, s);
+        if (k <= 512) CONV_CALL(bf16_t, 4);
+        else CONV_CALL(bf16_t, 8);
     }
+#undef CONV_CALL
     return launch_status();
 }
+
+extern "C" int imparo_in_proj_conv_decode(const void* x, const void* w, const float* in_bias, const float* conv_w,
+                                          const float* conv_b, float* state, const int32_t* slot, void* out,
+                                          int out_dtype, int m, int e, int k, int taps, int n_slots,
+                                          imparo_stream stream) {
+    return imparo_in_proj_conv_decode_normed(x, nullptr, 0, 0.f, w, in_bias, conv_w, conv_b, state, slot, out, out_dtype,
+                                             m, e, k, taps, n_slots, stream);
+}
+
 
 // Which kernel takes a product of up to 64 rows: 0 for the K-split kernel, else the waves per
 // block of the shared-activation kernel. Measured with cold weights (they never stay in cache
@@ -1281,6 +1313,7 @@ extern "C" int imparo_gemm_adds(int m, int n, int k, int dtype) {
     return dtype == IMPARO_BF16 && m > 64 && dma_plan(m, n, k, 1).tn != 0;
 }
 
+
 // ------------------------------------------------------------------ bfloat16, some rows (17..64)
 // A block of ST_WAVES waves takes 16 weight rows per wave and up to 16*MT
 // activation rows, and walks its part of K in chunks of 128. The activation
@@ -1300,11 +1333,18 @@ struct StreamSet {
     uint4 x[XP];      // this thread's pieces of the activation chunk
 };
 
+// With ssq_in (at most 16 rows, K in one piece) the activations are the residual stream times a norm's
+// weight, and each row's result is multiplied at the end by the row's scale rsqrt(sum of squares / K +
+// eps) (rows.h): the partial sums are asked for at the start and needed only then.
 template <typename TOut, int MT, int ST_WAVES>
 __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, const float* __restrict__ bias,
-    TOut* __restrict__ Y, int M, int N, int K_all, int k_per, int epilogue) {
+    TOut* __restrict__ Y, int M, int N, int K_all, int k_per, int epilogue, const float* __restrict__ ssq_in,
+    int n_parts, float eps) {
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16 * ST_LD];
+    __shared__ float norm_part[ST_WAVES * 4 * 16];
+    RowsSsq early;
+    if (ssq_in) rows_ssq_ask(early, ssq_in, n_parts, 0);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, g = lane >> 4;
@@ -1416,6 +1456,12 @@ __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
         step(kt + 2, s2, s3, s1);
         step(kt + 3, s3, s0, s2);
     }
+    float row_scale = 1.f;
+    if (ssq_in) {        // (rows beyond 16 have no sums: the host sends such products elsewhere)
+        norm_part[(tid >> 4) * 16 + (tid & 15)] = rows_ssq_sum(early, ssq_in, n_parts);
+        __syncthreads();
+        row_scale = rows_scale(norm_part, min(r16, M - 1), K_all, eps);
+    }
     // D layout of the 16x16 tile: lane holds column lane%16 (an activation row), rows 4*(lane/16)+i (weight rows)
     const int nq = n0 + g * 4;
 #pragma unroll
@@ -1424,7 +1470,8 @@ __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
         if (m >= M) continue;
         float v[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = acc[mt][i] + ((bias && nq + i < N) ? bias[nq + i] : 0.f);
+        for (int i = 0; i < 4; ++i)
+            v[i] = (ssq_in ? __fmul_rn(acc[mt][i], row_scale) : acc[mt][i]) + ((bias && nq + i < N) ? bias[nq + i] : 0.f);
         if (epilogue == EPI_SWIGLU) {
 #pragma unroll
             for (int i = 0; i < 4; i += 2)
@@ -1439,15 +1486,31 @@ __global__ __launch_bounds__(ST_WAVES * 64) void k_gemm_bf16_stream(
 
 template <typename TOut, int MT>
 static void launch_stream(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k,
-                          int epilogue, int nw, int slices, hipStream_t s) {
+                          int epilogue, int nw, int slices, hipStream_t s, const float* ssq_in = nullptr,
+                          int n_parts = 0, float eps = 0.f) {
     const int k_per = ((k + slices - 1) / slices + ST_BK - 1) / ST_BK * ST_BK;
     dim3 grid((unsigned)((n + nw * 16 - 1) / (nw * 16)), (unsigned)((k + k_per - 1) / k_per));
     if (nw == 8)
-        k_gemm_bf16_stream<TOut, MT, 8><<<grid, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
+        k_gemm_bf16_stream<TOut, MT, 8><<<grid, 8 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue, ssq_in, n_parts, eps);
     else if (nw == 4)
-        k_gemm_bf16_stream<TOut, MT, 4><<<grid, 4 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
+        k_gemm_bf16_stream<TOut, MT, 4><<<grid, 4 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue, ssq_in, n_parts, eps);
     else
-        k_gemm_bf16_stream<TOut, MT, 2><<<grid, 2 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue);
+        k_gemm_bf16_stream<TOut, MT, 2><<<grid, 2 * 64, 0, s>>>(x, w, bias, y, m, n, k, k_per, epilogue, ssq_in, n_parts, eps);
+}
+
+// For the products of a step of at most 16 rows (decode_rows.hip): a weight of many rows is streamed
+// faster by this kernel, whose waves share the activations, than by one block per 16 weight rows.
+bool imparo_stream_rows_pays(int m, int n, int k) { return m <= 16 && stream_waves(m, n, k) == 4; }
+
+int imparo_stream_rows(const bf16_t* x, const bf16_t* w, const float* bias, void* y, int out_dtype, int m, int n, int k,
+                       int epilogue, const float* ssq_in, int n_parts, float eps, hipStream_t s) {
+    const int nw = stream_waves(m, n, k);
+    if (!nw || m > 16) return IMPARO_BAD_ARGUMENT;
+    if (out_dtype == IMPARO_F32)
+        launch_stream<float, 1>(x, w, bias, (float*)y, m, n, k, epilogue, nw, 1, s, ssq_in, n_parts, eps);
+    else
+        launch_stream<bf16_t, 1>(x, w, bias, (bf16_t*)y, m, n, k, epilogue, nw, 1, s, ssq_in, n_parts, eps);
+    return launch_status();
 }
 
 // With a K that the kernel with loads straight into LDS does not take: the 256x256 tile with register

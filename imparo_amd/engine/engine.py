@@ -127,12 +127,16 @@ class Engine:
     `native_step`: a step's kernels are issued by one call into the kernel
     library (a step program) where every part of the model can describe itself
     to it; False, or a model with a part that cannot, runs the parts one by one
-    from here. Both issue the same kernels with the same arguments."""
+    from here. Both issue the same kernels with the same arguments, except that
+    the native step may fold a norm into the products around it in steps of at
+    most 16 single tokens (`fold_norms`: None where the library's plan says it
+    pays, False never, True wherever possible), which changes results by
+    rounding only."""
 
     def __init__(self, model_dir: str, dtype: str = "bfloat16", max_tokens: Optional[int] = None, page_size: int = 64,
                  max_requests: int = 64, device: str = "cuda:0", use_graphs: bool = True,
                  kv_budget_bytes: Optional[int] = None, num_pages=None, max_step_tokens: int = 8192,
-                 native_step: bool = True):
+                 native_step: bool = True, fold_norms: Optional[bool] = None):
         if dtype not in DTYPES:
             raise ValueError(f"dtype must be one of {sorted(DTYPES)}, got {dtype!r}")
         if sum(x is not None for x in (max_tokens, kv_budget_bytes, num_pages)) > 1:
@@ -182,6 +186,7 @@ class Engine:
         self._args = StepArgs()
         self._prefill_tile = ops.prefill_tile()
         if self.program is not None:
+            self.program.set_fold(1 if fold_norms is None else (2 if fold_norms else 0))
             self._size_workspace(max_requests)
 
     @staticmethod
@@ -429,6 +434,15 @@ class Engine:
         n = packed.host_seg_len
         tile = self._prefill_tile
         a.portion_tiles = int(((n[n > 1] + (tile - 1)) // tile).sum()) if lay["n_multi"] else 0
+        return a
+
+    def _step_args_for_rows(self, rows: int, context: Optional[int] = None) -> StepArgs:
+        """The shape of a step of `rows` single tokens (no addresses): for asking the program what such a step uses."""
+        a = self._args
+        context = context or self.page_size
+        a.n_groups, a.table_width = len(self.cache.groups), -(-context // self.page_size)
+        a.n_tokens, a.n_rows, a.n_want, a.n_single, a.n_portion = rows, rows, rows, rows, 0
+        a.max_seg_len, a.max_context, a.portion_tiles = 1, context, 0
         return a
 
     def _grow_for(self, packed: "_Packed") -> None:

@@ -121,6 +121,18 @@ class Scheduler:
             self._lib.imparo_sched_delete(self._s)
             self._s = None
 
+    def warm(self, longest_context: int) -> int:
+        """Has the engine capture, now, every decode step this scheduler can come to run: 1 to
+        `max_running` single-token rows at every block-table width up to `longest_context` tokens.
+        A shape that is first met while serving costs several steps' time; this moves that cost
+        to the start. Returns the number of shapes captured (0 for an engine that captures none)."""
+        warm = getattr(self.engine, "warm", None)
+        if warm is None:
+            return 0
+        page = self.engine.page_size
+        contexts = sorted({min(longest_context, pages * page) for pages in range(1, -(-longest_context // page) + 1)})
+        return warm(range(1, self.max_running + 1), contexts)
+
     # ------------------------------------------------------------ intake
     def add(self, request_id: Hashable, prompt: Sequence[int], params: SamplingParams) -> Request:
         if len(prompt) == 0:

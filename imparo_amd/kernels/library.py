@@ -50,9 +50,15 @@ _SIGNATURES = {
     "imparo_fill_sites": [P, P, P, I, I, P],
     "imparo_attention_decode_static": [P, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
     "imparo_load_code": [],
+    "imparo_rows_parts": [I],
+    # x, ssq_in, n_parts, eps, w, bias, y, out_dtype, x_io, ssq_out, weighted_out, weighted_by, m, n, k, epilogue, stream
+    "imparo_rows_gemm": [P, P, I, F, P, P, P, I, P, P, P, P, I, I, I, I, P],
+    "imparo_in_proj_conv_decode_normed": [P, P, I, F, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
+    "imparo_rows_fold_pays": [I, I, I],
     # a model's step as one call (kernels/program.py holds the structures)
     "imparo_program_new": ([I, I], P),
     "imparo_program_delete": ([P], None),
+    "imparo_program_set_fold": [P, I],
     "imparo_program_embedding": [P, P, I, I, I],
     "imparo_program_norm": [P, P, F, I, I],
     "imparo_program_attention": [P, P],

@@ -431,6 +431,49 @@ def in_proj_conv_decode(x: torch.Tensor, in_weight: torch.Tensor, in_bias: Optio
     return out
 
 
+def rows_parts(n: int) -> int:
+    """Partial sums of squares that `rows_gemm(..., into=...)` leaves for a weight of n rows."""
+    return int(library().imparo_rows_parts(int(n)))
+
+
+def rows_gemm(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+              swiglu: bool = False, ssq_in: Optional[torch.Tensor] = None, eps: float = 0.0,
+              into: Optional[torch.Tensor] = None, ssq_out: Optional[torch.Tensor] = None,
+              weighted_out: Optional[torch.Tensor] = None, weighted_by: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Products of a step of at most 16 rows with a norm of the residual stream folded in. x [m, k] and
+    w [n, k] bfloat16. With `ssq_in` [parts, 16] and `eps`, x is the stream times a norm's weight and row
+    r's result is multiplied by rsqrt(sum_p ssq_in[p][r] / k + eps). Stored to `out` ([m, n], or [m, n/2]
+    with `swiglu`), or added to `into` [m, n] float32 in place; then `ssq_out` [rows_parts(n), 16] receives
+    the partial sums of squares of the new rows and, with `weighted_by` [n], `weighted_out` [m, n]
+    bfloat16 the new rows times it."""
+    m, k = x.shape
+    n, kw = w.shape
+    if kw != k or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or not 0 < m <= 16 or k % 8:
+        raise KernelArgumentError("rows_gemm: 1 to 16 bfloat16 rows, a bfloat16 weight over the same inner size, "
+                                  "a multiple of 8")
+    n_parts = 0
+    if ssq_in is not None:
+        n_parts = ssq_in.shape[0]
+        _dev(ssq_in, "sums of squares", torch.float32, (n_parts, 16))
+    if into is not None:
+        if out is not None or swiglu or ssq_out is None:
+            raise KernelArgumentError("rows_gemm: adding to the stream stores nothing else and leaves sums of squares")
+        _dev(into, "stream", torch.float32, (m, n))
+        _dev(ssq_out, "sums of squares out", torch.float32, (rows_parts(n), 16))
+        epilogue, y, code = 2, None, F32
+    else:
+        if out is None:
+            raise KernelArgumentError("rows_gemm: an output is needed")
+        _dev(out, "rows_gemm out", None, (m, n // 2 if swiglu else n))
+        epilogue, y, code = int(swiglu), out, _code(out, "rows_gemm out")
+    _check(library().imparo_rows_gemm(
+        _dev(x, "x"), _dev(ssq_in, "sums of squares"), n_parts, float(eps), _dev(w, "weight"),
+        _dev(bias, "bias", torch.float32, (n,)), _dev(y, "out"), code, _dev(into, "stream"), _dev(ssq_out, "ssq out"),
+        _dev(weighted_out, "weighted out", torch.bfloat16, (m, n)), _dev(weighted_by, "weighted by", torch.float32, (n,)),
+        m, n, k, epilogue, _stream()), "rows_gemm")
+    return into if into is not None else out
+
+
 def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     n, vocab = logits.shape
     _check(library().imparo_argmax_rows(_dev(logits, "logits", torch.float32), _dev(out, "picks", torch.int32, (n,)),

@@ -91,6 +91,11 @@ class Program:
             self._lib.imparo_program_delete(self._h)
             self._h = None
 
+    def set_fold(self, mode: int) -> None:
+        """Norms folded into the products around them in steps of at most 16 single tokens:
+        0 never, 1 where the library's plan says it pays, 2 wherever the operations allow."""
+        self._ok(self._lib.imparo_program_set_fold(self._h, int(mode)), "set_fold")
+
     def _ok(self, status: int, what: str) -> None:
         if status:
             raise KernelArgumentError(f"{what}: the step program refused the operation (sizes that do not fit)")

@@ -894,3 +894,58 @@ def test_sample_rows(vocab):
     ops().sample_rows(row.to(DEV), torch.full((4000,), 1.0, device=DEV), uu.to(DEV), out)
     freq = torch.bincount(out.cpu().long(), minlength=5).float() / 4000
     assert (freq - torch.softmax(row[0], 0)).abs().max() < 0.03
+
+
+# ---------------------------------------------------------------- products with a folded norm (at most 16 rows)
+from imparo_amd.kernels import ops as _rows_ops
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (5, 200, 136), (13, 1536, 1536), (16, 2048, 8192), (8, 96, 320),
+                                   (16, 4608, 1024), (3, 13824, 1536)])
+def test_rows_product_added_to_the_stream_leaves_sums_of_squares_and_weighted_rows(m, n, k):
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(m * 1000 + n + k)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).to(torch.bfloat16)
+    bias = torch.randn(n, generator=g) * 0.1
+    stream = torch.randn(m, n, generator=g)
+    by = 1.0 + 0.1 * torch.randn(n, generator=g)
+    want = stream + x.float() @ w.float().t() + bias
+    into = stream.clone().to(dev)
+    parts = _rows_ops.rows_parts(n)
+    ssq = torch.full((parts, 16), 7.0, device=dev)
+    weighted = torch.zeros(m, n, dtype=torch.bfloat16, device=dev)
+    _rows_ops.rows_gemm(x.to(dev), w.to(dev), bias=bias.to(dev), into=into, ssq_out=ssq, weighted_out=weighted,
+                  weighted_by=by.to(dev))
+    torch.testing.assert_close(into.cpu(), want, rtol=2e-5, atol=2e-5 * float(want.abs().max()))
+    got_ssq = ssq.cpu().sum(0)
+    torch.testing.assert_close(got_ssq[:m], (into.cpu() ** 2).sum(-1), rtol=1e-5, atol=0)
+    assert float(got_ssq[m:].abs().max()) == 0.0 if m < 16 else True      # rows the step does not have: zero
+    torch.testing.assert_close(weighted.cpu().float(), (into.cpu() * by).to(torch.bfloat16).float(), rtol=2 ** -7, atol=1e-6)
+
+
+@pytest.mark.parametrize("swiglu", [False, True])
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (5, 200, 136), (13, 4608, 1536), (16, 16384, 2048), (9, 96, 320),
+                                   (16, 9216, 1024), (2, 3072, 2048)])
+def test_rows_product_scales_its_rows_at_the_end(m, n, k, swiglu):
+    """The activations are the stream times a norm's weight, rounded to bfloat16; the sums of squares come
+    in parts; the product must equal (rows * rsqrt(mean square + eps)) . W^T in float32."""
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(m + n + k)
+    stream = torch.randn(m, k, generator=g) * 3.0
+    norm_w = 1.0 + 0.1 * torch.randn(k, generator=g)
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).to(torch.bfloat16)
+    eps = 1e-5
+    weighted = (stream * norm_w).to(torch.bfloat16)
+    n_parts = 37
+    cut = torch.linspace(0, k, n_parts + 1).long()
+    ssq = torch.zeros(n_parts, 16)
+    for p in range(n_parts):
+        ssq[p, :m] = (stream[:, cut[p]:cut[p + 1]] ** 2).sum(-1)
+    scale = torch.rsqrt((stream ** 2).mean(-1, keepdim=True) + eps)
+    want = (weighted.float() @ w.float().t()) * scale
+    if swiglu:
+        want = torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2]
+    for out_dtype in (torch.float32, torch.bfloat16):
+        out = torch.zeros(m, n // 2 if swiglu else n, dtype=out_dtype, device=dev)
+        _rows_ops.rows_gemm(weighted.to(dev), w.to(dev), out=out, swiglu=swiglu, ssq_in=ssq.to(dev), eps=eps)
+        tol = 2e-5 if out_dtype == torch.float32 else 2 ** -7
+        torch.testing.assert_close(out.cpu().float(), want, rtol=tol, atol=tol * float(want.abs().max()))

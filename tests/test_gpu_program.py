@@ -1,6 +1,7 @@
 """The native step program against the parts run one by one: both issue the same kernels with the
-same arguments, so every step's logits are the same bits, in both dtypes, launch by launch and through
-captured graphs. Then the engine's first steps when nothing has run before them, and `Engine.warm`."""
+same arguments (with the program's folding of norms switched off), so every step's logits are the same
+bits, in both dtypes, launch by launch and through captured graphs. Then the folded norms against the
+plain implementation, the engine's first steps when nothing has run before them, and `Engine.warm`."""
 import random
 
 import pytest
@@ -25,7 +26,7 @@ def test_one_native_call_and_parts_one_by_one_give_the_same_bits(model_dirs, nam
     steps = mixed_schedule(random.Random(7), lengths, sizes=(1, 1, 1, 1, 2, 3, 9, 16, 40))
     pool = peak_pages(steps, 16)
     engines = [make_engine(model_dirs[name], dtype, page_size=16, max_tokens=pool * 16, max_requests=4,
-                           use_graphs=graphs, native_step=native) for native in (True, False)]
+                           use_graphs=graphs, native_step=native, fold_norms=False) for native in (True, False)]
     assert engines[0].program is not None and engines[1].program is None
     for entries, ends in steps:
         outs = [eng.step([StepEntry(f"r{rid}", prompts[rid][lo:hi], list(range(hi - lo))) for rid, lo, hi in entries])
@@ -94,3 +95,33 @@ def test_warm_captures_shapes_before_they_are_met(model_dirs, plain_models):
         out = eng.step([StepEntry(i, [s[len(s) - 4 + j]], [0]) for i, s in enumerate(seqs)]).cpu()
         check_logits(out, torch.stack([r[len(s) - 4 + j] for r, s in zip(refs, seqs)]), "bfloat16", f"warmed step {j}")
     assert set(eng._graphs) == shapes, "the steps ran from graphs that warm() had captured"
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_norms_folded_into_the_products_around_them(model_dirs, plain_models, name):
+    """Steps of at most 16 single tokens with every norm between two products folded away: the
+    product before it adds to the stream and leaves sums of squares and weighted rows, the product
+    behind it scales at its end. Five requests decode ten tokens each after prompts of different
+    lengths; every row is held to the plain implementation, and the folded engine to the unfolded
+    one within the same bound."""
+    from imparo_amd.engine import StepEntry
+    from tiny_configs import CONFIGS
+    vocab = CONFIGS[name][0]["vocab_size"]
+    seqs = [prompt_tokens(vocab, n + 10, 60 + i) for i, n in enumerate((1, 7, 16, 33, 50))]
+    refs = [plain_models[name].logits(s) for s in seqs]
+    outs = {}
+    for fold in (True, False):
+        eng = make_engine(model_dirs[name], "bfloat16", page_size=16, max_tokens=512, max_requests=8, fold_norms=fold)
+        shape = eng._args
+        for i, s in enumerate(seqs):
+            eng.step([StepEntry(i, s[:-10], [])])
+        got = []
+        for j in range(10):
+            out = eng.step([StepEntry(i, [s[len(s) - 10 + j]], [0]) for i, s in enumerate(seqs)]).cpu()
+            got.append(out.clone())
+            check_logits(out, torch.stack([r[len(s) - 10 + j] for r, s in zip(refs, seqs)]), "bfloat16",
+                         f"{name}, norms folded: {fold}, step {j}")
+        outs[fold] = torch.stack(got)
+        used = eng.program.needs(eng._step_args_for_rows(5))
+        assert ("fold_ssq" in used) == fold, "the decode step of five rows folds its norms exactly when asked to"
+    assert not torch.equal(outs[True], outs[False])     # two ways of rounding
