@@ -1,2 +1,2 @@
-from .pages import (PagePool, CacheGroup, CacheManager, PagedSpec, PagedArray, PAGE, kv_spec, FixedSpec, StateSpec,
+from .pages import (PagePool, CacheGroup, CacheManager, PagedSpec, PagedArray, PAGE, kv_spec, FixedSpec, FixedArray, StateSpec,
                     OutOfPages, CacheError)

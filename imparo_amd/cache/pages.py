@@ -137,11 +137,42 @@ def kv_spec(kv_heads: int, head_dim: int, window: Optional[int] = None, v_transp
 
 
 @dataclass(frozen=True)
-class FixedSpec:
-    """State of a fixed size per request (a conv history, a recurrent matrix),
-    float32; a request that has seen nothing starts from `init` everywhere."""
+class FixedArray:
+    """One tensor of a fixed-size state: its shape per request, its dtype
+    ("float32", "bfloat16", "int32", or "engine" for the engine's own dtype)
+    and the value a request that has seen nothing starts from (anything but
+    float32 starts from zero). The device tensor is [n_slots, *shape]."""
+    name: str
     shape: Tuple[int, ...]
+    dtype: str = "float32"
     init: float = 0.0
+
+    def __post_init__(self):
+        if self.dtype not in ("float32", "bfloat16", "int32", "engine"):
+            raise ValueError(f"state array {self.name!r}: dtype {self.dtype!r} is none of float32, bfloat16, int32, engine")
+        if self.dtype != "float32" and self.init != 0.0:
+            raise ValueError(f"state array {self.name!r}: only a float32 array can start from a value other than zero")
+
+
+@dataclass(frozen=True)
+class FixedSpec:
+    """State of a fixed size per request (a conv history, a recurrent matrix).
+    `FixedSpec(shape, init)` is one float32 array, named "state"; a mixer that
+    keeps several tensors of different shapes or dtypes (a recurrent matrix
+    beside a short history, a 16-bit state) names them in `arrays` instead."""
+    shape: Optional[Tuple[int, ...]] = None
+    init: float = 0.0
+    arrays: Tuple[FixedArray, ...] = ()
+
+    def __post_init__(self):
+        if (self.shape is None) == (len(self.arrays) == 0):
+            raise ValueError("a fixed spec is either one float32 array (shape, init) or a tuple of named arrays")
+        names = [a.name for a in self.arrays]
+        if len(set(names)) != len(names):
+            raise ValueError(f"a fixed spec names an array twice: {names}")
+
+    def all_arrays(self) -> Tuple[FixedArray, ...]:
+        return self.arrays or (FixedArray("state", tuple(self.shape), "float32", self.init),)
 
 
 StateSpec = Union[PagedSpec, FixedSpec, None]

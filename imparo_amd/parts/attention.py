@@ -69,6 +69,10 @@ class Attention:
         self.out = Linear(place_matrix(tensors[n["o"] + ".weight"], engine_dtype, device))
         norm = spec.get("qk_norm")
         if norm is not None:
+            # the kernels that norm a head know one norm: RMS with a weight per dimension, no offset
+            if getattr(norm, "kind", "rms_norm") != "rms_norm":
+                raise ValueError(f"this attention mixer norms q and k per head with an RMS norm; the plan names "
+                                 f"{norm.kind!r} (another norm on the heads is another mixer, with kernels of its own)")
             self.norm_eps = float(norm["eps"])
             self.q_norm = place_vector(tensors[n["q_norm"] + ".weight"], device)
             self.k_norm = place_vector(tensors[n["k_norm"] + ".weight"], device)

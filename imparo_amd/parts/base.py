@@ -122,7 +122,12 @@ class StepContext:
         return arrays["k"], arrays["v"], table
 
     def fixed_state(self, site: int) -> torch.Tensor:
+        """The site's fixed-size state [slots, *shape]: its one array, or the one named "state"."""
         return self.storage.fixed[site]
+
+    def fixed_arrays(self, site: int) -> Dict[str, torch.Tensor]:
+        """Every array of the site's fixed-size state by name, each [slots, *shape] in its own dtype."""
+        return self.storage.fixed_arrays[site]
 
 
 def emits(part, emit: str = "emit", forward: str = "forward") -> bool:

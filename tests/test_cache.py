@@ -329,3 +329,21 @@ def test_pool_sizes_from_a_budget_in_bytes():
         Engine.pool_sizes(specs, 64, torch.bfloat16, None, per_page - 1, None)
     with pytest.raises(ValueError, match="num_pages"):
         Engine.pool_sizes(specs, 64, torch.bfloat16, None, None, [7])
+
+
+def test_fixed_specs_name_one_array_or_several():
+    from imparo_amd.cache import FixedArray, FixedSpec
+    one = FixedSpec((2, 64), 0.5)
+    assert one.all_arrays() == (FixedArray("state", (2, 64), "float32", 0.5),)
+    two = FixedSpec(arrays=(FixedArray("r", (4, 4)), FixedArray("s", (8,), "bfloat16")))
+    assert [a.name for a in two.all_arrays()] == ["r", "s"] and two != one
+    with pytest.raises(ValueError, match="either one float32 array"):
+        FixedSpec()
+    with pytest.raises(ValueError, match="either one float32 array"):
+        FixedSpec((3,), arrays=(FixedArray("r", (3,)),))
+    with pytest.raises(ValueError, match="twice"):
+        FixedSpec(arrays=(FixedArray("r", (3,)), FixedArray("r", (4,))))
+    with pytest.raises(ValueError, match="other than zero"):
+        FixedArray("s", (8,), "bfloat16", init=1.0)
+    with pytest.raises(ValueError, match="dtype"):
+        FixedArray("s", (8,), "float16")

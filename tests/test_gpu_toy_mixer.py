@@ -59,6 +59,28 @@ class LeakyMean:
         return self.u(ctx, out.to(self.u.in_dtype), torch.float32, "mixer_out")
 
 
+class LeakyMeanThatCounts(LeakyMean):
+    """The same mixer keeping two tensors of fixed size per request, of different shapes and dtypes:
+    its running mean in float32 and, in bfloat16, how many tokens the request has fed so far."""
+
+    def cache_spec(self, page_size):
+        from imparo_amd.cache import FixedArray, FixedSpec
+        return FixedSpec(arrays=(FixedArray("mean", (self.width,)), FixedArray("fed", (2,), "bfloat16")))
+
+    def forward(self, ctx, site, owns_cache, h):
+        arrays = ctx.fixed_arrays(site)
+        z = self.w(ctx, h, torch.float32, "toy_z")
+        out = torch.empty_like(z)
+        for start, n, slot in zip(ctx.seg_start.tolist(), ctx.seg_len.tolist(), ctx.slot.tolist()):
+            s = arrays["mean"][slot].clone()
+            for t in range(start, start + n):
+                s = self.decay * s + (1.0 - self.decay) * z[t]
+                out[t] = s
+            arrays["mean"][slot] = s
+            arrays["fed"][slot, 0] += n
+        return self.u(ctx, out.to(self.u.in_dtype), torch.float32, "mixer_out")
+
+
 def plain_leaky(h, w, u, decay):
     z = h @ w.t()
     s = torch.zeros(h.shape[1])
@@ -160,3 +182,45 @@ def test_toy_model_generates_through_the_scheduler(toy):
     for tok in got:
         assert int(torch.argmax(plain_toy_logits(d, cfg, seq)[-1])) == tok
         seq.append(tok)
+
+
+def test_a_mixer_with_two_states_of_different_shape_and_dtype(toy, tmp_path):
+    """The same model with the toy mixer keeping a float32 mean and a bfloat16 counter per request:
+    both live in the request's slot, both start from zero when a slot is used again."""
+    import dataclasses, shutil
+    from imparo_amd import register_architecture, register_part, PartSpec
+    from imparo_amd.config import Lfm2Config, lfm2
+    from imparo_amd.engine import Engine, StepEntry
+    d, cfg = toy
+    register_part("mixer", "test_leaky_mean_counting", LeakyMeanThatCounts)
+
+    def read(c):
+        out = Lfm2Config.from_dict({k: v for k, v in c.items() if k not in ("toy_layers", "toy_decay")})
+        out.toy_layers, out.toy_decay = c["toy_layers"], c["toy_decay"]
+        return out
+
+    def build(c):
+        plan = lfm2.build_plan(c)
+        layers = list(plan.layers)
+        for i in c.toy_layers:
+            part = PartSpec("test_leaky_mean_counting", f"model.layers.{i}.toy", dict(width=c.hidden_size, decay=c.toy_decay))
+            layers[i] = layers[i].with_part("mixer", part)
+        return dataclasses.replace(plan, architecture="TestLeakyCountingForCausalLM", layers=layers)
+    register_architecture("TestLeakyCountingForCausalLM", read, build)
+    d2 = str(tmp_path / "counting")
+    shutil.copytree(d, d2)
+    with open(os.path.join(d2, "config.json"), "w") as f:
+        json.dump(dict(cfg, architectures=["TestLeakyCountingForCausalLM"]), f)
+    eng = Engine(d2, dtype="float32", max_tokens=512, page_size=8, max_requests=2)
+    assert eng.program is None                    # a part from outside: the parts run one by one
+    a = prompt_tokens(256, 21, 4)
+    ref = plain_toy_logits(d, cfg, a)
+    got = torch.cat([eng.step([StepEntry("a", a[:9], list(range(9)))]).cpu(),
+                     eng.step([StepEntry("a", a[9:], list(range(12)))]).cpu()])
+    check_logits(got, ref, "float32", "two states")
+    fed = eng.storage.fixed_arrays[0]["fed"]
+    assert fed.dtype == torch.bfloat16 and float(fed[eng.cache.slot_of["a"], 0]) == 21.0
+    eng.release("a")
+    again = eng.step([StepEntry("b", a, list(range(21)))]).cpu()          # the slot is used again: both start from zero
+    check_logits(again, ref, "float32", "two states, slot used again")
+    assert float(fed[eng.cache.slot_of["b"], 0]) == 21.0
