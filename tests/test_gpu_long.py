@@ -80,14 +80,21 @@ def test_a_borrowed_cache_at_head_size_64(long_model, tmp_path, dtype):
     check_logits(got, ref, dtype, f"borrowed cache {dtype}")
 
 
-def test_long_context_bfloat16_against_float32(long_model):
+def test_long_context_against_the_plain_implementation(long_model):
     """16,500 tokens in portions of 2,048 (tiles of 64 queries over hundreds of
     key tiles, a window of 700 that gives pages back), two short portions (their
     keys walked in parts), then single tokens over more than 64 splits of 256
-    keys, through captured steps."""
+    keys, through captured steps. Both dtypes are held to the plain implementation
+    at every row that was asked for, under the bound for this many keys, and the
+    bfloat16 run to the float32 run."""
+    from plain_lfm2 import PlainLfm2
     from imparo_amd.engine import StepEntry
+    from tolerances import bound
     N = 16500
     toks = prompt_tokens(512, N + 137 + 40, 99)
+    asked = [r for lo in range(0, N, 2048) for r in range(min(N, lo + 2048) - 8, min(N, lo + 2048))]
+    asked += list(range(N, N + 137 + 40))
+    ref = PlainLfm2(long_model).logits(toks)[asked]
     runs = {}
     for dtype in ("float32", "bfloat16"):
         eng = make_engine(long_model, dtype, page_size=64, max_tokens=N + 256, max_requests=2)
@@ -102,6 +109,7 @@ def test_long_context_bfloat16_against_float32(long_model):
         held = eng.cache.held_pages("l")
         assert held[0] == (N + 177 + 63) // 64 and held[1] <= 700 // 64 + 3    # the window's group holds a dozen pages
         runs[dtype] = torch.cat(out)
+        check_logits(runs[dtype], ref, dtype, f"16,677 tokens, {dtype}", rel=bound(dtype, len(LONG["layer_types"]), N + 177))
     check_logits(runs["bfloat16"], runs["float32"], "bfloat16", "long context")
 
 
