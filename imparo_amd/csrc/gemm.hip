@@ -757,8 +757,8 @@ __global__ __launch_bounds__(64 * NWM * NWN) void k_gemm_bf16_dma(const bf16_t* 
     // stores. A staged row is 136 floats: the two rows a store instruction touches, 4 apart,
     // fall on disjoint banks. Each wave has a region of its own, so no barrier between passes.
     __syncthreads();                                   // every wave is done with the operands in LDS
-    constexpr int EP_LD = (NWN == 2 && NWM == 2) ? 136 : WN + 8;
-    constexpr int LPR = ((NWN == 2 && NWM == 2) || 64 % (WN / 4)) ? 32 : WN / 4;   // lanes to a staged row
+    constexpr int EP_LD = (NWN == 2 && NWM == 2 && TN > 1) ? 136 : WN + 8;
+    constexpr int LPR = ((NWN == 2 && NWM == 2 && TN > 1) || 64 % (WN / 4)) ? 32 : WN / 4;   // lanes to a staged row
     static_assert((4 * EP_LD) % 64 == 32 && NW / 2 * 32 * EP_LD * 4 <= (BM + BN) * DM_BK * 2, "staging layout");
     float* staged = reinterpret_cast<float*>(wave >= NW / 2 ? stage1 : stage0) + (wave % (NW / 2)) * (32 * EP_LD);
     const int out_col = (lane % LPR) * 4;              // of the wave's columns: lanes past them (narrow tiles) sit out
@@ -833,8 +833,8 @@ static bool dma_tile_takes(int m, int n, int k) {
     return k % (2 * DM_BK) == 0 && (long long)m * k < (1LL << 31) && (long long)n * k < (1LL << 31);
 }
 
-// Which tile (bm = 256 or 128 activation rows, tn = 4, 3, 2 for 256, 192, 128 weight rows; 192 with
-// bm 256 only), on how many stages, and how many slices of K suit a product of many rows; tn = 0:
+// Which tile (bm = 256 or 128 activation rows, tn = 4, 3, 2, 1 for 256, 192, 128, 64 weight rows; 192 with
+// bm 256 only, 64 with bm 128 only), on how many stages, and how many slices of K suit a product of many rows; tn = 0:
 // none (a K the kernel does not take). A model of the time, fitted to this machine over 128 to 8,192
 // rows and seven weight shapes, every tile and 1 to 8 slices measured (what it picks is within 1 % of
 // the fastest on average and within 7 % on every shape whose consumer can add slices):
@@ -842,6 +842,10 @@ static bool dma_tile_takes(int m, int n, int k) {
 //     second with all 256 (clocks, L2), in between in proportion:
 //         128x128 0.46 .. 0.78 us    128x256 0.70 .. 1.08    256x128 0.66 .. 1.08
 //         256x192 0.89 .. 1.30       256x256 1.03 .. 1.58
+//   - a tile of 128 rows by 64 weight rows on four waves and four stages takes 0.35 .. 0.50 us a step: with at
+//     most 128 rows (one tile down the rows) it makes twice the blocks of the 128x128 tile out of a weight
+//     that is streamed once, and a block's share of the weights is what bounds such a product (measured at
+//     96 and 128 rows: 21 us against 27 on gate/up, 8 to 13 against 11 to 18 on the sliced products);
 //   - two blocks fit a CU where their stages take 80 KB or less each (the 128x128 tile on two
 //     stages); a step of both then takes 1.09 us, and with two on some CUs only, in between;
 //   - the 128x128 tile can instead keep four stages (one block a CU, three steps' loads in flight):
@@ -866,19 +870,22 @@ static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
         if (k % (128 * slices) != 0 || (slices > 1 && k / slices < 512)) continue;
         for (int bm = 256; bm >= 128; bm /= 2) {
             const int tiles_m = (m + bm - 1) / bm;
-            for (int tn = 4; tn >= 2; --tn) {
+            for (int tn = 4; tn >= 1; --tn) {
                 if (tn == 3 && bm != 256) continue;
+                if (tn == 1 && bm != 128) continue;
                 const int bn = 64 * tn;
                 for (int stages = 2; stages <= 4; stages += 2) {
-                    // four stages: the 128x128 tile, K-steps in fours
-                    if (stages == 4 && (bm != 128 || tn != 2 || (k / slices) % (4 * DM_BK) != 0)) continue;
+                    // four stages: the 128x128 tile and the 128x64 one (which runs on four only), K-steps in fours
+                    if (stages == 4 && (bm != 128 || tn > 2 || (k / slices) % (4 * DM_BK) != 0)) continue;
+                    if (stages == 2 && tn == 1) continue;
                     const long long blocks = (long long)tiles_m * ((n + bn - 1) / bn) * slices;
                     const int at_once = 256 * ((bm + bn) * DM_BK * 2 * stages <= 80 * 1024 ? 2 : 1);
                     const long long rounds = (blocks + at_once - 1) / at_once;
                     const long long per_round = (blocks + rounds - 1) / rounds;
                     const double cus = (double)std::min<long long>(256, per_round);
                     double few, all;
-                    if (bm == 128 && tn == 2) few = stages == 4 ? 0.33 : 0.46, all = stages == 4 ? 0.53 : 0.78;
+                    if (bm == 128 && tn == 1) few = 0.35, all = 0.50;
+                    else if (bm == 128 && tn == 2) few = stages == 4 ? 0.33 : 0.46, all = stages == 4 ? 0.53 : 0.78;
                     else if (bm == 128) few = 0.70, all = 1.08;
                     else if (tn == 2) few = 0.66, all = 1.08;
                     else if (tn == 3) few = 0.89, all = 1.30;
@@ -886,6 +893,10 @@ static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
                     double step = per_round > 256 ? all + (1.09 - all) * (per_round - 256) / 256.0    // some CUs, or all, with two
                                                   : few + (all - few) * cus / 256.0;
                     if (tiles_m <= 2) step = std::max(step, stages == 4 ? 0.36 : 0.55);
+                    // one tile down the rows: a block streams its weight rows alone, 128 bytes of each a
+                    // step, and one CU draws about 28 GB/s of cold weights (0.60 us a step measured on the
+                    // 128x128 tile at 128 rows, where the figures above would have it at 0.43)
+                    if (tiles_m == 1) step = std::max(step, bn * 128.0 / 28e3);
                     const double ends = 4.3 + 0.116 * (bm * bn / 1024.0);
                     const double from_memory = ((double)m + n) * k * 2.0 / 5.5e6;
                     const double cost = std::max(rounds * (k / slices / DM_BK * step + ends), from_memory + ends) +
@@ -902,7 +913,7 @@ static DmaPlan dma_plan(int m, int n, int k, int fixed_slices) {
 }
 
 // `slices` must leave every slice a multiple of 128 of K (dma_tile_takes(m, n, k / slices) and k % slices == 0).
-// bm: 256 or 128 activation rows to a tile; tn: 4, 3 (bm 256 only) or 2 for 256, 192 or 128 weight rows.
+// bm: 256 or 128 activation rows to a tile; tn: 4, 3 (bm 256 only), 2 or 1 (bm 128 only) for 256, 192, 128 or 64 weight rows.
 template <typename TOut>
 static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TOut* y, int m, int n, int k, int epilogue,
                       int bm, int tn, int slices, hipStream_t s, int stages = 2) {
@@ -912,7 +923,11 @@ static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TOut*
 #define DMA_GO(TMI, TN, NWN)                                                                                         \
     k_gemm_bf16_dma<TOut, TMI, TN, NWN><<<grid, 128 * NWN, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m,     \
                                                                    tiles_n, epilogue)
-    if (bm == 128 && tn == 4)
+    if (bm == 128 && tn == 1 && stages == 4)   // 64 wide: four waves of 64 rows by 32
+        k_gemm_bf16_dma<TOut, 2, 1, 2, 2, 4><<<grid, 256, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
+    else if (bm == 128 && tn == 1)
+        k_gemm_bf16_dma<TOut, 2, 1, 2, 2, 2><<<grid, 256, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
+    else if (bm == 128 && tn == 4)
         DMA_GO(2, 2, 4);
     else if (bm == 128 && stages == 4)
         k_gemm_bf16_dma<TOut, 2, 1, 4, 2, 4><<<grid, 512, 0, s>>>(x, w, bias, y, m, n, k, k / slices, tiles_m, tiles_n, epilogue);
@@ -1564,6 +1579,10 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
         // 358, 352: 128 activation rows to a tile, 256 and 128 wide
         if ((force == 358 || force == 352) && k % slices == 0 && dma_tile_takes(m, n, k / slices) && dma_tile_takes(m, n, k))
             return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, 128, force == 358 ? 4 : 2, slices, s);
+        // 351, 451: 128 activation rows by 64 weight rows, on two stages and on four
+        if ((force == 351 || force == 451) && k % slices == 0 && dma_tile_takes(m, n, k / slices) && dma_tile_takes(m, n, k) &&
+            (force == 351 || (k / slices) % (4 * DM_BK) == 0))
+            return launch_dma<TOut>(x, w, bias, y, m, n, k, epilogue, 128, 1, slices, s, force == 451 ? 4 : 2);
         const int tiles_m = (m + BG_BM - 1) / BG_BM, tiles_n = (n + BG_BN - 1) / BG_BN;
         const long long total = (long long)tiles_m * tiles_n;
         if (total > 0x7fffff00LL) return IMPARO_BAD_ARGUMENT;
@@ -1580,7 +1599,8 @@ static int launch_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TOut
 // that each kernel can be met at any shape: 1 the K-split kernel, 2, 4 or 8 the shared-activation
 // kernel with that many waves, 256 the 256x256 tile with register staging, 258 / 263 / 262 the tile
 // with loads straight into LDS at 256 rows by 256 / 192 / 128, 358 / 352 the same at 128 rows by
-// 256 / 128, 452 the 128 by 128 tile on four stages; with a variant, any number of K slices is taken.
+// 256 / 128, 452 the 128 by 128 tile on four stages, 351 / 451 the 128 by 64 tile on two / four stages;
+// with a variant, any number of K slices is taken.
 static int gemm_variant(const void* x, const void* w, const float* bias, void* y, int dtype, int out_dtype,
                         int m, int n, int k, int epilogue, int slices, int variant, imparo_stream stream) {
     if (!x || !w || !y || m < 0 || n <= 0 || k <= 0) return IMPARO_BAD_ARGUMENT;

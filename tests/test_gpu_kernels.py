@@ -157,10 +157,12 @@ def test_gemm_with_many_weight_rows(m, k):
                                         (1500, 3900, 640, 0), (2600, 3904, 200, 0), (70, 100, 128, 0),
                                         (700, 1000, 384, 258), (700, 1000, 384, 262), (700, 1000, 384, 263),
                                         (700, 1000, 384, 358), (700, 1000, 384, 352),
-                                        (700, 1000, 256, 452), (700, 1000, 1280, 452), (130, 250, 2048, 452)])
+                                        (700, 1000, 256, 452), (700, 1000, 1280, 452), (130, 250, 2048, 452),
+                                        (700, 1000, 384, 351), (100, 250, 2048, 451), (128, 1000, 512, 451),
+                                        (128, 16384, 2048, 0), (96, 2048, 8192, 0), (65, 3072, 2048, 0)])
 def test_gemm_with_large_tiles(m, n, k, tile):
     """Many rows: K a multiple of 128 goes to the kernel that loads straight into LDS, with a tile
-    of 256 or 128 rows by 256, 192 or 128 weight rows, whichever its plan finds fastest (`tile`
+    of 256 or 128 rows by 256, 192, 128 or 64 weight rows, whichever its plan finds fastest (`tile`
     other than 0 names one, an argument of the entry point for tests and measurements, so that each is met);
     another K to the tile kernels with register staging. Edges in both directions, an odd number
     of column pairs, a bias, both epilogues and output types."""
