@@ -100,7 +100,7 @@ class _DecodeGraph:
 
 REGION_CAP = 256 << 20   # bytes of one scratch region that are reserved up front; beyond that it grows when needed
 TABLE_BUCKET = 8     # captured steps round their block-table width up to a multiple of this many pages, or more
-MAX_GRAPHS = 256     # captured batch shapes kept; beyond that the one unused for longest goes
+MAX_GRAPHS = 256     # captured batch shapes kept (more if `warm` is asked for more); beyond that the one unused for longest goes
 
 
 def table_bucket(pages: int) -> int:
@@ -175,6 +175,7 @@ class Engine:
         # HIP graph: the launches of a step cost more host time than the step's kernels take
         self.use_graphs = use_graphs
         self._graphs: Dict[Tuple[int, int], _DecodeGraph] = {}
+        self.max_graphs = MAX_GRAPHS
         self._graph_pool = None
         self._capture_stream = None
         self.vocab_size = self.plan.vocab_size
@@ -321,7 +322,7 @@ class Engine:
         key = (rows, width)
         g = self._graphs.get(key)
         if g is None:
-            if len(self._graphs) >= MAX_GRAPHS:      # each holds an executable graph and its index arrays
+            if len(self._graphs) >= self.max_graphs:      # each holds an executable graph and its index arrays
                 del self._graphs[min(self._graphs, key=lambda k: self._graphs[k].last_used)]
             g = self._graphs[key] = _DecodeGraph()
         g.last_used = self.steps_run
@@ -360,10 +361,14 @@ class Engine:
         if not (self.use_graphs and self.model.graph_safe):
             return made
         G = len(self.cache.groups)
-        for n in sorted(set(int(r) for r in rows)):
-            for context in sorted(set(int(c) for c in contexts)):
-                if n < 1 or context < 1:
-                    raise ValueError("warm: rows and contexts are positive numbers")
+        rows, contexts = sorted(set(int(r) for r in rows)), sorted(set(int(c) for c in contexts))
+        if any(n < 1 for n in rows) or any(c < 1 for c in contexts):
+            raise ValueError("warm: rows and contexts are positive numbers")
+        wanted = {(n, table_bucket(-(-c // self.page_size))) for n in rows for c in contexts}
+        # what the caller asks for is kept: room for all of it beside what is there
+        self.max_graphs = max(self.max_graphs, len(set(self._graphs) | wanted))
+        for n in rows:
+            for context in contexts:
                 width = table_bucket(-(-context // self.page_size))
                 g = self._graph_for(n, width)
                 if g.graph is not None:

@@ -95,6 +95,9 @@ def test_warm_captures_shapes_before_they_are_met(model_dirs, plain_models):
         out = eng.step([StepEntry(i, [s[len(s) - 4 + j]], [0]) for i, s in enumerate(seqs)]).cpu()
         check_logits(out, torch.stack([r[len(s) - 4 + j] for r, s in zip(refs, seqs)]), "bfloat16", f"warmed step {j}")
     assert set(eng._graphs) == shapes, "the steps ran from graphs that warm() had captured"
+    # more shapes than the engine keeps by default: all of what was asked for stays
+    eng.max_graphs = 4
+    assert eng.warm(rows=[1, 2, 3, 4], contexts=[100, 300, 900]) == 6 and len(eng._graphs) == 12
 
 
 @pytest.mark.parametrize("name", ["A", "B", "C"])
