@@ -2,10 +2,9 @@
 option; C adds a sliding window on some attention layers (a second cache
 group) and float32-stored tensors.
 
-A and B are the two tiny configurations of the build's baseline in every size
-and option but one: `max_position_embeddings` is 1024 and 2048 here where the
-baseline says 128 and 256, because the tests run sequences of 150 to 330
-tokens through them (portions over several pages, long decoding, mixed
+`max_position_embeddings` of A and B is 1024 and 2048, eight times what models
+of this size would state (128 and 256), because the tests run sequences of 150
+to 330 tokens through them (portions over several pages, long decoding, mixed
 schedules that use pages again) and the engine refuses a request that would
 pass the model's positions. Nothing in the computation reads that number."""
 
