@@ -105,7 +105,7 @@ int imparo_attention_decode(const void* q, const void* k_cache, const void* v_ca
 // Head sizes 64 and 128 (imparo_attention_decode_qkv_takes); a layer that reads another layer's cache
 // finds the row's key there already and takes the two-launch form.
 int imparo_attention_decode_qkv_takes(int head_dim, int n_freq);
-int imparo_attention_decode_qkv_pays(int n_rows);       // few rows: the one launch is the faster way
+int imparo_attention_decode_qkv_pays(int n_rows, int n_splits);   // few rows over not too many splits: the one launch is the faster way
 int imparo_attention_decode_qkv(const float* qkv, const float* q_weight, const float* k_weight, float eps,
                                 const float* inv_freq, int n_freq, int interleaved, void* k_cache, void* v_cache,
                                 int write_kv, void* out, float* part_o, float* part_ml, const int32_t* rows,

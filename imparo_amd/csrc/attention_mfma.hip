@@ -1275,8 +1275,12 @@ extern "C" int imparo_attention_decode_qkv_takes(int head_dim, int n_freq) {
 }
 // ... and for how many rows it is the faster way: every block of a row's splits makes the row's queries
 // again, which a launch of its own does once (measured at 4,096 keys: 18.9 against 16.7 + 4.6 us for 8
-// rows, 6 us a layer slower for 64).
-extern "C" int imparo_attention_decode_qkv_pays(int n_rows) { return n_rows <= 16; }
+// rows, 6 us a layer slower for 64). With many splits a row the repeated work adds up: whole decode steps
+// of 1 to 16 rows at 4,096 to 32,768 keys are 1 to 3 % faster with the one launch up to 16 rows x 64 splits
+// and 8 x 128, and 1.3 % slower at 16 x 128.
+extern "C" int imparo_attention_decode_qkv_pays(int n_rows, int n_splits) {
+    return n_rows <= 16 && (long long)n_rows * n_splits <= 1024;
+}
 
 extern "C" int imparo_attention_decode_qkv(const float* qkv, const float* q_weight, const float* k_weight, float eps,
                                            const float* inv_freq, int n_freq, int interleaved, void* k_cache,

@@ -11,6 +11,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <algorithm>
 #include <string>
 #include <vector>
 
@@ -280,7 +281,8 @@ struct Walk {
         const Out qkv = consume(d.qkv, IMPARO_F32, p->r_mixer_in, false);
         const int64_t o_bytes = (int64_t)T * d.heads * d.head_dim * element_size(dt);
         if (dt != d.out.dtype) return fail(IMPARO_BAD_ARGUMENT, "an output projection whose weight dtype differs from the attention output's");
-        if (d.v_transposed && d.owns_cache && a->n_single == T && a->n_portion == 0 && imparo_attention_decode_qkv_pays(T) &&
+        const int decode_splits = std::max(1, (a->max_context + imparo_attention_decode_split() - 1) / imparo_attention_decode_split());
+        if (d.v_transposed && d.owns_cache && a->n_single == T && a->n_portion == 0 && imparo_attention_decode_qkv_pays(T, decode_splits) &&
             imparo_attention_decode_qkv_takes(d.head_dim, d.n_freq)) {
             // every row brings one token: head norm, rotation and the write of the new key and value ride in the attention launch
             void* o = get(p->r_mixer_mid, o_bytes);

@@ -37,7 +37,7 @@ _SIGNATURES = {
     # seg_start, positions, table, stride, page, heads, kv_heads, head_dim, n_pages, scale, window, n_splits, stream
     "imparo_attention_decode_qkv": [P, P, P, F, P, I, I, P, P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
     "imparo_attention_decode_qkv_takes": [I, I],
-    "imparo_attention_decode_qkv_pays": [I],
+    "imparo_attention_decode_qkv_pays": [I, I],
     "imparo_attention_prefill": [P, P, P, P, P, P, I, P, I, I, P, P, P, P, I, I, I, I, I, I, F, I, P],
     "imparo_attention_prefill_splits": [I, I, I, I, I],
     "imparo_attention_decode_split": [],

@@ -293,9 +293,10 @@ def attention_decode_qkv_takes(head_dim: int, n_freq: int) -> bool:
     return bool(library().imparo_attention_decode_qkv_takes(int(head_dim), int(n_freq)))
 
 
-def attention_decode_qkv_pays(n_rows: int) -> bool:
-    """Whether the one launch is the faster way for a step of this many rows."""
-    return bool(library().imparo_attention_decode_qkv_pays(int(n_rows)))
+def attention_decode_qkv_pays(n_rows: int, max_context: int) -> bool:
+    """Whether the one launch is the faster way for a step of this many rows whose longest context is `max_context`."""
+    n_splits = max(1, -(-int(max_context) // decode_split()))
+    return bool(library().imparo_attention_decode_qkv_pays(int(n_rows), n_splits))
 
 
 def attention_decode_qkv(qkv, q_weight, k_weight, eps: float, inv_freq, k_cache, v_cache, out, part_o, part_ml,

@@ -119,7 +119,7 @@ class Attention:
         inv_freq = self.position.inv_freq
         interleaved = bool(getattr(self.position, "interleaved", False))
         if (vt and owns_cache and ctx.single_rows is not None and ctx.n_single_rows == T and not ctx.n_portion_rows
-                and ops.attention_decode_qkv_pays(T)
+                and ops.attention_decode_qkv_pays(T, ctx.max_context)
                 and ops.attention_decode_qkv_takes(self.head_dim, 0 if inv_freq is None else inv_freq.shape[0])):
             # every row brings one token: head norm, rotation and the write of the new key and value ride
             # in the attention launch (the new key is weighed in from registers)
