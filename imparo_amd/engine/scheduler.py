@@ -357,6 +357,8 @@ def generate(model, input_ids: Sequence[Sequence[int]], max_tokens: int = 16, te
     `parallel` (a smaller pool makes requests wait or be recomputed)."""
     from .engine import Engine
     from ..sampling.sampler import Sampler
+    if len(input_ids) == 0:
+        return []
     if isinstance(model, Engine):
         engine = model
     else:
