@@ -136,6 +136,10 @@ def test_stop_token_and_entry_point_defaults(loud_model_dirs, loud_plain_models)
     # the reply ends at the stop token, which is not handed out
     got = generate(loud_model_dirs["A"], [p], max_tokens=10, dtype="float32", stop_token_ids=[full[at]])
     assert got == [full[:at]]
+    # no prompts, no replies; a prompt without tokens is refused by name
+    assert generate(loud_model_dirs["A"], []) == []
+    with pytest.raises(ValueError, match="at least one prompt token"):
+        generate(loud_model_dirs["A"], [p, []], max_tokens=2, dtype="float32")
 
 
 def test_waiting_after_every_step_generates_the_same(loud_model_dirs):
